@@ -1,0 +1,103 @@
+"""Oracle (test infrastructure): remove-padding pack / unpack index maps and masks.
+
+Pure integer logic, restated as the per-sequence Python loops the reference uses:
+
+* ``mindspeed_rl/utils/remove_padding.py:10-87``   ``preprocess_packed_seqs``
+* ``mindspeed_rl/utils/remove_padding.py:90-136``  ``postprocess_packed_seqs``
+* ``mindspeed_rl/utils/pad_process.py:74-141``     ``truncate_middle_and_pad`` / ``truncate_prompt_and_pad``
+* ``mindspeed_rl/utils/utils.py:57-67``            ``generate_mask``
+* ``mindspeed_rl/models/loss/base_loss_func.py:47-53`` window ``[P-1, P+R-1)``
+
+Pinned by the reference-held vectors of ``tests/ut/utils/test_utils.py:22-28`` and
+``tests/ut/utils/test_pad_process.py:48-62`` and by round-trip / brute-force properties.
+"""
+import torch
+
+
+def generate_mask(data_pad, seq_lengths):
+    """``utils/utils.py:57-67``: ``[B, data_pad.size(1)]`` int64, ones then trailing zeros."""
+    width = data_pad.size(1)
+    rows = []
+    for n in seq_lengths.flatten().tolist():
+        n_pad = width - n
+        row = [1.0] * width
+        if n_pad > 0:
+            # python slice semantics of ``row[-n_pad:] = 0``: a length above ``width`` cannot
+            # occur here (n_pad <= 0), a negative length zeroes at most the whole row
+            for k in range(max(width - n_pad, 0), width):
+                row[k] = 0.0
+        rows.append(row)
+    return torch.tensor(rows, dtype=torch.int64)
+
+
+def preprocess_packed_seqs(input_ids, labels, attention_mask_1d, tp_size):
+    """``utils/remove_padding.py:10-87``.
+
+    Returns ``(ids[1,T], position_ids[1,T], labels[1,T], seqlens[B] int32, cu_seqlens_padded[B+1] int32)``.
+    """
+    batch, width = input_ids.shape
+    if attention_mask_1d.shape != (batch, width):
+        raise ValueError("attention_mask_1d must have shape (batch_size, seq_len) matching input_ids")
+    seqlens = attention_mask_1d.sum(dim=1, dtype=torch.int32)
+    pad = (tp_size - (seqlens % tp_size)) % tp_size
+    padded = seqlens + pad
+    cu_padded = torch.zeros(batch + 1, dtype=torch.int32)
+    cu_padded[1:] = torch.cumsum(padded, dim=0)
+    total = int(padded.sum().item())
+
+    ids_packed = torch.zeros(total, dtype=input_ids.dtype)
+    pos_packed = torch.zeros(total, dtype=torch.int32)
+    labels_packed = torch.zeros(total, dtype=input_ids.dtype)
+    for i in range(batch):
+        lo = cu_padded[i].item()
+        hi = cu_padded[i + 1].item()
+        n = seqlens[i].item()
+        ids_packed[lo:lo + n] = input_ids[i, :n]
+        labels_packed[lo:lo + n] = labels[i, :n]
+        pos_packed[lo:hi] = torch.arange(hi - lo, dtype=torch.int32)
+    return (ids_packed.unsqueeze(0), pos_packed.unsqueeze(0), labels_packed.unsqueeze(0),
+            seqlens, cu_padded)
+
+
+def postprocess_packed_seqs(output, seqlens_in_batch, cu_seqlens_padded, seq_len, prompt_length=None):
+    """``utils/remove_padding.py:90-136``: packed ``[1,T,...]`` -> ``[B,seq_len,...]``."""
+    if output.shape[0] != 1:
+        raise ValueError("Expected output tensor to have shape[0] == 1 (packed batch dimension)")
+    batch = seqlens_in_batch.shape[0]
+    unpacked = torch.zeros([batch, seq_len] + list(output.shape[2:]), dtype=output.dtype)
+    for i in range(batch):
+        lo = cu_seqlens_padded[i].item()
+        n = seqlens_in_batch[i].item()
+        if prompt_length is not None:
+            skip = prompt_length[i].item() - 1
+            if skip < n:
+                n -= skip + 1
+                lo += skip
+        unpacked[i, :n] = output[0, lo:lo + n]
+    return unpacked
+
+
+def _window_copy(responses, input_tensor, truncate_lengths, pad_value, trailing):
+    rows, width = input_tensor.shape[0], input_tensor.shape[1]
+    window = torch.clamp(truncate_lengths, 0, width)
+    out = torch.full((rows, responses.shape[-1]) + trailing, pad_value, dtype=input_tensor.dtype)
+    for i in range(rows):
+        lo = window[i, 0].item()
+        hi = window[i, 1].item()
+        out[i, :hi - lo] = input_tensor[i, lo:hi]
+    return out
+
+
+def truncate_prompt_and_pad(responses, input_tensor, truncate_lengths, pad_value=0.0):
+    """``utils/pad_process.py:109-141``: ``[B,S]`` -> ``[B, responses.shape[-1]]``."""
+    return _window_copy(responses, input_tensor, truncate_lengths, pad_value, ())
+
+
+def truncate_middle_and_pad(responses, input_tensor, truncate_lengths, pad_value=0.0):
+    """``utils/pad_process.py:74-106``: ``[B,S,V]`` -> ``[B, responses.shape[-1], V]``."""
+    return _window_copy(responses, input_tensor, truncate_lengths, pad_value, (input_tensor.shape[2],))
+
+
+def response_window(prompt_length, response_length):
+    """``models/loss/base_loss_func.py:47-53``: ``cat([P, P+R], dim=1) - 1``."""
+    return torch.cat([prompt_length, prompt_length + response_length], dim=1) - 1
