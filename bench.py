@@ -1,0 +1,276 @@
+#!/usr/bin/env python3
+"""Benchmark of the actor log-prob + GRPO loss hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c0|c4chunk]
+
+One step = one pass of the path over one synthetic packed batch resident in HBM: the fused
+vocabulary sweep (log-prob + entropy + logsumexp), the unpack to [B, L], the fused policy loss
+with its five statistics (one device-to-host copy), and the backward down to dlogits.  Default
+workload is the Qwen2.5-7B-shaped GRPO actor step: 16 prompts x 8 responses, response lengths
+uniform in [512, 2048] (about 164k packed rows), vocabulary 152064, bf16 logits ~N(0, 3), labels
+drawn from softmax(logits), clip 0.2, k3 KL 0.001, token-mean loss.
+
+Prints ONE JSON line: tokens/s for the whole step, the roofline of the dominant kernel (the
+backward sweep) from HIP events recorded on the launch stream inside the timed region, and a CPU
+baseline: the oracle's restatement of the reference's torch op chain, timed on this host's cores
+on a bounded row sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "mindspeed-rl_amd"))
+
+HBM_PEAK_GBPS = 8000.0
+
+WORKLOADS = {
+    # name: prompts, group, r_lo, r_hi, vocab, dtype, sigma, description
+    "c1": dict(prompts=16, group=8, r_lo=512, r_hi=2048, vocab=152064, dtype="bf16", sigma=3.0,
+               desc="configs[1]: Qwen2.5-7B-shaped GRPO actor step, 16x8 responses, R~U[512,2048], V=152064 bf16"),
+    "c0": dict(prompts=4, group=4, r_lo=64, r_hi=256, vocab=32000, dtype="f32", sigma=2.0,
+               desc="configs[0]: 4x4 responses, R~U[64,256], V=32000 fp32"),
+    "c4chunk": dict(prompts=1, group=4, r_lo=8192, r_hi=24576, vocab=129280, dtype="bf16", sigma=3.0,
+                    desc="one ~64k-row chunk of configs[4]: V=129280 bf16, DAPO-length responses"),
+}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS))
+    ap.add_argument("--entropy-coeff", type=float, default=0.001,
+                    help="non-zero so that the forward computes entropy and the backward its gradient")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-rows", type=int, default=2048, help="rows of the CPU baseline sample")
+    ap.add_argument("--copy-ceiling", action="store_true", help="also time the plain copy kernel")
+    ap.add_argument("--seed", type=int, default=0)
+    return ap.parse_args()
+
+
+def make_lengths(torch, w, seed):
+    gen = torch.Generator().manual_seed(seed)
+    batch = w["prompts"] * w["group"]
+    rlen = torch.randint(w["r_lo"], w["r_hi"] + 1, (batch, 1), generator=gen, dtype=torch.int32)
+    plen = torch.ones(batch, 1, dtype=torch.int32)       # the path needs prompt_length >= 1
+    p = torch.rand(w["prompts"], 1, generator=gen).repeat(1, w["group"]).reshape(batch, 1)
+    rewards = torch.bernoulli(p, generator=gen)
+    return plen, rlen, rewards
+
+
+def build_device_batch(torch, mrl, w, plen, rlen, rewards, dev, seed):
+    """Synthetic batch in HBM, in the layout the training engine hands to the loss."""
+    batch = plen.shape[0]
+    seqlens = (plen + rlen).flatten().to(torch.int32)
+    cu = torch.zeros(batch + 1, dtype=torch.int32)
+    cu[1:] = torch.cumsum(seqlens, 0)
+    total = int(cu[-1])
+    vocab = w["vocab"]
+    tdtype = torch.bfloat16 if w["dtype"] == "bf16" else torch.float32
+    logits = torch.empty(1, total, vocab, dtype=tdtype, device=dev)
+    labels = torch.empty(1, total, dtype=torch.int64, device=dev)
+    g = torch.Generator(device=dev).manual_seed(seed)
+    chunk = 4096
+    for lo in range(0, total, chunk):
+        hi = min(total, lo + chunk)
+        z = (torch.randn(hi - lo, vocab, generator=g, device=dev) * w["sigma"]).to(tdtype)
+        logits[0, lo:hi] = z
+        # a sample from softmax(z): Gumbel-max
+        u = torch.rand(hi - lo, vocab, generator=g, device=dev).clamp_(1e-20, 1.0)
+        labels[0, lo:hi] = torch.argmax(z.float() - torch.log(-torch.log(u)), dim=-1)
+        del z, u
+    resp_w = int(rlen.max())
+    b = {
+        "labels": labels,
+        "responses": torch.zeros(batch, resp_w, dtype=torch.int32, device=dev),
+        "response_length": rlen.to(dev),
+        "prompt_length": plen.to(dev),
+    }
+    kw = dict(use_remove_padding=True, seqlens_in_batch=seqlens.to(dev), cu_seqlens_padded=cu.to(dev),
+              seq_len=int(seqlens.max()))
+    rmask = mrl.generate_mask(b["responses"], b["response_length"])
+    adv, _ = mrl.compute_group_norm_advantage_return(rewards.to(dev), rmask, b["response_length"], w["group"])
+    b["advantages"] = adv
+    # behaviour / reference log-probs: current + N(0, 0.05)
+    ref_fn = mrl.LossFuncFactory.get_instance("ray_grpo", "reference")
+    with torch.no_grad():
+        lp0 = ref_fn.compute_loss(logits, b, forward_only=True, **kw)
+    maskf = rmask.to(torch.float32)
+    b["old_log_prob"] = (lp0 + torch.randn(lp0.shape, generator=g, device=dev) * 0.05) * maskf
+    b["ref_log_prob"] = (lp0 + torch.randn(lp0.shape, generator=g, device=dev) * 0.05) * maskf
+    return logits, b, kw, total
+
+
+def cpu_baseline(torch, w, rows_target, entropy_coeff, seed):
+    """Times the oracle (torch-CPU restatement of the reference op chain) fwd+bwd on a bounded
+    sample of the same workload: one group of G responses with lengths scaled so that the packed
+    batch has about `rows_target` rows at the full vocabulary."""
+    from oracle import advantage as o_adv
+    from oracle import loss as o_loss
+    from oracle import packing as o_pack
+    threads = os.cpu_count() or 1
+    threads = min(threads, int(os.environ.get("OMP_NUM_THREADS", threads)))
+    torch.set_num_threads(threads)
+    gen = torch.Generator().manual_seed(seed + 1)
+    group, vocab = w["group"], w["vocab"]
+    mean_len = max(rows_target // group - 1, 4)
+    rlen = torch.randint(max(mean_len * 3 // 4, 1), mean_len * 5 // 4 + 1, (group, 1), generator=gen, dtype=torch.int32)
+    plen = torch.ones(group, 1, dtype=torch.int32)
+    width, resp_w = int((plen + rlen).max()), int(rlen.max())
+    ids = torch.randint(0, vocab, (group, width), generator=gen)
+    mask1d = o_pack.generate_mask(ids, plen + rlen)
+    labels = torch.cat([ids[:, 1:], torch.zeros(group, 1, dtype=ids.dtype)], 1)
+    _, _, p_lab, seqlens, cu = o_pack.preprocess_packed_seqs(ids, labels, mask1d, 1)
+    total = int(cu[-1])
+    tdtype = torch.bfloat16 if w["dtype"] == "bf16" else torch.float32
+    logits = (torch.randn(1, total, vocab, generator=gen) * w["sigma"]).to(tdtype)
+    rmask = o_pack.generate_mask(torch.zeros(group, resp_w), rlen)
+    rewards = torch.bernoulli(torch.full((group, 1), 0.5), generator=gen)
+    adv, _ = o_adv.compute_group_norm_advantage_return(rewards, rmask, rlen, group)
+    b = {"labels": p_lab, "responses": torch.zeros(group, resp_w, dtype=torch.int32), "response_length": rlen,
+         "prompt_length": plen, "advantages": adv}
+    kw = dict(use_remove_padding=True, seqlens_in_batch=seqlens, cu_seqlens_padded=cu, seq_len=width)
+    # the reference receives fp32 logits from the model's last stage
+    z32 = logits.float()
+    lp0 = o_loss.logprob_computer(z32, b, True, **kw)[0]
+    b["old_log_prob"] = (lp0 + torch.randn(lp0.shape, generator=gen) * 0.05) * rmask
+    b["ref_log_prob"] = (lp0 + torch.randn(lp0.shape, generator=gen) * 0.05) * rmask
+    meta = dict(clip_ratio=0.2, kl_coef=0.001, kl_penalty="low_var_kl", entropy_coeff=entropy_coeff)
+    tokens = int(rlen.sum())
+
+    def one():
+        z = z32.detach().requires_grad_()
+        t0 = time.perf_counter()
+        loss, _ = o_loss.grpo_compute_loss(z, b, meta, **kw)
+        loss.backward()
+        return time.perf_counter() - t0
+
+    one()
+    times = sorted(one() for _ in range(3))
+    med = times[len(times) // 2]
+    return {
+        "value": tokens / med, "unit": "tokens/s", "cores": threads, "kind": "port",
+        "sample": "%d responses, %d packed rows x V=%d (fp32 up-cast), oracle fwd+bwd, median of 3 after 1 warm-up, "
+                  "%.2f s per pass" % (group, total, vocab, med),
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (no collectives exist on this path); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import mindspeed_rl_amd as mrl
+    from mindspeed_rl_amd import _lib, vocab_ops
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    _lib.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    w = WORKLOADS[args.workload]
+    plen, rlen, rewards = make_lengths(torch, w, args.seed)
+    logits, b, kw, total = build_device_batch(torch, mrl, w, plen, rlen, rewards, dev, args.seed)
+    tokens = int(rlen.sum())
+    vocab = w["vocab"]
+    ebytes = logits.element_size()
+
+    f = mrl.LossFuncFactory.get_instance("ray_grpo", "actor")
+    f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.001), "kl_penalty": "low_var_kl",
+                          "entropy_coeff": args.entropy_coeff})
+
+    def step():
+        z = logits.detach().requires_grad_()
+        loss, stats = f.compute_loss(z, b, **kw)
+        (dz,) = torch.autograd.grad(loss, z)
+        return loss, stats, dz
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    vocab_ops.kernel_events = []
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss, stats, dz = step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    events = vocab_ops.kernel_events
+    vocab_ops.kernel_events = None
+    ms_per_step = elapsed * 1e3 / args.steps
+
+    def avg_ms(name):
+        ts = [s.elapsed_time(e) for (n, s, e, _) in events if n == name]
+        return sum(ts) / len(ts) if ts else float("nan")
+
+    fwd_ms, bwd_ms = avg_ms("mrl_vocab_logprob_fwd"), avg_ms("mrl_vocab_logprob_bwd")
+    live_rows = tokens                                    # rows with a non-zero incoming gradient
+    dead_rows = total - live_rows
+    fwd_bytes = total * vocab * ebytes
+    bwd_bytes = live_rows * 2 * vocab * ebytes + dead_rows * vocab * ebytes
+    bwd_gbps = bwd_bytes / (bwd_ms * 1e-3) / 1e9
+    fwd_gbps = fwd_bytes / (fwd_ms * 1e-3) / 1e9
+    step_gbps = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
+
+    result = {
+        "metric": "tokens/sec for logprob+GRPO loss fwd+bwd; achieved HBM GB/s as % of peak",
+        "value": tokens / (ms_per_step * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": w["dtype"],
+        "data": "synthetic",
+        "config": {
+            "workload": w["desc"], "responses": int(plen.shape[0]), "packed_rows": total, "response_tokens": tokens,
+            "vocab": vocab, "accumulate": "f32", "clip": 0.2, "kl": "low_var_kl 0.001",
+            "entropy_coeff": args.entropy_coeff, "loss": "token-mean",
+        },
+        "roofline": {
+            "kernel": "vocab_bwd_kernel (mrl_vocab_logprob_bwd)", "bound": "hbm", "achieved": bwd_gbps,
+            "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": bwd_gbps / HBM_PEAK_GBPS, "traffic": None,
+            "bytes_per_launch": bwd_bytes, "avg_ms": bwd_ms,
+        },
+        "kernels": {
+            "vocab_fwd": {"avg_ms": fwd_ms, "GBps": fwd_gbps, "frac": fwd_gbps / HBM_PEAK_GBPS,
+                          "bytes_per_launch": fwd_bytes},
+            "vocab_bwd": {"avg_ms": bwd_ms, "GBps": bwd_gbps, "frac": bwd_gbps / HBM_PEAK_GBPS,
+                          "bytes_per_launch": bwd_bytes},
+        },
+        "step_hbm": {"GBps": step_gbps, "frac": step_gbps / HBM_PEAK_GBPS,
+                     "algorithmic_bytes_per_step": fwd_bytes + bwd_bytes},
+        "stats": {k: float(v) for k, v in stats.items()},
+        "loss": float(loss),
+    }
+    if args.copy_ceiling:
+        n = 8 << 30
+        src = torch.empty(n, dtype=torch.uint8, device=dev)
+        dst = torch.empty(n, dtype=torch.uint8, device=dev)
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for _ in range(2):
+            _lib.call("mrl_copy_bytes", src.data_ptr(), dst.data_ptr(), n, _lib.stream(dev))
+        s.record()
+        for _ in range(5):
+            _lib.call("mrl_copy_bytes", src.data_ptr(), dst.data_ptr(), n, _lib.stream(dev))
+        e.record()
+        torch.cuda.synchronize()
+        result["copy_ceiling_GBps"] = 2 * n * 5 / (s.elapsed_time(e) * 1e-3) / 1e9
+        del src, dst
+    del dz
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(torch, w, args.cpu_rows, args.entropy_coeff, args.seed)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

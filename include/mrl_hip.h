@@ -1,0 +1,232 @@
+/*
+ * mrl_hip.h - C ABI of libmrl_hip.so: MI355X (gfx950) kernels for the actor log-probability
+ * and GRPO/DAPO policy-loss path of MindSpeed-RL.
+ *
+ * The reference has no native code and no FFI for this path: every function below replaces a
+ * chain of torch ops in the reference's Python (cited per entry point, paths relative to the
+ * reference tree).  Host code binds these symbols with ctypes.
+ *
+ * Conventions, all entry points:
+ *   - plain C: raw DEVICE pointers, explicit int64 sizes, dtype enums, the HIP stream as void*
+ *     (NULL = the null stream); no ownership is taken, nothing is allocated or freed;
+ *   - kernels are enqueued asynchronously on `stream`, no hidden synchronisation;
+ *   - return 0 on success, a negative mrl_status otherwise (nothing is launched then);
+ *     mrl_last_error() gives the message of the calling thread's last failure;
+ *   - tensors are dense row-major; "nullable" pointers may be NULL.
+ */
+#ifndef MRL_HIP_H_
+#define MRL_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MRL_VERSION 100
+
+enum mrl_status {
+    MRL_OK = 0,
+    MRL_ERR_INVALID_ARG = -1,  /* NULL where a pointer is required, negative size, bad enum */
+    MRL_ERR_UNSUPPORTED = -2,  /* dtype / size combination the kernels do not cover        */
+    MRL_ERR_MISALIGNED = -3,   /* pointer not aligned to its element size                  */
+    MRL_ERR_LAUNCH = -4        /* the HIP runtime rejected the launch                      */
+};
+
+enum mrl_dtype {
+    MRL_F32 = 0,
+    MRL_BF16 = 1,
+    MRL_F16 = 2,
+    MRL_I32 = 3,
+    MRL_I64 = 4,
+    MRL_U8 = 5, /* also torch.bool */
+    MRL_F64 = 6
+};
+
+enum mrl_kl_penalty {
+    MRL_KL_NONE = 0,      /* DAPO: kl_loss == 0 (dapo_actor_loss_func.py:150) */
+    MRL_KL_KL = 1,        /* logp - ref                                        */
+    MRL_KL_ABS = 2,       /* |logp - ref|                                      */
+    MRL_KL_MSE = 3,       /* 0.5 (logp - ref)^2                                */
+    MRL_KL_LOW_VAR = 4    /* k3 with clamps +-20 / +-10 (utils/compute.py:120-126) */
+};
+
+/* Library version (MRL_VERSION of the build). */
+int mrl_version(void);
+
+/* Message of the calling thread's last failed call ("" if none). */
+const char* mrl_last_error(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Vocabulary sweep, forward.  Replaces compute_log_probs (mindspeed_rl/utils/compute.py:29-51,
+ * i.e. Megatron's vocab_parallel_cross_entropy at tp=1), _VocabParallelEntropy.forward
+ * (utils/compute.py:56-73) and the caller's `output.div_(temperature)`
+ * (models/base/base_training_engine.py:237) in ONE read of the logits.
+ *
+ *   z' = logits * inv_temperature
+ *   lse[t]     = logsumexp_j z'[t,j]
+ *   logp[t]    = z'[t, label_t] - lse[t]      (label outside [0,vocab): max_j z'[t,j] - lse[t],
+ *                                               which is what Megatron's target mask yields)
+ *   entropy[t] = lse[t] - sum_j softmax(z')_j z'[t,j]
+ *
+ * logits: [n_rows, vocab] of logits_dtype (F32, BF16, F16), row t at logits + t*row_stride
+ * elements; it is only read.  labels: [n_rows] I32 or I64.  row_active (nullable): [n_rows]
+ * bytes, rows with 0 are skipped and get logp = entropy = lse = 0.  entropy and lse are
+ * nullable; logp is required.  Accumulation is fp32.
+ */
+int mrl_vocab_logprob_fwd(const void* logits, int logits_dtype, int64_t n_rows, int64_t vocab,
+                          int64_t row_stride, const void* labels, int labels_dtype,
+                          const uint8_t* row_active, float inv_temperature, float* logp,
+                          float* entropy, float* lse, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Vocabulary sweep, backward.  Replaces Megatron's cross-entropy backward,
+ * _VocabParallelEntropy.backward (utils/compute.py:76-85) and autograd of the temperature
+ * division with one read of the logits and one write of dlogits:
+ *
+ *   p = exp(z' - lse)
+ *   dlogits[t,j] = inv_temperature * ( g_logp[t] * (onehot(label_t)_j - p_j)
+ *                                      - g_entropy[t] * p_j * (z'_j - (lse[t] - entropy[t])) )
+ *
+ * lse (and entropy, if g_entropy is given) are the forward's outputs.  g_logp and g_entropy are
+ * [n_rows] fp32, each nullable (NULL = zero).  Rows whose incoming gradients are both zero are
+ * written as zeros without reading the logits.  dlogits has dlogits_dtype (F32, BF16, F16) and
+ * its own row stride; it may alias logits exactly (same pointer, dtype and stride) for an
+ * in-place backward.
+ */
+int mrl_vocab_logprob_bwd(const void* logits, int logits_dtype, int64_t n_rows, int64_t vocab,
+                          int64_t row_stride, const void* labels, int labels_dtype,
+                          float inv_temperature, const float* lse, const float* entropy,
+                          const float* g_logp, const float* g_entropy, void* dlogits,
+                          int dlogits_dtype, int64_t dlogits_row_stride, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Remove-padding index maps.  Replace the per-sequence Python loops of preprocess_packed_seqs
+ * (mindspeed_rl/utils/remove_padding.py:38-87).  All integer results are bit-exact.
+ *
+ * mrl_pack_index_build: seqlens[i] = int32 sum of attention_mask[i,:] (mask dtype I64, I32, U8
+ * or F32; if attention_mask is NULL, seqlens is an input), pad_i = (align - len_i % align) %
+ * align, cu_seqlens_padded[0] = 0, cu_seqlens_padded[i+1] = int32 running sum of len_i + pad_i.
+ * total (nullable) receives cu_seqlens_padded[batch] as int64.  One workgroup; batch <= 2^20.
+ */
+int mrl_pack_index_build(const void* attention_mask, int mask_dtype, int64_t batch, int64_t width,
+                         int64_t align, int32_t* seqlens, int32_t* cu_seqlens_padded,
+                         int64_t* total, void* stream);
+
+/* mrl_pack_rows: dst[t] = src[i, t - cu[i]] for cu[i] <= t < cu[i] + seqlens[i], else 0;
+ * position_ids[t] = t - cu[i] (runs through the alignment padding, remove_padding.py:66-72).
+ * src/dst (and the optional second pair src2/dst2, e.g. ids and labels in one launch) hold
+ * elem_bytes = 4 or 8 byte integers; src is [batch, width], dst is [total].  position_ids
+ * (nullable) is int32 [total].  Positions t >= cu[batch] are written as 0. */
+int mrl_pack_rows(const void* src, void* dst, const void* src2, void* dst2, int elem_bytes,
+                  int64_t batch, int64_t width, const int32_t* seqlens,
+                  const int32_t* cu_seqlens_padded, int64_t total, int32_t* position_ids,
+                  void* stream);
+
+/* mrl_unpad_gather: postprocess_packed_seqs (remove_padding.py:116-136).  packed is
+ * [total, inner] of elem_bytes (2, 4 or 8) bytes, out is [batch, seq_len, inner], fully
+ * written (zeros where nothing is copied).  Per sequence: start = cu[i], n = seqlens[i]; if
+ * prompt_length is given (I32 or I64, [batch]) and P_i - 1 < n then n -= P_i, start += P_i - 1;
+ * out[i, :n] = packed[start : start + n].  Where the reference raises on n > seq_len this
+ * kernel copies the first seq_len entries. */
+int mrl_unpad_gather(const void* packed, int elem_bytes, int64_t total, int64_t inner,
+                     const int32_t* seqlens, const int32_t* cu_seqlens_padded,
+                     const void* prompt_length, int prompt_dtype, int64_t batch, int64_t seq_len,
+                     void* out, void* stream);
+
+/* mrl_pad_scatter: adjoint of mrl_unpad_gather for fp32 gradients with inner == 1:
+ * g_packed[t] = g_out[i, t - start_i] if t lies in sequence i's copied window, else 0.
+ * Written as a gather over t (binary search in cu), so it is deterministic. */
+int mrl_pad_scatter(const float* g_out, int64_t batch, int64_t seq_len, const int32_t* seqlens,
+                    const int32_t* cu_seqlens_padded, const void* prompt_length, int prompt_dtype,
+                    int64_t total, float* g_packed, void* stream);
+
+/* mrl_window_gather: truncate_prompt_and_pad / truncate_middle_and_pad
+ * (mindspeed_rl/utils/pad_process.py:74-141).  src is [batch, width, inner] of elem_bytes, window
+ * is [batch, 2] (I32 or I64) = (start, end), clamped to [0, width]; out is [batch, out_len,
+ * inner], filled with pad_bits (the element's bit pattern, low elem_bytes bytes) and then
+ * out[i, :end-start] = src[i, start:end].  Copies at most out_len entries per row. */
+int mrl_window_gather(const void* src, int elem_bytes, int64_t batch, int64_t width, int64_t inner,
+                      const void* window, int window_dtype, int64_t out_len, uint64_t pad_bits,
+                      void* out, void* stream);
+
+/* mrl_window_scatter: adjoint of mrl_window_gather for fp32, inner == 1: g_src is [batch, width],
+ * g_src[i, start+j] = g_out[i, j] for j < min(end-start, out_len), zero elsewhere. */
+int mrl_window_scatter(const float* g_out, int64_t batch, int64_t width, const void* window,
+                       int window_dtype, int64_t out_len, float* g_src, void* stream);
+
+/* mrl_generate_mask: generate_mask (mindspeed_rl/utils/utils.py:57-67): out[i, j] =
+ * (j < lengths[i]) as int64, [batch, width]; lengths is I32 or I64.  Negative lengths give an
+ * all-zero row, lengths above width an all-one row. */
+int mrl_generate_mask(const void* lengths, int lengths_dtype, int64_t batch, int64_t width,
+                      int64_t* out, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Group-relative advantages.  Replaces compute_group_norm_advantage_return
+ * (mindspeed_rl/trainer/utils/compute_utils.py:152-191): rows i*group .. (i+1)*group-1 form one
+ * group; in fp64, score = (r - mean) / (unbiased_std + 1e-6); cast to fp32; advantages[i, j] =
+ * score_i * mask[i, j].  rewards: [batch] F32 or F64; mask: [batch, width] F32, I64, I32 or U8;
+ * advantages / returns: [batch, width] fp32 (returns nullable, a second copy as in the
+ * reference).  batch must be a multiple of group.  group == 1 yields NaN, as torch.std does. */
+int mrl_group_advantage(const void* rewards, int rewards_dtype, int64_t batch, int64_t group,
+                        const void* mask, int mask_dtype, int64_t width, float* advantages,
+                        float* returns, void* stream);
+
+/* DAPO dynamic-sampling predicate (mindspeed_rl/workers/dynamic_sampling.py:81-86): keep[r] = 1
+ * for every row of a group iff numpy.std(group) > 0 or the group has one member, else 0.  The
+ * arithmetic follows numpy's (pairwise summation, mean, squared deviations, in the metric's own
+ * dtype F32 or F64) so that the comparison with 0 is bit-exact.  n need not be a multiple of
+ * group: the last group is short, as python slicing makes it. */
+int mrl_group_keep_mask(const void* metric, int metric_dtype, int64_t n, int64_t group,
+                        uint8_t* keep, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Policy loss, forward.  Replaces _compute_grpo_policy_loss
+ * (mindspeed_rl/models/loss/grpo_actor_loss_func.py:127-144), _compute_dapo_policy_loss
+ * (dapo_actor_loss_func.py:129-152), compute_kl_penalty (utils/compute.py:100-133), the
+ * masked_mean calls (utils/torch_functional.py:38-59) and the dynamic-batch rescale
+ * (grpo_actor_loss_func.py:74-79) with one launch plus a tiny finalize launch.
+ *
+ * All per-token tensors are [batch, width] fp32, dense.  old_log_prob NULL means ratio == 1;
+ * ref_log_prob is required unless kl_penalty == MRL_KL_NONE; entropy NULL means zeros.  The mask
+ * is either `mask` ([batch, width] of mask_dtype F32, I64, I32, U8) or, if mask is NULL,
+ * j < response_length[i] (I32 or I64).  ratio is clamped to [clip_lo, clip_hi] (pass
+ * float(1 - eps_low), float(1 + eps_high)).  seq_mean = 0: token mean with the reference's 1e-8
+ * in the denominator; seq_mean = 1: DAPO's mean over sequences of per-sequence token means
+ * (no epsilon: an all-masked row gives NaN, and the clip fraction is 0, as in the reference).
+ *
+ * out[8] (fp32): [0] loss_scale * pg_loss (the tensor the caller back-propagates),
+ *   [1] pg_loss, [2] pg_clipfrac, [3] ppo_kl, [4] kl_loss, [5] entropy mean, [6] sum(mask),
+ *   [7] number of rows.
+ * row_sums: workspace of batch*8 floats, kept for the backward.
+ */
+int mrl_policy_loss_fwd(const float* log_prob, const float* old_log_prob,
+                        const float* ref_log_prob, const float* advantages, const float* entropy,
+                        const void* mask, int mask_dtype, const void* response_length,
+                        int length_dtype, int64_t batch, int64_t width, float clip_lo,
+                        float clip_hi, int kl_penalty, float kl_coef, float entropy_coeff,
+                        int seq_mean, float loss_scale, float* row_sums, float* out,
+                        void* stream);
+
+/* Policy loss, backward: what autograd derives from the torch expression of the reference,
+ * including torch.max's half/half split on ties and clamp's closed-interval pass-through.
+ * upstream (nullable) is a DEVICE scalar multiplying everything (Megatron's loss scaling).
+ * g_log_prob [batch, width] is required; g_entropy is nullable (needed if entropy_coeff != 0). */
+int mrl_policy_loss_bwd(const float* log_prob, const float* old_log_prob,
+                        const float* ref_log_prob, const float* advantages, const void* mask,
+                        int mask_dtype, const void* response_length, int length_dtype,
+                        int64_t batch, int64_t width, float clip_lo, float clip_hi,
+                        int kl_penalty, float kl_coef, float entropy_coeff, int seq_mean,
+                        float loss_scale, const float* row_sums, const float* out,
+                        const float* upstream, float* g_log_prob, float* g_entropy, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Plain device-to-device copy kernel of n_bytes (multiple of 16, 16-byte aligned pointers);
+ * used to calibrate the rocprofv3 FETCH_SIZE / WRITE_SIZE counters and as the measured
+ * bandwidth ceiling next to the 8 TB/s vendor peak.  No counterpart in the reference. */
+int mrl_copy_bytes(const void* src, void* dst, int64_t n_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MRL_HIP_H_ */

@@ -1,0 +1,24 @@
+"""mindspeed_rl_amd - MI355X (gfx950) kernels for MindSpeed-RL's actor log-probability and
+GRPO / DAPO policy-loss path, behind the reference's own Python call surface.
+
+Everything here dispatches to libmrl_hip.so (C ABI in ``include/mrl_hip.h``); there is no CPU
+or eager fallback.  Build the library with ``python -m mindspeed_rl_amd._build``.
+"""
+from . import _lib
+from .advantage import (FixedKLController, compute_group_norm_advantage_return, dynamic_sampling_keep,
+                        dynamic_sampling_keep_mask)
+from .functional import masked_mean, masked_sum
+from .loss import (BaseLossFunc, DAPOActorLossFunc, GRPOActorLossFunc, LossFuncFactory, LossRegister,
+                   MultimodalLogProbComputer, ReferenceLossFunc, StandardLogProbComputer, policy_loss)
+from .packing import (generate_mask, pack_index, postprocess_packed_seqs, preprocess_packed_seqs, response_window,
+                      truncate_middle_and_pad, truncate_prompt_and_pad)
+from .vocab_ops import (compute_kl_penalty, compute_log_probs, get_parallel_state, get_vocab_parallel,
+                        set_parallel_state, set_vocab_parallel, vocab_logprob_entropy, vocab_parallel_cross_entropy,
+                        vocab_parallel_entropy)
+
+__version__ = "0.1.0"
+
+
+def library_version():
+    """MRL_VERSION of the loaded libmrl_hip.so (loads it; raises if it is not built)."""
+    return _lib.load().mrl_version()

@@ -1,0 +1,370 @@
+"""Loss registry and the GRPO / DAPO / reference loss objects.
+
+Host-side mirror of ``mindspeed_rl/models/loss/`` of the reference: the registry
+(``loss_register.py``, ``loss_func_factory.py``), ``BaseLossFunc`` (``base_loss_func.py``), the
+text-only log-prob strategy (``logprob_computer.py:73-145``), ``GRPOActorLossFunc``
+(``grpo_actor_loss_func.py``), ``DAPOActorLossFunc`` (``dapo_actor_loss_func.py``) and
+``ReferenceLossFunc`` (``reference_loss_func.py``).  Class names, registry keys, method
+signatures, keyword arguments, return values and error behaviour are the reference's; the work
+is done by the HIP kernels of libmrl_hip.so.
+"""
+from abc import ABC, abstractmethod
+from typing import Dict, Tuple
+
+import torch
+
+from . import _lib
+from .packing import (generate_mask, postprocess_packed_seqs, response_window, truncate_middle_and_pad,
+                      truncate_prompt_and_pad)
+from .vocab_ops import compute_log_probs, vocab_logprob_entropy, vocab_parallel_entropy
+
+STAT_KEYS = ("actor/pg_loss", "actor/pg_clipfrac", "actor/ppo_kl", "actor/kl_loss", "actor/entropy")
+
+
+# ------------------------------------------------------------------------------------ registry
+class LossRegister:
+    """Class registry keyed ``stage + "_" + role`` (reference: ``loss_register.py:4-23``).
+    Registering a key again replaces the previous class - that is the plug-in point."""
+
+    class_map = dict()
+
+    @classmethod
+    def _key(cls, stage: str, role: str) -> str:
+        return stage + "_" + role
+
+    @classmethod
+    def register_loss(cls, stage: str, role: str):
+        def decorate(klass):
+            cls.class_map[cls._key(stage, role)] = klass
+            return klass
+
+        return decorate
+
+    @classmethod
+    def get_class(cls, stage: str, role: str):
+        return cls.class_map.get(cls._key(stage, role))
+
+    @classmethod
+    def get_instance(cls, stage: str, role: str, *args, **kwargs):
+        klass = cls.get_class(stage, role)
+        return None if klass is None else klass(*args, **kwargs)
+
+
+class LossFuncFactory(LossRegister):
+    """Reference: ``loss_func_factory.py:5-6`` - its own map, separate from the base class."""
+
+    class_map = dict()
+
+
+# ------------------------------------------------------------------------------------ policy loss op
+def _mask_args(mask, response_length, dev):
+    """(mask tensor or None, length tensor or None) in a dtype the kernel reads directly."""
+    if mask is not None:
+        if mask.dtype not in (torch.float32, torch.int64, torch.int32, torch.uint8, torch.bool):
+            mask = mask.to(torch.float32)
+        return mask.to(dev).contiguous(), None
+    lens = response_length
+    if lens.dtype not in (torch.int32, torch.int64):
+        lens = lens.to(torch.int64)
+    return None, lens.to(dev).reshape(-1).contiguous()
+
+
+class _PolicyLoss(torch.autograd.Function):
+    """log_prob [B,L] (+ entropy [B,L]) -> (scaled loss, out[8]) through mrl_policy_loss_fwd/_bwd."""
+
+    @staticmethod
+    def forward(ctx, log_prob, entropy, old_log_prob, ref_log_prob, advantages, mask, lens, cfg):
+        dev = _lib.require_device(log_prob, entropy, old_log_prob, ref_log_prob, advantages, mask, lens)
+        batch, width = log_prob.shape
+
+        def dense(t):
+            return None if t is None else t.to(torch.float32).contiguous()
+
+        lp, ent, old, ref, adv = dense(log_prob), dense(entropy), dense(old_log_prob), dense(ref_log_prob), dense(
+            advantages)
+        row_sums = torch.empty(max(batch, 1) * 8, dtype=torch.float32, device=dev)
+        out = torch.empty(8, dtype=torch.float32, device=dev)
+        scalars = (cfg["clip_lo"], cfg["clip_hi"], cfg["kl_penalty"], cfg["kl_coef"], cfg["entropy_coeff"],
+                   cfg["seq_mean"], cfg["loss_scale"])
+        _lib.call("mrl_policy_loss_fwd", _lib.ptr(lp), _lib.ptr(old), _lib.ptr(ref), _lib.ptr(adv), _lib.ptr(ent),
+                  _lib.ptr(mask), _lib.dtype_code(mask) if mask is not None else _lib.F32, _lib.ptr(lens),
+                  _lib.dtype_code(lens) if lens is not None else _lib.I32, batch, width, *scalars,
+                  _lib.ptr(row_sums), _lib.ptr(out), _lib.stream(dev))
+        ctx.save_for_backward(lp, old, ref, adv, mask, lens, row_sums, out)
+        ctx.scalars = scalars
+        ctx.want_entropy_grad = entropy is not None and entropy.requires_grad
+        ctx.mark_non_differentiable(out)
+        return out[0].clone(), out      # the loss gets its own storage: autograd outputs must not alias
+
+    @staticmethod
+    def backward(ctx, g_loss, _g_out):
+        lp, old, ref, adv, mask, lens, row_sums, out = ctx.saved_tensors
+        dev = lp.device
+        batch, width = lp.shape
+        upstream = g_loss.to(torch.float32).reshape(1).contiguous()
+        g_lp = torch.empty_like(lp)
+        g_ent = torch.empty_like(lp) if ctx.want_entropy_grad else None
+        _lib.call("mrl_policy_loss_bwd", _lib.ptr(lp), _lib.ptr(old), _lib.ptr(ref), _lib.ptr(adv), _lib.ptr(mask),
+                  _lib.dtype_code(mask) if mask is not None else _lib.F32, _lib.ptr(lens),
+                  _lib.dtype_code(lens) if lens is not None else _lib.I32, batch, width, *ctx.scalars,
+                  _lib.ptr(row_sums), _lib.ptr(out), _lib.ptr(upstream), _lib.ptr(g_lp), _lib.ptr(g_ent),
+                  _lib.stream(dev))
+        return g_lp, g_ent, None, None, None, None, None, None
+
+
+def policy_loss(log_prob, entropy, old_log_prob, ref_log_prob, advantages, mask=None, response_length=None, *,
+                clip_low, clip_high, kl_penalty=None, kl_coef=0.0, entropy_coeff=0.0, token_level_loss=True,
+                loss_scale=1.0):
+    """Fused clipped-ratio surrogate + KL penalty + entropy bonus.
+
+    Returns ``(loss, out)``: ``loss`` is the 0-dim tensor to back-propagate (``loss_scale *
+    pg_loss``), ``out`` the 8 device scalars ``[scaled loss, pg_loss, pg_clipfrac, ppo_kl,
+    kl_loss, entropy, sum(mask), rows]``.  ``clip_low`` / ``clip_high`` are the epsilons;
+    ``kl_penalty`` is one of ``None, 'kl', 'abs', 'mse', 'low_var_kl'``.
+    """
+    if kl_penalty is None:
+        kl_code = _lib.KL_NONE
+    elif kl_penalty in _lib.KL_BY_NAME:
+        kl_code = _lib.KL_BY_NAME[kl_penalty]
+    else:
+        raise NotImplementedError          # 'full' and unknown kinds, as compute_kl_penalty does
+    dev = log_prob.device
+    mask_t, lens_t = _mask_args(mask, response_length, dev)
+    cfg = dict(clip_lo=float(1.0 - clip_low), clip_hi=float(1.0 + clip_high), kl_penalty=kl_code,
+               kl_coef=float(kl_coef), entropy_coeff=float(entropy_coeff), seq_mean=0 if token_level_loss else 1,
+               loss_scale=float(loss_scale))
+    return _PolicyLoss.apply(log_prob, entropy, old_log_prob, ref_log_prob, advantages, mask_t, lens_t, cfg)
+
+
+# ------------------------------------------------------------------------------------ log-prob strategy
+class LogProbComputer:
+    def compute(self, output, batch, skip_entropy, **kwargs):
+        raise NotImplementedError
+
+
+class StandardLogProbComputer(LogProbComputer):
+    """Reference: ``logprob_computer.py:73-145`` at context-parallel size 1.
+
+    One fused sweep gives log-prob and (unless skipped) entropy of every packed / padded row; the
+    index-map kernels then cut out the ``[B, L]`` response window.  Extra keyword
+    ``inv_temperature`` folds the caller's temperature division into the sweep (default 1)."""
+
+    @staticmethod
+    def _get_log_probs_remove_prompt_pad(logprob, batch):
+        window = response_window(batch["prompt_length"], batch["response_length"])
+        return truncate_prompt_and_pad(batch["responses"], logprob, window)
+
+    def compute(self, output, batch, skip_entropy, **kwargs):
+        labels = batch["labels"]
+        inv_t = float(kwargs.get("inv_temperature", 1.0))
+        log_probs, entropy, _ = vocab_logprob_entropy(output, labels, inv_temperature=inv_t,
+                                                      want_entropy=not skip_entropy,
+                                                      grad_inplace=bool(kwargs.get("grad_inplace", False)))
+        if kwargs.get("use_remove_padding", False):
+            seqlens = kwargs.get("seqlens_in_batch", None)
+            cu = kwargs.get("cu_seqlens_padded", None)
+            seq_len = batch["responses"].shape[-1]
+
+            def cut(x):
+                return postprocess_packed_seqs(x, seqlens, cu, seq_len, prompt_length=batch["prompt_length"])
+        else:
+            def cut(x):
+                return self._get_log_probs_remove_prompt_pad(x, batch)
+
+        log_probs = cut(log_probs)
+        entropy = torch.zeros_like(log_probs) if skip_entropy else cut(entropy)
+        return log_probs, entropy
+
+
+class MultimodalLogProbComputer(LogProbComputer):
+    """Reference: ``logprob_computer.py:40-70``: logits are cut to the response window first and
+    scored against ``responses``; entropy is taken over the full output."""
+
+    def compute(self, output, batch, skip_entropy, **kwargs):
+        responses = batch["responses"]
+        window = response_window(batch["prompt_length"], batch["response_length"])
+        logits = truncate_middle_and_pad(responses, output, window)
+        log_probs = compute_log_probs(logits, responses)
+        entropy = torch.zeros_like(log_probs) if skip_entropy else vocab_parallel_entropy(output)
+        return log_probs, entropy
+
+
+# ------------------------------------------------------------------------------------ loss objects
+class BaseLossFunc(ABC):
+    """Reference: ``base_loss_func.py:13-57``."""
+
+    def __init__(self):
+        self.logprob_computer = StandardLogProbComputer()
+
+    def add_loss_meta_info(self, meta_info: Dict):
+        pass
+
+    @abstractmethod
+    def compute_loss(self, output: torch.Tensor, batch: Dict[str, torch.Tensor], forward_only=False,
+                     non_loss_data=True, **kwargs) -> Tuple[torch.Tensor, Dict]:
+        pass
+
+    @staticmethod
+    def _get_compute_log_probs_input(output: torch.Tensor, batch: Dict[str, torch.Tensor]):
+        if "responses" not in batch:
+            raise ValueError("The responses is None")
+        responses = batch["responses"]
+        window = response_window(batch["prompt_length"], batch["response_length"])
+        return responses, truncate_middle_and_pad(responses, output, window)
+
+    @staticmethod
+    def _get_log_probs_remove_prompt_pad(logprob: torch.Tensor, batch: Dict[str, torch.Tensor]):
+        window = response_window(batch["prompt_length"], batch["response_length"])
+        return truncate_prompt_and_pad(batch["responses"], logprob, window)
+
+    def compute_log_probs(self, output, batch: Dict[str, torch.Tensor], skip_entropy=True, **kwargs):
+        return self.logprob_computer.compute(output, batch, skip_entropy, **kwargs)
+
+
+def _finish(loss, out):
+    """The five statistics as python floats from ONE device-to-host copy (the reference issues five
+    ``.item()`` calls); ``abs`` on the policy loss as in ``grpo_actor_loss_func.py:91-97``."""
+    host = out.detach().cpu().tolist()
+    stats = {
+        STAT_KEYS[0]: abs(host[1]),
+        STAT_KEYS[1]: host[2],
+        STAT_KEYS[2]: host[3],
+        STAT_KEYS[3]: host[4],
+        STAT_KEYS[4]: host[5],
+    }
+    return loss, stats
+
+
+def _dynamic_scale(batch, forward_only, kwargs):
+    """``responses.size(0) / actual_micro_batch_size`` under dynamic batch size, else 1."""
+    if kwargs.get("use_dynamic_bsz", False) and not forward_only:
+        return batch["responses"].size(0) / kwargs.get("actual_micro_batch_size", None)
+    return 1.0
+
+
+@LossFuncFactory.register_loss("ray_grpo", "actor")
+class GRPOActorLossFunc(BaseLossFunc):
+    """Reference: ``grpo_actor_loss_func.py:14-144``."""
+
+    def __init__(self):
+        super().__init__()
+        self.clip_ratio = 0.2
+        self.entropy_coeff = 0.0
+
+    def add_loss_meta_info(self, meta_info: Dict):
+        if meta_info is None:
+            return
+        if "clip_ratio" in meta_info.keys():
+            self.clip_ratio = float(meta_info["clip_ratio"])
+        for key in ("kl_ctrl", "entropy_coeff", "kl_penalty"):
+            if key in meta_info.keys():
+                setattr(self, key, meta_info[key])
+
+    @staticmethod
+    def _get_policy_loss_input(batch: Dict[str, torch.Tensor]):
+        if "responses" not in batch:
+            raise ValueError("The responses is None")
+        response_mask = generate_mask(batch["responses"], batch["response_length"])
+        return (response_mask, batch.get("old_log_prob"), batch.get("advantages"), batch.get("ref_log_prob"))
+
+    def compute_loss(self, output: torch.Tensor, batch: Dict[str, torch.Tensor], forward_only=False,
+                     non_loss_data=True, **kwargs) -> Tuple[torch.Tensor, Dict]:
+        if "responses" not in batch:
+            raise ValueError("The responses is None")
+        if forward_only:
+            log_probs, _ = super().compute_log_probs(output=output, batch=batch, **kwargs)
+            return log_probs
+        log_probs, entropy = super().compute_log_probs(output=output, batch=batch,
+                                                       skip_entropy=(self.entropy_coeff == 0), **kwargs)
+        # batch['response_mask'] is ignored here, as in the reference: the mask is j < response_length
+        loss, out = policy_loss(log_probs, entropy if self.entropy_coeff != 0 else None, batch.get("old_log_prob"),
+                                batch.get("ref_log_prob"), batch.get("advantages"),
+                                response_length=batch["response_length"], clip_low=self.clip_ratio,
+                                clip_high=self.clip_ratio, kl_penalty=self.kl_penalty, kl_coef=self.kl_ctrl.value,
+                                entropy_coeff=self.entropy_coeff, token_level_loss=True,
+                                loss_scale=_dynamic_scale(batch, forward_only, kwargs))
+        return _finish(loss, out)
+
+    @staticmethod
+    def _compute_grpo_policy_loss(old_log_prob, log_prob, ref_log_prob, advantages, entropy, eos_mask, cliprange,
+                                  kl_ctrl, kl_penalty, entropy_coeff):
+        """Reference: ``grpo_actor_loss_func.py:100-144``.  Returns ``(pg_loss, pg_clipfrac, ppo_kl,
+        kl_loss, entropy_loss)`` as 0-dim tensors; ``pg_loss`` is differentiable."""
+        loss, out = policy_loss(log_prob, entropy, old_log_prob, ref_log_prob, advantages, mask=eos_mask,
+                                clip_low=cliprange, clip_high=cliprange, kl_penalty=kl_penalty,
+                                kl_coef=kl_ctrl.value, entropy_coeff=entropy_coeff, token_level_loss=True)
+        return loss, out[2], out[3], out[4], out[5]
+
+
+@LossFuncFactory.register_loss("ray_dapo", "actor")
+class DAPOActorLossFunc(BaseLossFunc):
+    """Reference: ``dapo_actor_loss_func.py:13-152``."""
+
+    def __init__(self):
+        super().__init__()
+        self.clip_ratio = 0.2
+        self.entropy_coeff = 0.0
+
+    def add_loss_meta_info(self, meta_info: Dict):
+        if meta_info is None:
+            return
+        casts = (("clip_ratio", float), ("kl_ctrl", None), ("entropy_coeff", None), ("token_level_loss", bool),
+                 ("clip_higher_enable", bool), ("clip_ratio_low", float), ("clip_ratio_high", float))
+        for key, cast in casts:
+            if key in meta_info.keys():
+                setattr(self, key, meta_info[key] if cast is None else cast(meta_info[key]))
+
+    @staticmethod
+    def _get_policy_loss_input(batch: Dict[str, torch.Tensor]):
+        if "responses" not in batch:
+            raise ValueError("The responses is None")
+        response_mask = batch["response_mask"] if "response_mask" in batch else \
+            generate_mask(batch["responses"], batch["response_length"])
+        return response_mask, batch.get("old_log_prob"), batch.get("advantages")
+
+    def compute_loss(self, output: torch.Tensor, batch: Dict[str, torch.Tensor], forward_only=False,
+                     non_loss_data=True, **kwargs) -> Tuple[torch.Tensor, Dict]:
+        if "responses" not in batch:
+            raise ValueError("The responses is None")
+        if forward_only:
+            log_probs, _ = super().compute_log_probs(output=output, batch=batch, **kwargs)
+            return log_probs
+        log_probs, entropy = super().compute_log_probs(output=output, batch=batch,
+                                                       skip_entropy=(self.entropy_coeff == 0), **kwargs)
+        if not self.clip_higher_enable:
+            self.clip_ratio_low = self.clip_ratio
+            self.clip_ratio_high = self.clip_ratio
+        mask = batch["response_mask"] if "response_mask" in batch else None
+        loss, out = policy_loss(log_probs, entropy if self.entropy_coeff != 0 else None, batch.get("old_log_prob"),
+                                None, batch.get("advantages"), mask=mask,
+                                response_length=None if mask is not None else batch["response_length"],
+                                clip_low=self.clip_ratio_low, clip_high=self.clip_ratio_high, kl_penalty=None,
+                                entropy_coeff=self.entropy_coeff, token_level_loss=self.token_level_loss,
+                                loss_scale=_dynamic_scale(batch, forward_only, kwargs))
+        return _finish(loss, out)
+
+    @staticmethod
+    def _compute_dapo_policy_loss(old_log_prob, log_prob, entropy, entropy_coeff, advantages, eos_mask,
+                                  clip_ratio_low, clip_ratio_high, token_level_loss):
+        """Reference: ``dapo_actor_loss_func.py:105-152``.  In sequence-mean mode the clip fraction
+        is 0 and a row with an empty mask makes the loss NaN, as in the reference."""
+        loss, out = policy_loss(log_prob, entropy, old_log_prob, None, advantages, mask=eos_mask,
+                                clip_low=clip_ratio_low, clip_high=clip_ratio_high, kl_penalty=None,
+                                entropy_coeff=entropy_coeff, token_level_loss=token_level_loss)
+        return loss, out[2], out[3], out[4], out[5]
+
+
+@LossFuncFactory.register_loss("ray_grpo", "reference")
+@LossFuncFactory.register_loss("ray_ppo", "reference")
+class ReferenceLossFunc(BaseLossFunc):
+    """Reference: ``reference_loss_func.py:9-25``: forward-only log-prob of the reference policy."""
+
+    def __init__(self):
+        super(ReferenceLossFunc, self).__init__()
+
+    def compute_loss(self, output: torch.Tensor, batch: Dict[str, torch.Tensor], forward_only=False,
+                     non_loss_data=True, **kwargs) -> Tuple[torch.Tensor, Dict]:
+        log_probs, _ = super().compute_log_probs(output=output, batch=batch, **kwargs)
+        if forward_only:
+            return log_probs
+        return None

@@ -35,8 +35,9 @@ class FixedKLController:
 
 
 def dynamic_sampling_keep(metric_values, n_samples_per_prompt):
-    """Row indices kept by the DAPO filter, in order."""
-    values = np.asarray(metric_values, dtype=np.float64).reshape(-1)
+    """Row indices kept by the DAPO filter, in order.  ``np.std`` runs in the dtype it is given
+    (float32 metrics stay float32, python lists become float64), as in the reference."""
+    values = np.asarray(metric_values).reshape(-1)
     kept = []
     for lo in range(0, len(values), n_samples_per_prompt):
         group = values[lo:lo + n_samples_per_prompt]

@@ -1,0 +1,618 @@
+"""GPU parity tests: every HIP entry point, called through the C ABI (ctypes) by the package's
+host code, against the CPU oracle on the same seeded inputs.
+
+Tolerances (fp32 accumulate against the oracle's fp32 up-cast): index maps, masks and group
+assignment bit-exact; logp / entropy / advantages 1e-3 abs; loss 1e-4 rel; dlogits 2e-3 abs.
+The observed errors are far smaller; tighter bounds are asserted where the arithmetic allows.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import mindspeed_rl_amd as mrl
+from mindspeed_rl_amd import _lib
+from oracle import advantage as o_adv
+from oracle import loss as o_loss
+from oracle import packing as o_pack
+from oracle import vocab as o_vocab
+
+pytestmark = pytest.mark.gpu
+
+TOL_LOGP = 1e-3
+TOL_DLOGITS = 2e-3
+TOL_LOSS_REL = 1e-4
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    _lib.load()
+    return torch.device("cuda:0")
+
+
+def _logits(gen, rows, vocab, dtype, scale=3.0):
+    return (torch.randn(rows, vocab, generator=gen) * scale).to(dtype)
+
+
+# --------------------------------------------------------------------------------- vocab sweep
+@pytest.mark.parametrize("dtype,vocab,rows", [
+    (torch.float32, 32000, 64), (torch.bfloat16, 152064, 24), (torch.bfloat16, 129280, 16),
+    (torch.float16, 32000, 32), (torch.float32, 501, 37), (torch.bfloat16, 1003, 19),
+    (torch.bfloat16, 7, 5), (torch.float32, 3, 4), (torch.bfloat16, 8200, 9),
+])
+@pytest.mark.parametrize("label_dtype", [torch.int64, torch.int32])
+def test_vocab_forward_backward_parity(dev, dtype, vocab, rows, label_dtype):
+    gen = torch.Generator().manual_seed(vocab * 7 + rows)
+    z = _logits(gen, rows, vocab, dtype)
+    y = torch.randint(0, vocab, (rows,), generator=gen).to(label_dtype)
+    # incoming gradients of realistic size (|A|/N in training is far smaller still): a bf16 dlogit
+    # carries 2^-9 relative rounding, so the absolute tolerance presumes |dlogit| < 1
+    g_lp = torch.randn(rows, generator=gen) * 0.1
+    g_h = torch.randn(rows, generator=gen) * 0.01
+    g_lp[0] = 0.0
+    g_h[0] = 0.0                                        # a dead row: zeros without reading
+    # oracle on the fp32 up-cast
+    zo = z.float().requires_grad_()
+    lp_o = o_vocab.compute_log_probs(zo, y.long())
+    h_o = o_vocab.vocab_parallel_entropy(zo)
+    (dz_o,) = torch.autograd.grad((lp_o * g_lp).sum() + (h_o * g_h).sum(), zo)
+    lp64, h64, lse64 = o_vocab.logprob_entropy_fp64(z, y)
+
+    zd = z.to(dev).requires_grad_()
+    lp, h, lse = mrl.vocab_logprob_entropy(zd, y.to(dev))
+    assert lp.dtype == torch.float32 and lp.shape == (rows,)
+    assert (lp.cpu() - lp_o.detach()).abs().max().item() < TOL_LOGP
+    assert (h.cpu() - h_o.detach()).abs().max().item() < TOL_LOGP
+    # against fp64 the kernel is as good as the fp32 torch chain
+    assert (lp.cpu().double() - lp64).abs().max().item() < 2e-5
+    assert (h.cpu().double() - h64).abs().max().item() < 5e-5
+    assert (lse.cpu().double() - lse64).abs().max().item() < 2e-5
+    (dz,) = torch.autograd.grad([lp, h], zd, [g_lp.to(dev), g_h.to(dev)])
+    assert dz.dtype == dtype and dz.shape == z.shape
+    assert (dz.float().cpu() - dz_o).abs().max().item() < TOL_DLOGITS
+    assert torch.equal(dz[0].cpu(), torch.zeros(vocab, dtype=dtype))
+    assert torch.equal(zd.detach().cpu(), z), "the sweep must not write its input"
+
+
+def test_vocab_entropy_skipped_and_separate_functions(dev):
+    gen = torch.Generator().manual_seed(5)
+    z = _logits(gen, 33, 4096, torch.bfloat16)
+    y = torch.randint(0, 4096, (1, 33), generator=gen)
+    zd = z.to(dev).unsqueeze(0).requires_grad_()
+    lp = mrl.compute_log_probs(zd, y.to(dev))
+    assert lp.shape == (1, 33)
+    lp_o = o_vocab.compute_log_probs(z.float().unsqueeze(0), y)
+    assert (lp.detach().cpu() - lp_o).abs().max().item() < 1e-4
+    ent = mrl.vocab_parallel_entropy(zd)
+    assert (ent.detach().cpu() - o_vocab.vocab_parallel_entropy(z.float().unsqueeze(0))).abs().max().item() < 1e-4
+    ce = mrl.vocab_parallel_cross_entropy(vocab_parallel_logits=zd, target=y.to(dev))
+    assert torch.equal(ce, -lp)
+    # gradient of logp alone (no entropy term compiled in)
+    g = torch.randn(1, 33, generator=gen) * 0.1
+    (dz,) = torch.autograd.grad(lp, zd, g.to(dev))
+    zo = z.float().unsqueeze(0).requires_grad_()
+    (dz_o,) = torch.autograd.grad(o_vocab.compute_log_probs(zo, y), zo, g)
+    assert (dz.float().cpu() - dz_o).abs().max().item() < TOL_DLOGITS
+    # an injected cross entropy is honoured (the reference's hook)
+    calls = []
+
+    def fake_ce(vocab_parallel_logits, target):
+        calls.append(1)
+        return torch.zeros(target.shape, device=target.device)
+
+    mrl.set_vocab_parallel(fake_ce)
+    try:
+        assert mrl.compute_log_probs(zd, y.to(dev)).abs().sum().item() == 0 and calls
+    finally:
+        mrl.set_vocab_parallel(None)
+
+
+def test_vocab_out_of_range_labels_temperature_and_row_mask(dev):
+    gen = torch.Generator().manual_seed(6)
+    z = _logits(gen, 12, 2048, torch.float32, scale=4.0)
+    y = torch.randint(0, 2048, (12,), generator=gen)
+    y[3] = -1
+    y[7] = 2048
+    temp = 0.7
+    zo = (z / temp).requires_grad_()
+    lp_o = o_vocab.compute_log_probs(zo, y)
+    h_o = o_vocab.vocab_parallel_entropy(zo)
+    g = torch.randn(12, generator=gen)
+    (dz_o,) = torch.autograd.grad((lp_o * g).sum() + (h_o * 0.3).sum(), zo)
+    dz_o = dz_o / temp                                  # autograd of output.div_(temperature)
+    active = torch.ones(12, dtype=torch.bool)
+    active[5] = False
+    zd = z.to(dev).requires_grad_()
+    lp, h, _ = mrl.vocab_logprob_entropy(zd, y.to(dev), inv_temperature=1.0 / temp, row_active=active.to(dev))
+    keep = active.clone()
+    assert (lp.cpu()[keep] - lp_o.detach()[keep]).abs().max().item() < 1e-4
+    assert (h.cpu()[keep] - h_o.detach()[keep]).abs().max().item() < 1e-4
+    assert lp[5].item() == 0.0 and h[5].item() == 0.0
+    gd = g.clone()
+    gd[5] = 0.0
+    gh = torch.full((12,), 0.3)
+    gh[5] = 0.0
+    (dz,) = torch.autograd.grad([lp, h], zd, [gd.to(dev), gh.to(dev)])
+    dz_o[5] = 0.0
+    assert (dz.cpu() - dz_o).abs().max().item() < 1e-4
+
+
+def test_vocab_strided_rows_inplace_and_fp32_grad(dev):
+    gen = torch.Generator().manual_seed(8)
+    rows, vocab, stride = 10, 1000, 1024
+    buf = torch.zeros(rows, stride, dtype=torch.bfloat16)
+    buf[:, :vocab] = _logits(gen, rows, vocab, torch.bfloat16)
+    y = torch.randint(0, vocab, (rows,), generator=gen)
+    g = torch.randn(rows, generator=gen) * 0.1
+    zo = buf[:, :vocab].float().requires_grad_()
+    lp_o = o_vocab.compute_log_probs(zo, y)
+    (dz_o,) = torch.autograd.grad(lp_o, zo, g)
+    bd = buf.to(dev)
+    view = bd[:, :vocab]
+    lp = torch.empty(rows, device=dev)
+    lse = torch.empty(rows, device=dev)
+    s = _lib.stream(dev)
+    yd = y.to(dev)
+    _lib.call("mrl_vocab_logprob_fwd", view.data_ptr(), _lib.BF16, rows, vocab, stride, yd.data_ptr(), _lib.I64, None,
+              1.0, lp.data_ptr(), None, lse.data_ptr(), s)
+    assert (lp.cpu() - lp_o.detach()).abs().max().item() < 1e-4
+    gd = g.to(dev)
+    # fp32 gradient from bf16 logits, separate buffer with its own stride
+    d32 = torch.full((rows, 1000), 7.0, device=dev)
+    _lib.call("mrl_vocab_logprob_bwd", view.data_ptr(), _lib.BF16, rows, vocab, stride, yd.data_ptr(), _lib.I64, 1.0,
+              lse.data_ptr(), None, gd.data_ptr(), None, d32.data_ptr(), _lib.F32, 1000, s)
+    assert (d32.cpu() - dz_o).abs().max().item() < 1e-5
+    # in-place: dlogits overwrite the logits, padding columns stay untouched
+    bd[:, vocab:] = 5.0
+    _lib.call("mrl_vocab_logprob_bwd", view.data_ptr(), _lib.BF16, rows, vocab, stride, yd.data_ptr(), _lib.I64, 1.0,
+              lse.data_ptr(), None, gd.data_ptr(), None, view.data_ptr(), _lib.BF16, stride, s)
+    torch.cuda.synchronize()
+    assert (bd[:, :vocab].float().cpu() - dz_o).abs().max().item() < TOL_DLOGITS
+    assert (bd[:, vocab:] == 5.0).all().item()
+    # misaligned base pointer (odd element offset): scalar head/tail path and the scalar backward
+    flat = torch.zeros(rows * 1001 + 3, dtype=torch.bfloat16, device=dev)
+    odd = flat[3:].view(rows, 1001)[:, :1000]
+    odd.copy_(buf[:, :vocab].to(dev))
+    lp2 = torch.empty(rows, device=dev)
+    _lib.call("mrl_vocab_logprob_fwd", odd.data_ptr(), _lib.BF16, rows, vocab, 1001, yd.data_ptr(), _lib.I64, None, 1.0,
+              lp2.data_ptr(), None, lse.data_ptr(), s)
+    assert torch.allclose(lp2, lp, atol=1e-6)
+    dodd = torch.empty(rows, 1000, dtype=torch.bfloat16, device=dev)
+    _lib.call("mrl_vocab_logprob_bwd", odd.data_ptr(), _lib.BF16, rows, vocab, 1001, yd.data_ptr(), _lib.I64, 1.0,
+              lse.data_ptr(), None, gd.data_ptr(), None, dodd.data_ptr(), _lib.BF16, 1000, s)
+    assert (dodd.float().cpu() - dz_o).abs().max().item() < TOL_DLOGITS
+
+
+def test_vocab_properties_at_full_vocab(dev):
+    """Size-independent properties at the Qwen2.5 vocabulary (152064, bf16), generated on the device."""
+    torch.manual_seed(11)
+    rows, vocab = 512, 152064
+    z = (torch.randn(rows, vocab, device=dev) * 3).to(torch.bfloat16)
+    y = torch.randint(0, vocab, (rows,), device=dev)
+    zr = z.requires_grad_()
+    lp, h, lse = mrl.vocab_logprob_entropy(zr, y)
+    # against torch on the device in fp32 (a second, independent implementation)
+    ref = torch.log_softmax(z.float(), -1)
+    assert (lp - ref.gather(-1, y[:, None]).squeeze(-1)).abs().max().item() < 1e-4
+    ent_ref = -(ref.exp() * ref).sum(-1)
+    assert (h - ent_ref).abs().max().item() < 2e-4
+    assert ((h >= 0) & (h <= math.log(vocab) + 1e-4)).all().item()
+    # shifting a row by a constant that bf16 represents exactly leaves logp and entropy unchanged
+    z2 = (z.detach().float() + 8.0).to(torch.bfloat16)
+    exact = (z2.float() - 8.0 == z.detach().float()).all(-1)
+    lp2, h2, lse2 = mrl.vocab_logprob_entropy(z2, y)
+    assert exact.any().item()
+    assert (lp2 - lp)[exact].abs().max().item() < 1e-4 and (lse2 - lse - 8.0)[exact].abs().max().item() < 1e-4
+    # every row of dlogits sums to ~0 (softmax gradients are tangent to the simplex)
+    g_lp = torch.randn(rows, device=dev) * 0.1
+    g_h = torch.randn(rows, device=dev) * 0.01
+    (dz,) = torch.autograd.grad([lp, h], zr, [g_lp, g_h])
+    assert dz.float().sum(-1).abs().max().item() < 2e-2          # bf16 rounding of 152064 terms
+    closed = g_lp[:, None] * (torch.nn.functional.one_hot(y, vocab) - ref.exp()) \
+        - g_h[:, None] * ref.exp() * (z.detach().float() - (ref.exp() * z.detach().float()).sum(-1, keepdim=True))
+    assert (dz.float() - closed).abs().max().item() < TOL_DLOGITS
+    # linearity in the incoming gradient
+    (dz2,) = torch.autograd.grad([mrl.vocab_logprob_entropy(zr, y)[0]], zr, [2.0 * g_lp])
+    (dz1,) = torch.autograd.grad([mrl.vocab_logprob_entropy(zr, y)[0]], zr, [g_lp])
+    assert (dz2.float() - 2 * dz1.float()).abs().max().item() < 2e-3
+
+
+# --------------------------------------------------------------------------------- index maps
+def _random_lengths(gen, batch, width, max_prompt=6):
+    plen = torch.randint(1, max_prompt, (batch, 1), generator=gen, dtype=torch.int32)
+    rlen = torch.randint(0, width - max_prompt, (batch, 1), generator=gen, dtype=torch.int32)
+    return plen, rlen
+
+
+@pytest.mark.parametrize("align", [1, 2, 8, 16])
+@pytest.mark.parametrize("id_dtype", [torch.int64, torch.int32])
+def test_pack_unpack_bit_exact(dev, align, id_dtype):
+    gen = torch.Generator().manual_seed(100 + align)
+    batch, width, resp_w = 37, 96, 90
+    plen, rlen = _random_lengths(gen, batch, width)
+    rlen[4] = 0
+    rlen[5] = 0                                          # empty responses, back to back
+    ids = torch.randint(1, 50000, (batch, width), generator=gen).to(id_dtype)
+    labels = torch.cat([ids[:, 1:], torch.zeros(batch, 1, dtype=id_dtype)], 1)
+    mask_o = o_pack.generate_mask(ids, plen + rlen)
+    mask = mrl.generate_mask(ids.to(dev), (plen + rlen).to(dev))
+    assert mask.dtype == torch.int64 and torch.equal(mask.cpu(), mask_o)
+    want = o_pack.preprocess_packed_seqs(ids, labels, mask_o, align)
+    got = mrl.preprocess_packed_seqs(ids.to(dev), labels.to(dev), mask, align)
+    for a, b in zip(got, want):
+        assert a.dtype == b.dtype and a.shape == b.shape
+        assert torch.equal(a.cpu(), b)
+    _, _, _, seqlens, cu = got
+    # unpack, with and without the prompt shift, fp32 and int payloads, and a trailing dimension
+    packed = torch.randn(1, want[0].shape[1], generator=gen)
+    for prompt in (None, plen):
+        w = o_pack.postprocess_packed_seqs(packed, want[3], want[4], resp_w if prompt is not None else width, prompt)
+        g = mrl.postprocess_packed_seqs(packed.to(dev), seqlens, cu, resp_w if prompt is not None else width,
+                                        None if prompt is None else prompt.to(dev))
+        assert torch.equal(g.cpu(), w)
+    back = mrl.postprocess_packed_seqs(got[0], seqlens, cu, width)
+    assert torch.equal(back.cpu(), ids * mask_o.to(id_dtype))
+    p3 = torch.randn(1, want[0].shape[1], 5, generator=gen).to(torch.bfloat16)
+    w3 = o_pack.postprocess_packed_seqs(p3, want[3], want[4], resp_w, plen)
+    g3 = mrl.postprocess_packed_seqs(p3.to(dev), seqlens, cu, resp_w, plen.to(dev))
+    assert torch.equal(g3.cpu(), w3)
+    # adjoint: <unpack(x), g> == <x, scatter(g)>, and the scatter equals autograd of the oracle
+    x = packed.clone().requires_grad_()
+    go = torch.randn(batch, resp_w, generator=gen)
+    (gx_o,) = torch.autograd.grad(o_pack.postprocess_packed_seqs(x, want[3], want[4], resp_w, plen), x, go)
+    xd = packed.to(dev).requires_grad_()
+    (gx,) = torch.autograd.grad(mrl.postprocess_packed_seqs(xd, seqlens, cu, resp_w, plen.to(dev)), xd, go.to(dev))
+    assert torch.equal(gx.cpu(), gx_o)
+
+
+def test_pack_index_edge_cases(dev):
+    # empty batch row, all-zero mask rows, float and bool masks, int32 lengths
+    mask = torch.tensor([[1, 1, 1, 0], [0, 0, 0, 0], [1, 0, 0, 0], [1, 1, 1, 1]])
+    for cast in (torch.int64, torch.int32, torch.bool, torch.float32):
+        seqlens, cu, total = mrl.pack_index(mask.to(cast).to(dev), 4)
+        assert seqlens.tolist() == [3, 0, 1, 4] and cu.tolist() == [0, 4, 4, 8, 12] and total.item() == 12
+    ids = torch.arange(16).view(4, 4)
+    got = mrl.preprocess_packed_seqs(ids.to(dev), ids.to(dev), mask.to(dev), 4)
+    want = o_pack.preprocess_packed_seqs(ids, ids, mask, 4)
+    for a, b in zip(got, want):
+        assert torch.equal(a.cpu(), b)
+    # a batch larger than one scan chunk (1024) with ragged lengths
+    gen = torch.Generator().manual_seed(3)
+    lens = torch.randint(0, 50, (2500,), generator=gen, dtype=torch.int32)
+    big = o_pack.generate_mask(torch.zeros(2500, 50), lens)
+    seqlens, cu, total = mrl.pack_index(big.to(dev), 8)
+    padded = (lens + 7) // 8 * 8
+    assert torch.equal(seqlens.cpu(), lens)
+    assert cu.cpu().tolist() == [0] + torch.cumsum(padded, 0).tolist()
+    assert total.item() == int(padded.sum())
+
+
+def test_padded_window_bit_exact(dev, reference_vectors):
+    v = reference_vectors["truncate_middle_and_pad"]
+    out = mrl.truncate_middle_and_pad(torch.tensor(v["responses"]).to(dev), torch.tensor(v["input_tensor"]).to(dev),
+                                      torch.tensor(v["truncate_lengths"]).to(dev), v["pad_value"])
+    assert torch.equal(out.cpu(), torch.tensor(v["expected"]))
+    v = reference_vectors["generate_mask"]
+    m = mrl.generate_mask(torch.tensor(v["data_pad"]).to(dev), torch.tensor(v["seq_lengths"]).to(dev))
+    assert m.cpu().tolist() == v["expected"]
+    gen = torch.Generator().manual_seed(21)
+    batch, width, resp_w = 23, 70, 64
+    plen, rlen = _random_lengths(gen, batch, width)
+    window = o_pack.response_window(plen, rlen)
+    assert torch.equal(mrl.response_window(plen.to(dev), rlen.to(dev)).cpu(), window)
+    resp = torch.zeros(batch, resp_w)
+    vals = torch.randn(batch, width, generator=gen)
+    for pad in (0.0, -1.5):
+        want = o_pack.truncate_prompt_and_pad(resp, vals, window, pad)
+        got = mrl.truncate_prompt_and_pad(resp.to(dev), vals.to(dev), window.to(dev), pad)
+        assert torch.equal(got.cpu(), want)
+    v3 = torch.randn(batch, width, 6, generator=gen).to(torch.bfloat16)
+    assert torch.equal(mrl.truncate_middle_and_pad(resp.to(dev), v3.to(dev), window.to(dev)).cpu(),
+                       o_pack.truncate_middle_and_pad(resp, v3, window))
+    # windows that leave [0, width] are clamped like torch.clamp does
+    wild = window.clone()
+    wild[0] = torch.tensor([-3, 5])
+    wild[1] = torch.tensor([60, 200])
+    assert torch.equal(mrl.truncate_prompt_and_pad(resp.to(dev), vals.to(dev), wild.to(dev)).cpu(),
+                       o_pack.truncate_prompt_and_pad(resp, vals, wild))
+    x = vals.clone().requires_grad_()
+    go = torch.randn(batch, resp_w, generator=gen)
+    (gx_o,) = torch.autograd.grad(o_pack.truncate_prompt_and_pad(resp, x, window), x, go)
+    xd = vals.to(dev).requires_grad_()
+    (gx,) = torch.autograd.grad(mrl.truncate_prompt_and_pad(resp.to(dev), xd, window.to(dev)), xd, go.to(dev))
+    assert torch.equal(gx.cpu(), gx_o)
+
+
+# --------------------------------------------------------------------------------- advantages
+def test_group_advantage_parity(dev, reference_vectors):
+    v = reference_vectors["group_norm_advantage"]
+    adv, ret = mrl.compute_group_norm_advantage_return(
+        torch.tensor(v["token_level_rewards"]), torch.tensor(v["eos_mask"]).to(dev),
+        torch.tensor(v["response_length"]), v["n_sample_per_prompt"])
+    assert torch.allclose(adv.cpu(), torch.tensor(v["advantages"]), atol=1e-4)
+    assert torch.allclose(ret.cpu(), torch.tensor(v["returns"]), atol=1e-4)
+    assert adv.data_ptr() != ret.data_ptr()
+    gen = torch.Generator().manual_seed(31)
+    for batch, group, width in [(128, 8, 2048), (16, 4, 256), (128, 16, 333), (6, 1, 4), (64, 64, 7)]:
+        rewards = torch.bernoulli(torch.rand(batch // group, 1, generator=gen).repeat(1, group), generator=gen)
+        rewards = rewards.reshape(batch, 1)
+        rewards[:group] = 1.0                          # an all-equal group: exactly zero
+        lens = torch.randint(0, width + 1, (batch,), generator=gen)
+        for mask in (o_pack.generate_mask(torch.zeros(batch, width), lens),
+                     o_pack.generate_mask(torch.zeros(batch, width), lens).float(),
+                     o_pack.generate_mask(torch.zeros(batch, width), lens).bool()):
+            want, _ = o_adv.compute_group_norm_advantage_return(rewards, mask, torch.zeros(batch, 1), group)
+            got, got_ret = mrl.compute_group_norm_advantage_return(rewards.to(dev), mask.to(dev),
+                                                                   torch.zeros(batch, 1), group)
+            assert got.dtype == torch.float32 and got.shape == (batch, width)
+            if group == 1:
+                live = mask.bool()
+                assert torch.isnan(got.cpu()[live]).all() and torch.isnan(want[live]).all()
+                continue
+            assert (got.cpu() - want).abs().max().item() < 1e-6
+            assert torch.equal(got, got_ret)
+            assert torch.equal(got[:group].cpu(), torch.zeros(group, width))
+            # group assignment is row // G exactly: the sign pattern of each row follows its own group
+            assert torch.equal((got.cpu() != 0), (want != 0))
+    # gaussian rewards in fp64
+    rewards = torch.randn(48, 1, generator=gen, dtype=torch.float64)
+    mask = torch.ones(48, 3)
+    want, _ = o_adv.compute_group_norm_advantage_return(rewards, mask, torch.zeros(48, 1), 6)
+    got, _ = mrl.compute_group_norm_advantage_return(rewards.to(dev), mask.to(dev), torch.zeros(48, 1), 6)
+    assert (got.cpu() - want).abs().max().item() < 1e-6
+
+
+def test_dynamic_sampling_keep_bit_exact(dev):
+    rng = np.random.default_rng(7)
+    cases = [([1, 1, 1, 1, 0, 1, 0, 0, 0.5, 0.5, 0.5, 0.5, 0, 0, 0, 1e-100], 4), ([0, 0, 0, 1e-300], 4),
+             ([0.1, 0.1, 0.1], 3), ([0.1] * 4, 4), ([3.0, 3.0], 1), ([2.0, 2.0], 2), ([1, 0, 1, 1, 1], 2)]
+    for n, group in [(128, 16), (128, 8), (4096, 16), (300, 7), (2048, 256), (1000, 200)]:
+        p = rng.beta(0.5, 0.5, size=(n + group - 1) // group)
+        vals = (rng.random(n) < np.repeat(p, group)[:n]).astype(np.float64)
+        cases.append((vals.tolist(), group))
+        cases.append((np.round(rng.random(n), 1).tolist(), group))     # many equal-valued groups
+    for vals, group in cases:
+        for dt in (torch.float64, torch.float32):
+            t = torch.tensor(vals, dtype=dt)
+            want = o_adv.dynamic_sampling_keep(t.numpy(), group)
+            want = [i for i in want if i < len(vals)]
+            got = mrl.dynamic_sampling_keep(t.to(dev), group)
+            assert got == want, (vals[:8], group, dt)
+
+
+# --------------------------------------------------------------------------------- policy loss
+def _loss_case(gen, rows, cols):
+    lp = -torch.rand(rows, cols, generator=gen) * 3
+    old = lp + torch.randn(rows, cols, generator=gen) * 0.3
+    ref = lp + torch.randn(rows, cols, generator=gen) * 0.3
+    adv = torch.randn(rows, 1, generator=gen).repeat(1, cols)
+    ent = torch.rand(rows, cols, generator=gen) * 2
+    lens = torch.randint(1, cols + 1, (rows, 1), generator=gen, dtype=torch.int32)
+    return lp, old, ref, adv, ent, lens
+
+
+def _check_loss(got, want, g_got, g_want):
+    for a, b in zip(got, want):
+        a, b = float(a), float(b)
+        assert abs(a - b) <= TOL_LOSS_REL * abs(b) + 1e-7, (got, want)
+    for a, b in zip(g_got, g_want):
+        assert (a.cpu() - b).abs().max().item() <= 1e-6 + 1e-4 * b.abs().max().item()
+
+
+@pytest.mark.parametrize("kl", ["low_var_kl", "kl", "abs", "mse"])
+@pytest.mark.parametrize("with_old", [True, False])
+def test_grpo_policy_loss_parity(dev, kl, with_old):
+    gen = torch.Generator().manual_seed(41)
+    lp, old, ref, adv, ent, lens = _loss_case(gen, 16, 257)
+    if not with_old:
+        old = None
+    ref[0, :5] = lp[0, :5] + torch.tensor([25.0, -25.0, 3.0, -3.0, 0.0])    # both k3 clamps, abs at 0
+    mask = o_pack.generate_mask(lp, lens)
+    lp_o, ent_o = lp.clone().requires_grad_(), ent.clone().requires_grad_()
+    want = o_loss.grpo_policy_loss(old, lp_o, ref, adv, ent_o, mask, 0.2, 0.05, kl, 0.01)
+    g_want = torch.autograd.grad(want[0], [lp_o, ent_o])
+    ctrl = mrl.FixedKLController(0.05)
+    lp_d, ent_d = lp.to(dev).requires_grad_(), ent.to(dev).requires_grad_()
+    got = mrl.GRPOActorLossFunc._compute_grpo_policy_loss(
+        None if old is None else old.to(dev), lp_d, ref.to(dev), adv.to(dev), ent_d, mask.to(dev), 0.2, ctrl, kl, 0.01)
+    g_got = torch.autograd.grad(got[0], [lp_d, ent_d], torch.tensor(1.0, device=dev))
+    _check_loss(got, want, g_got, g_want)
+    # an upstream scale multiplies the gradient
+    got2 = mrl.GRPOActorLossFunc._compute_grpo_policy_loss(
+        None if old is None else old.to(dev), lp_d, ref.to(dev), adv.to(dev), ent_d, mask.to(dev), 0.2, ctrl, kl, 0.01)
+    (g2,) = torch.autograd.grad(got2[0] * 0.125, [lp_d])
+    assert torch.allclose(g2, g_got[0] * 0.125, atol=1e-9)
+
+
+def test_policy_loss_ties_clip_edges_and_nan_outside_mask(dev):
+    # ratio exactly on the clip bounds, zero advantages (ties), NaN outside the mask
+    lo, hi = float(np.float32(1.0 - 0.2)), float(np.float32(1.0 + 0.2))
+    old = torch.zeros(1, 8)
+    lp = torch.tensor([[math.log(lo), math.log(hi), 0.0, 0.5, -0.5, 0.1, float("nan"), 0.3]])
+    adv = torch.tensor([[1.0, -1.0, 0.0, 0.0, 0.0, -2.0, 1.0, float("nan")]])
+    mask = torch.tensor([[1, 1, 1, 1, 1, 1, 0, 0]])
+    ent = torch.zeros(1, 8)
+    lp_o = lp.clone().requires_grad_()
+    want = o_loss.grpo_policy_loss(old, lp_o, lp.detach().clone(), adv, ent, mask, 0.2, 0.0, "low_var_kl", 0.0)
+    (g_want,) = torch.autograd.grad(want[0], lp_o)
+    lp_d = lp.to(dev).requires_grad_()
+    got = mrl.GRPOActorLossFunc._compute_grpo_policy_loss(old.to(dev), lp_d, lp.to(dev), adv.to(dev), ent.to(dev),
+                                                           mask.to(dev), 0.2, mrl.FixedKLController(0.0),
+                                                           "low_var_kl", 0.0)
+    (g_got,) = torch.autograd.grad(got[0], lp_d)
+    assert not math.isnan(float(got[0]))
+    _check_loss(got, want, [g_got[:, :6]], [g_want[:, :6]])
+    assert torch.equal(g_got[:, 6:].cpu(), torch.zeros(1, 2))
+
+
+@pytest.mark.parametrize("token_level", [True, False])
+def test_dapo_policy_loss_parity(dev, token_level, reference_vectors):
+    v = reference_vectors["dapo_policy_loss_inputs"]
+    t = {k: torch.tensor(v[k], dtype=torch.float32) for k in ("old_log_prob", "log_prob", "entropy", "advantages",
+                                                              "eos_mask")}
+    for old in (t["old_log_prob"], None):
+        want = o_loss.dapo_policy_loss(old, t["log_prob"], t["entropy"], v["entropy_coeff"], t["advantages"],
+                                       t["eos_mask"], v["clip_ratio_low"], v["clip_ratio_high"], token_level)
+        got = mrl.DAPOActorLossFunc._compute_dapo_policy_loss(
+            None if old is None else old.to(dev), t["log_prob"].to(dev), t["entropy"].to(dev), v["entropy_coeff"],
+            t["advantages"].to(dev), t["eos_mask"].to(dev), v["clip_ratio_low"], v["clip_ratio_high"], token_level)
+        assert len(got) == 5 and all(isinstance(x, torch.Tensor) for x in got)
+        _check_loss(got, want, [], [])
+    gen = torch.Generator().manual_seed(43)
+    lp, old, _, adv, ent, lens = _loss_case(gen, 24, 500)
+    mask = o_pack.generate_mask(lp, lens).float()
+    lp_o, ent_o = lp.clone().requires_grad_(), ent.clone().requires_grad_()
+    want = o_loss.dapo_policy_loss(old, lp_o, ent_o, 0.003, adv, mask, 0.2, 0.28, token_level)
+    g_want = torch.autograd.grad(want[0], [lp_o, ent_o])
+    lp_d, ent_d = lp.to(dev).requires_grad_(), ent.to(dev).requires_grad_()
+    got = mrl.DAPOActorLossFunc._compute_dapo_policy_loss(old.to(dev), lp_d, ent_d, 0.003, adv.to(dev), mask.to(dev),
+                                                           0.2, 0.28, token_level)
+    g_got = torch.autograd.grad(got[0], [lp_d, ent_d])
+    _check_loss(got, want, g_got, g_want)
+    assert float(got[3]) == 0.0
+    if not token_level:
+        assert float(got[1]) == 0.0                    # the reference's overwritten-operand clip fraction
+        mask[3] = 0                                    # an all-masked row: NaN, as in the reference
+        got = mrl.DAPOActorLossFunc._compute_dapo_policy_loss(old.to(dev), lp.to(dev), ent.to(dev), 0.0, adv.to(dev),
+                                                               mask.to(dev), 0.2, 0.28, False)
+        assert math.isnan(float(got[0]))
+
+
+# --------------------------------------------------------------------------------- end to end
+def _make_batch(gen, n_prompts, group, r_lo, r_hi, vocab, dtype, scale, align, prompt_hi=2):
+    """Synthetic GRPO micro-batch in the layout the training engine hands to the loss."""
+    batch = n_prompts * group
+    rlen = torch.randint(r_lo, r_hi + 1, (batch, 1), generator=gen, dtype=torch.int32)
+    plen = torch.randint(1, prompt_hi + 1, (batch, 1), generator=gen, dtype=torch.int32)
+    width = int((plen + rlen).max())
+    resp_w = int(rlen.max())
+    ids = torch.randint(0, vocab, (batch, width), generator=gen)
+    mask1d = o_pack.generate_mask(ids, plen + rlen)
+    ids = ids * mask1d
+    labels = torch.cat([ids[:, 1:], torch.zeros(batch, 1, dtype=ids.dtype)], 1)
+    p_ids, _, p_lab, seqlens, cu = o_pack.preprocess_packed_seqs(ids, labels, mask1d, align)
+    total = p_ids.shape[1]
+    logits = (torch.randn(1, total, vocab, generator=gen) * scale).to(dtype)
+    p = torch.rand(n_prompts, 1, generator=gen).repeat(1, group).reshape(batch, 1)
+    rewards = torch.bernoulli(p, generator=gen)
+    rmask = o_pack.generate_mask(torch.zeros(batch, resp_w), rlen)
+    adv, _ = o_adv.compute_group_norm_advantage_return(rewards, rmask, rlen, group)
+    b = {"labels": p_lab, "responses": torch.zeros(batch, resp_w, dtype=torch.int32), "response_length": rlen,
+         "prompt_length": plen, "advantages": adv}
+    kw = dict(use_remove_padding=True, seqlens_in_batch=seqlens, cu_seqlens_padded=cu, seq_len=width)
+    # behaviour / reference policy log-probs: current + N(0, 0.05), from the oracle, detached
+    lp0 = o_loss.logprob_computer(logits.float(), b, True, **kw)[0]
+    b["old_log_prob"] = (lp0 + torch.randn(lp0.shape, generator=gen) * 0.05) * rmask
+    b["ref_log_prob"] = (lp0 + torch.randn(lp0.shape, generator=gen) * 0.05) * rmask
+    return logits, b, kw, rewards, (ids, labels, mask1d)
+
+
+def _to_dev(d, dev):
+    return {k: (v.to(dev) if isinstance(v, torch.Tensor) else v) for k, v in d.items()}
+
+
+@pytest.mark.parametrize("entropy_coeff", [0.0, 0.001])
+def test_grpo_compute_loss_config0_packed(dev, entropy_coeff):
+    """configs[0]: 4 prompts x G=4, R in [64,256], V=32000 fp32 logits ~N(0,2), eps 0.2, k3 KL 0.001."""
+    gen = torch.Generator().manual_seed(0)
+    logits, b, kw, rewards, _ = _make_batch(gen, 4, 4, 64, 256, 32000, torch.float32, 2.0, 1, prompt_hi=1)
+    meta = dict(clip_ratio=0.2, kl_coef=0.001, kl_penalty="low_var_kl", entropy_coeff=entropy_coeff)
+    zo = logits.clone().requires_grad_()
+    want_loss, want_stats = o_loss.grpo_compute_loss(zo, b, meta, **kw)
+    (dz_o,) = torch.autograd.grad(want_loss, zo)
+
+    f = mrl.LossFuncFactory.get_instance("ray_grpo", "actor")
+    f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.001), "kl_penalty": "low_var_kl",
+                          "entropy_coeff": entropy_coeff})
+    zd = logits.to(dev).requires_grad_()
+    bd, kwd = _to_dev(b, dev), _to_dev(kw, dev)
+    # advantages computed on the device from the rewards agree with the oracle's
+    rmask = mrl.generate_mask(bd["responses"], bd["response_length"])
+    adv_d, _ = mrl.compute_group_norm_advantage_return(rewards.to(dev), rmask, bd["response_length"], 4)
+    assert (adv_d.cpu() - b["advantages"]).abs().max().item() < 1e-6
+    lp = f.compute_loss(zd, bd, forward_only=True, **kwd)
+    lp_o = o_loss.grpo_compute_loss(logits, b, meta, forward_only=True, **kw)
+    assert lp.shape == lp_o.shape and (lp.cpu() - lp_o).abs().max().item() < TOL_LOGP
+    loss, stats = f.compute_loss(zd, bd, **kwd)
+    assert loss.dim() == 0 and set(stats) == set(want_stats)
+    assert all(isinstance(x, float) for x in stats.values())
+    assert abs(loss.item() - want_loss.item()) <= TOL_LOSS_REL * abs(want_loss.item()) + 1e-7
+    for k in want_stats:
+        assert abs(stats[k] - want_stats[k]) <= TOL_LOSS_REL * abs(want_stats[k]) + 1e-6, k
+    (dz,) = torch.autograd.grad(loss, zd)
+    assert (dz.cpu() - dz_o).abs().max().item() < TOL_DLOGITS
+    scale = dz_o.abs().max().item()
+    assert (dz.cpu() - dz_o).abs().max().item() < 1e-3 * scale + 1e-9      # relative, since dlogits are tiny
+    # Megatron scales the loss before backward: the gradient follows
+    (dz2,) = torch.autograd.grad(f.compute_loss(zd, bd, **kwd)[0] * 64.0, zd)
+    assert torch.allclose(dz2, dz * 64.0, rtol=1e-5, atol=1e-12)
+    # dynamic batch size rescales the loss only
+    loss3, stats3 = f.compute_loss(zd, bd, use_dynamic_bsz=True, actual_micro_batch_size=4.0, **kwd)
+    assert loss3.item() == pytest.approx(loss.item() * 4.0, rel=1e-6) and stats3 == stats
+    ref = mrl.LossFuncFactory.get_instance("ray_grpo", "reference")
+    assert torch.equal(ref.compute_loss(zd, bd, forward_only=True, **kwd), lp)
+    assert ref.compute_loss(zd, bd, forward_only=False, **kwd) is None
+    with pytest.raises(ValueError, match="The responses is None"):
+        f.compute_loss(zd, {k: v for k, v in bd.items() if k != "responses"},
+                       **{k: v for k, v in kwd.items() if k != "use_remove_padding"})
+
+
+def test_padded_vs_packed_and_dapo_bf16(dev):
+    """configs[2]/[4] in small: the same responses as a padded [B,S] batch and packed with
+    alignment 8, bf16 logits, an empty-response group, DAPO clip-higher with sequence mean."""
+    gen = torch.Generator().manual_seed(2)
+    logits, b, kw, rewards, (ids, labels, mask1d) = _make_batch(gen, 3, 4, 5, 40, 4096, torch.bfloat16, 3.0, 8)
+    b["response_length"][4:8] = 0            # note: lengths only shrink the loss mask here
+    meta = dict(entropy_coeff=0.002, token_level_loss=True, clip_higher_enable=True, clip_ratio_low=0.2,
+                clip_ratio_high=0.28)
+    batch, width = ids.shape
+    seqlens, cu = kw["seqlens_in_batch"], kw["cu_seqlens_padded"]
+    padded = torch.zeros(batch, width, 4096, dtype=torch.bfloat16)
+    for i in range(batch):
+        padded[i, :seqlens[i]] = logits[0, cu[i]:cu[i] + seqlens[i]]
+    f = mrl.LossFuncFactory.get_instance("ray_dapo", "actor")
+    f.add_loss_meta_info({"entropy_coeff": 0.002, "token_level_loss": True, "clip_higher_enable": True,
+                          "clip_ratio_low": 0.2, "clip_ratio_high": 0.28, "clip_ratio": 0.2})
+    bd, kwd = _to_dev(b, dev), _to_dev(kw, dev)
+    zo = logits.float().requires_grad_()
+    want_loss, want_stats = o_loss.dapo_compute_loss(zo, b, meta, **kw)
+    (dz_o,) = torch.autograd.grad(want_loss, zo)
+    zd = logits.to(dev).requires_grad_()
+    loss, stats = f.compute_loss(zd, bd, **kwd)
+    assert abs(loss.item() - want_loss.item()) <= TOL_LOSS_REL * abs(want_loss.item()) + 1e-7
+    for k in want_stats:
+        assert abs(stats[k] - want_stats[k]) <= TOL_LOSS_REL * abs(want_stats[k]) + 1e-6, k
+    (dz,) = torch.autograd.grad(loss, zd)
+    assert dz.dtype == torch.bfloat16
+    assert (dz.float().cpu() - dz_o).abs().max().item() < TOL_DLOGITS
+    # padded layout through the same loss object: same loss, same statistics
+    bp = dict(bd, labels=labels.to(dev))
+    zp = padded.to(dev).requires_grad_()
+    loss_p, stats_p = f.compute_loss(zp, bp)
+    assert loss_p.item() == pytest.approx(loss.item(), rel=1e-6)
+    for k in stats:
+        assert stats_p[k] == pytest.approx(stats[k], rel=1e-6, abs=1e-9)
+    (dzp,) = torch.autograd.grad(loss_p, zp)
+    for i in range(batch):
+        assert torch.equal(dzp[i, :seqlens[i]].cpu(), dz[0, cu[i]:cu[i] + seqlens[i]].cpu())
+    # sequence-mean mode and a response mask handed in by the caller
+    f.add_loss_meta_info({"token_level_loss": False})
+    meta["token_level_loss"] = False
+    b2 = dict(b, response_length=torch.clamp(b["response_length"], min=1))
+    rm = o_pack.generate_mask(b["responses"], b2["response_length"]).float()
+    rm[:, ::3] = 0
+    rm[:, 0] = 1
+    b2["response_mask"] = rm
+    want_loss, want_stats = o_loss.dapo_compute_loss(logits.float(), b2, meta, **kw)
+    loss, stats = f.compute_loss(zd, _to_dev(b2, dev), **kwd)
+    assert abs(loss.item() - want_loss.item()) <= TOL_LOSS_REL * abs(want_loss.item()) + 1e-7
+    assert stats["actor/pg_clipfrac"] == 0.0 and stats["actor/kl_loss"] == 0.0
+
+
+def test_copy_kernel_moves_bytes(dev):
+    src = torch.randint(0, 255, (1 << 20,), dtype=torch.uint8, device=dev)
+    dst = torch.zeros_like(src)
+    _lib.call("mrl_copy_bytes", src.data_ptr(), dst.data_ptr(), src.numel(), _lib.stream(dev))
+    assert torch.equal(src, dst)
