@@ -30,7 +30,6 @@ def compute_group_norm_advantage_return(token_level_rewards, eos_mask, response_
     mask = eos_mask
     if mask.dtype not in (torch.float32, torch.int64, torch.int32, torch.uint8, torch.bool):
         mask = mask.to(torch.float32)
-    mask = mask.contiguous()
     dev = _lib.require_device(mask)
     rewards = torch.as_tensor(token_level_rewards).detach()
     if rewards.dtype not in (torch.float32, torch.float64):
@@ -41,8 +40,9 @@ def compute_group_norm_advantage_return(token_level_rewards, eos_mask, response_
         raise RuntimeError("shape '%s' is invalid for input of size %d" % (list(response_length.shape), batch))
     if batch % n_sample_per_prompt != 0:
         raise RuntimeError("shape '[-1, %d]' is invalid for input of size %d" % (n_sample_per_prompt, batch))
-    if mask.dim() != 2 or mask.shape[0] != batch:
-        raise RuntimeError("eos_mask must have shape (%d, L)" % batch)
+    if mask.dim() != 2 or mask.shape[0] not in (1, batch):
+        raise RuntimeError("eos_mask must have shape (%d, L) or (1, L)" % batch)
+    mask = mask.expand(batch, mask.shape[1]).contiguous()      # the reference broadcasts the mask
     width = mask.shape[1]
     adv = torch.empty((batch, width), dtype=torch.float32, device=dev)
     ret = torch.empty((batch, width), dtype=torch.float32, device=dev)
