@@ -221,6 +221,79 @@ int mrl_policy_loss_bwd(const float* log_prob, const float* old_log_prob,
                         const float* upstream, float* g_log_prob, float* g_entropy, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Fused forward + backward ("eager gradient").  The loss gradient of a token depends only on
+ * that token's own log-prob, its old/ref log-probs, advantage and mask, and on denominators
+ * that are known from the mask before the sweep - so dlogits can be produced in the SAME pass
+ * that computes the log-prob: one read of the logits and one write of dlogits for the whole
+ * path (2 bytes-moved units instead of 3), with each row held in registers by one workgroup.
+ * Replaces, in one chain: compute_log_probs + vocab_parallel_entropy (utils/compute.py:29-97),
+ * postprocess_packed_seqs / truncate_prompt_and_pad (the response window), the policy loss
+ * (grpo_actor_loss_func.py:127-144, dapo_actor_loss_func.py:129-152) and all their backwards.
+ *
+ * Call order: mrl_fused_loss_prepare -> mrl_fused_logprob_loss -> mrl_fused_loss_reduce, and
+ * mrl_scale_rows when autograd later delivers an upstream gradient.
+ */
+
+/* Largest vocabulary the row-in-registers kernels hold for a logits dtype (0 = bad dtype). */
+int64_t mrl_fused_max_vocab(int logits_dtype);
+
+/* Step 1.  Maps the [batch, width] loss operands onto logits rows.
+ *   layout 0, packed [n_rows, V] logits: sequence i owns the rows postprocess_packed_seqs copies
+ *     (start = cu[i], n = seqlens[i]; with prompt_length and P_i - 1 < n: n -= P_i, start += P_i - 1);
+ *   layout 1, padded [batch, padded_seq_len, V] logits: rows [P_i - 1, P_i + R_i - 1) clamped to
+ *     [0, padded_seq_len] of block i (base_loss_func.py:47-53, pad_process.py:120-123).
+ * Row start_i + j holds token (i, j), j < min(n, width).  The mask is `mask` ([batch, width] F32,
+ * I64, I32, U8) or j < response_length[i].  old_log_prob / ref_log_prob may be NULL.
+ * Outputs: row_start int64 [batch], row_count int32 [batch], seq_mask_sum float [batch] (sum of
+ * each mask row), row_ops float [n_rows * 8] = {old, ref, adv, mask, w_pg, 1/(N+1e-8), 0, 0} per
+ * logits row, mask = 0 for rows outside every window; N = sum of the whole mask; w_pg is
+ * 1/(N+1e-8) (seq_mean 0) or 1/(batch * seq_mask_sum[i]) (seq_mean 1).  prompt_length >= 1. */
+int mrl_fused_loss_prepare(int layout, int64_t batch, int64_t width, int64_t n_rows,
+                           const int32_t* seqlens, const int32_t* cu_seqlens_padded,
+                           int64_t padded_seq_len, const void* prompt_length, int prompt_dtype,
+                           const void* response_length, int response_dtype,
+                           const float* old_log_prob, const float* ref_log_prob,
+                           const float* advantages, const void* mask, int mask_dtype, int seq_mean,
+                           int64_t* row_start, int32_t* row_count, float* seq_mask_sum,
+                           float* row_ops, void* stream);
+
+/* Step 2.  The sweep.  Per row with a non-zero mask: logp, entropy (if `entropy` is given) as in
+ * mrl_vocab_logprob_fwd; the token's loss terms as in mrl_policy_loss_fwd; then
+ *   dlogits = grad_scale * d(loss)/d(logits)   (grad_scale = loss_scale * the upstream gradient
+ *   the caller expects, normally 1)
+ * written in the logits dtype.  Rows with mask 0 get zero dlogits and are not read.  dlogits may
+ * alias logits exactly (in-place).  row_terms float [n_rows * 8] receives {pg, clipped, old-lp,
+ * kl, entropy, 1} * mask per row for step 3.  logp / entropy: nullable [n_rows] outputs.
+ * has_old = 0 means old_log_prob = log_prob.detach() (ratio 1).  Needs 16-byte aligned rows,
+ * vocab % (16/elem) == 0 and vocab <= mrl_fused_max_vocab(dtype), else MRL_ERR_UNSUPPORTED (use
+ * the split fwd/bwd entry points then). */
+int mrl_fused_logprob_loss(const void* logits, int logits_dtype, int64_t n_rows, int64_t vocab,
+                           int64_t row_stride, const void* labels, int labels_dtype,
+                           float inv_temperature, const float* row_ops, int has_old,
+                           float clip_lo, float clip_hi, int kl_penalty, float kl_coef,
+                           float entropy_coeff, float grad_scale, void* dlogits,
+                           int64_t dlogits_row_stride, float* logp, float* entropy,
+                           float* row_terms, void* stream);
+
+/* Step 3.  Sums row_terms per sequence (tokens with a non-zero mask but no logits row enter with
+ * log_prob = entropy = 0, as in the split path) and finalizes out[8] / row_sums exactly like
+ * mrl_policy_loss_fwd. */
+int mrl_fused_loss_reduce(const float* row_terms, const int64_t* row_start,
+                          const int32_t* row_count, int64_t batch, int64_t width,
+                          const float* old_log_prob, const float* ref_log_prob,
+                          const float* advantages, const void* mask, int mask_dtype,
+                          const void* response_length, int response_dtype, float clip_lo,
+                          float clip_hi, int kl_penalty, float kl_coef, float entropy_coeff,
+                          int seq_mean, float loss_scale, float* row_sums, float* out,
+                          void* stream);
+
+/* x[r, :] *= (*upstream / assumed) in place, unless that ratio is exactly 1 (then the kernel
+ * exits without touching memory).  Lets the eager gradient honour whatever scalar autograd
+ * delivers (Megatron's 1/num_microbatches and loss scale) without a host synchronisation. */
+int mrl_scale_rows(void* x, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                   const float* upstream, float assumed, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Plain device-to-device copy kernel of n_bytes (multiple of 16, 16-byte aligned pointers);
  * used to calibrate the rocprofv3 FETCH_SIZE / WRITE_SIZE counters and as the measured
  * bandwidth ceiling next to the 8 TB/s vendor peak.  No counterpart in the reference. */

@@ -7,119 +7,15 @@
 // one element-wise launch that re-derives each token's local gradient from the inputs and the
 // saved denominators.
 #include "mrl_internal.h"
+#include "policy_terms.h"
+#include "row_sweep.h"
 
 namespace {
 
+using namespace mrl_loss;
+
 constexpr int kBlock = 256;
 constexpr int kWaves = kBlock / 64;
-
-// slots of row_sums[i*8 + ...]
-enum { S_PG = 0, S_CLIP = 1, S_PPOKL = 2, S_KL = 3, S_ENT = 4, S_MASK = 5, S_N = 8 };
-
-struct Params {
-    float clip_lo, clip_hi, kl_coef, entropy_coeff, loss_scale;
-    int kl_penalty, seq_mean;
-};
-
-__device__ __forceinline__ float mask_at(const void* __restrict__ mask, int mdtype, const void* __restrict__ lens,
-                                         int ldtype, int64_t i, int64_t j, int64_t width) {
-    if (mask != nullptr) {
-        const int64_t e = i * width + j;
-        switch (mdtype) {
-            case MRL_I64: return (float) reinterpret_cast<const int64_t*>(mask)[e];
-            case MRL_I32: return (float) reinterpret_cast<const int32_t*>(mask)[e];
-            case MRL_U8: return (float) reinterpret_cast<const uint8_t*>(mask)[e];
-            default: return reinterpret_cast<const float*>(mask)[e];
-        }
-    }
-    const int64_t n = ldtype == MRL_I32 ? (int64_t) reinterpret_cast<const int32_t*>(lens)[i]
-                                        : reinterpret_cast<const int64_t*>(lens)[i];
-    return j < n ? 1.f : 0.f;
-}
-
-// torch.maximum: NaN wins
-__device__ __forceinline__ float torch_max(float a, float b) {
-    if (a != a) return a;
-    if (b != b) return b;
-    return a > b ? a : b;
-}
-
-__device__ __forceinline__ float clampf(float x, float lo, float hi) {
-    // torch.clamp(x, lo, hi) = min(max(x, lo), hi), NaN propagates
-    if (x != x) return x;
-    return fminf(fmaxf(x, lo), hi);
-}
-
-struct Token {
-    float pg;        // max(surr1, surr2)
-    float clipped;   // surr2 > surr1
-    float neg_logr;  // old - lp
-    float kl;        // KL penalty term
-    float d_pg;      // d pg / d lp
-    float d_kl;      // d kl / d lp
-};
-
-template <bool kGrad>
-__device__ __forceinline__ Token token_terms(float lp, float old, bool has_old, float ref, float adv,
-                                             const Params& p) {
-    Token t;
-    const float logr = has_old ? lp - old : 0.f;   // old == lp.detach() when absent
-    const float ratio = expf(logr);
-    t.neg_logr = -logr;
-    const float na = -adv;
-    const float clipped_ratio = clampf(ratio, p.clip_lo, p.clip_hi);
-    const float s1 = na * ratio;
-    const float s2 = na * clipped_ratio;
-    t.pg = torch_max(s1, s2);
-    t.clipped = s2 > s1 ? 1.f : 0.f;
-    t.d_pg = 0.f;
-    t.d_kl = 0.f;
-    if (kGrad) {
-        // d s1/d lp = na*ratio; d s2/d lp = na*ratio inside the closed clip interval, else 0;
-        // torch.maximum sends the gradient to the larger operand and halves it on ties
-        const float g1 = na * ratio;
-        const float g2 = (ratio >= p.clip_lo && ratio <= p.clip_hi) ? g1 : 0.f;
-        if (s1 > s2) t.d_pg = g1;
-        else if (s2 > s1) t.d_pg = g2;
-        else if (s1 == s2) t.d_pg = 0.5f * g1 + 0.5f * g2;
-        else t.d_pg = s1 + s2;   // NaN operands: propagate NaN
-    }
-    switch (p.kl_penalty) {
-        case MRL_KL_KL:
-            t.kl = lp - ref;
-            if (kGrad) t.d_kl = 1.f;
-            break;
-        case MRL_KL_ABS: {
-            const float d = lp - ref;
-            t.kl = fabsf(d);
-            if (kGrad) t.d_kl = d > 0.f ? 1.f : (d < 0.f ? -1.f : 0.f);
-            break;
-        }
-        case MRL_KL_MSE: {
-            const float d = lp - ref;
-            t.kl = 0.5f * (d * d);
-            if (kGrad) t.d_kl = d;
-            break;
-        }
-        case MRL_KL_LOW_VAR: {
-            const float raw = ref - lp;
-            const float c = clampf(raw, -20.f, 20.f);
-            const float e = expf(c);
-            const float k3 = e - c - 1.f;
-            t.kl = clampf(k3, -10.f, 10.f);
-            if (kGrad) {
-                const bool inner = raw >= -20.f && raw <= 20.f;
-                const bool outer = k3 >= -10.f && k3 <= 10.f;
-                t.d_kl = (inner && outer) ? -(e - 1.f) : 0.f;
-            }
-            break;
-        }
-        default:
-            t.kl = 0.f;
-            break;
-    }
-    return t;
-}
 
 __device__ __forceinline__ double block_sum(double v, double* lds) {
 #pragma unroll
@@ -131,6 +27,10 @@ __device__ __forceinline__ double block_sum(double v, double* lds) {
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) r += lds[w];
     return r;
+}
+
+__device__ __forceinline__ int64_t load_i64(const void* p, int dtype, int64_t i) {
+    return dtype == MRL_I32 ? (int64_t) reinterpret_cast<const int32_t*>(p)[i] : reinterpret_cast<const int64_t*>(p)[i];
 }
 
 __global__ __launch_bounds__(kBlock) void policy_loss_rows_kernel(
@@ -227,6 +127,134 @@ __global__ __launch_bounds__(kBlock) void policy_loss_bwd_kernel(
     if (g_ent) g_ent[e] = gent;
 }
 
+// ----------------------------------------------------------------------------- fused-path helpers
+// Window of logits rows that belongs to sequence i, and the sum of its mask row.
+//   layout 0 (packed [T, V] logits): the window postprocess_packed_seqs copies
+//   layout 1 (padded [B, S, V] logits): [P-1, P+R-1) clamped to [0, S], inside row block i
+__global__ __launch_bounds__(kBlock) void fused_seq_kernel(
+    int layout, int64_t width, const int32_t* __restrict__ seqlens, const int32_t* __restrict__ cu, int64_t padded_s,
+    const void* __restrict__ prompt, int pdtype, const void* __restrict__ resp, int rdtype,
+    const void* __restrict__ mask, int mdtype, int64_t* __restrict__ row_start, int32_t* __restrict__ row_count,
+    float* __restrict__ seq_msum) {
+    __shared__ double lds[kWaves];
+    const int64_t i = blockIdx.x;
+    float acc = 0.f;
+    for (int64_t j = threadIdx.x; j < width; j += kBlock) acc += mask_at(mask, mdtype, resp, rdtype, i, j, width);
+    const double msum = block_sum((double)acc, lds);
+    if (threadIdx.x == 0) {
+        int64_t start, n;
+        if (layout == 0) {
+            start = (int64_t)cu[i];
+            n = (int64_t)seqlens[i];
+            if (prompt != nullptr) {
+                const int64_t skip = load_i64(prompt, pdtype, i) - 1;
+                if (skip < n) {
+                    n -= skip + 1;
+                    start += skip;
+                }
+            }
+        } else {
+            const int64_t p = load_i64(prompt, pdtype, i), r = load_i64(resp, rdtype, i);
+            int64_t lo = p - 1, hi = p + r - 1;
+            lo = lo < 0 ? 0 : (lo > padded_s ? padded_s : lo);
+            hi = hi < 0 ? 0 : (hi > padded_s ? padded_s : hi);
+            start = i * padded_s + lo;
+            n = hi - lo;
+        }
+        if (n < 0) n = 0;
+        if (n > width) n = width;
+        row_start[i] = start;
+        row_count[i] = (int32_t)n;
+        seq_msum[i] = (float)msum;
+    }
+}
+
+// Loss operands of every logits row: one thread per row finds its (sequence, token) by a binary
+// search over the window starts.  Every workgroup first re-derives N = sum of all mask sums in a
+// fixed order (batch is small), so no extra launch or atomic is needed.
+__global__ __launch_bounds__(kBlock) void fused_row_ops_kernel(
+    int64_t batch, int64_t width, int64_t n_rows, const int64_t* __restrict__ row_start,
+    const int32_t* __restrict__ row_count, const float* __restrict__ seq_msum, const float* __restrict__ old,
+    const float* __restrict__ ref, const float* __restrict__ adv, const void* __restrict__ mask, int mdtype,
+    const void* __restrict__ resp, int rdtype, int seq_mean, float* __restrict__ row_ops) {
+    __shared__ double lds[kWaves];
+    double part = 0.0;
+    for (int64_t i = threadIdx.x; i < batch; i += kBlock) part += (double)seq_msum[i];
+    const double total = block_sum(part, lds);
+    const float inv_tok = (float)(1.0 / (total + 1e-8));
+    const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (t >= n_rows) return;
+    float o = 0.f, rf = 0.f, a = 0.f, m = 0.f, wpg = 0.f;
+    if (batch > 0 && t >= row_start[0]) {
+        int64_t lo = 0, hi = batch;                     // largest i with row_start[i] <= t
+        while (hi - lo > 1) {
+            const int64_t mid = (lo + hi) >> 1;
+            if (row_start[mid] <= t) lo = mid; else hi = mid;
+        }
+        const int64_t i = lo, j = t - row_start[i];
+        if (j < (int64_t)row_count[i]) {
+            m = mask_at(mask, mdtype, resp, rdtype, i, j, width);
+            if (m != 0.f) {
+                const int64_t e = i * width + j;
+                o = old ? old[e] : 0.f;
+                rf = ref ? ref[e] : 0.f;
+                a = adv[e];
+                wpg = seq_mean ? 1.f / ((float)batch * seq_msum[i]) : inv_tok;
+            }
+        }
+    }
+    float* ops = row_ops + t * MRL_ROW_OPS;
+    ops[MRL_OP_OLD] = o;
+    ops[MRL_OP_REF] = rf;
+    ops[MRL_OP_ADV] = a;
+    ops[MRL_OP_MASK] = m;
+    ops[MRL_OP_WPG] = wpg;
+    ops[MRL_OP_INVTOK] = inv_tok;
+    ops[6] = 0.f;
+    ops[7] = 0.f;
+}
+
+// Per-sequence sums of the per-row loss terms written by the fused sweep.  Tokens that carry a
+// non-zero mask but have no logits row (j >= row_count) enter with log_prob = entropy = 0, which
+// is what they hold in the unpacked [B, L] tensor of the split path.
+__global__ __launch_bounds__(kBlock) void fused_seq_reduce_kernel(
+    const float* __restrict__ row_terms, const int64_t* __restrict__ row_start, const int32_t* __restrict__ row_count,
+    int64_t width, const float* __restrict__ old, const float* __restrict__ ref, const float* __restrict__ adv,
+    const void* __restrict__ mask, int mdtype, const void* __restrict__ resp, int rdtype, Params p,
+    float* __restrict__ row_sums) {
+    __shared__ double lds[kWaves];
+    const int64_t i = blockIdx.x;
+    const int64_t start = row_start[i];
+    const int64_t count = row_count[i];
+    float acc[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int64_t j = threadIdx.x; j < width; j += kBlock) {
+        if (j < count) {
+            const float* t = row_terms + (start + j) * S_N;
+#pragma unroll
+            for (int q = 0; q < 6; ++q) acc[q] += t[q];
+        } else {
+            const float m = mask_at(mask, mdtype, resp, rdtype, i, j, width);
+            if (m == 0.f) continue;
+            const int64_t e = i * width + j;
+            const Token t = token_terms<false>(0.f, old ? old[e] : 0.f, old != nullptr, ref ? ref[e] : 0.f, adv[e], p);
+            acc[S_PG] += t.pg * m;
+            acc[S_CLIP] += t.clipped * m;
+            acc[S_PPOKL] += t.neg_logr * m;
+            acc[S_KL] += t.kl * m;
+            acc[S_MASK] += m;
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < 6; ++q) {
+        const double s = block_sum((double)acc[q], lds);
+        if (threadIdx.x == 0) row_sums[i * S_N + q] = (float)s;
+    }
+    if (threadIdx.x == 0) {
+        row_sums[i * S_N + 6] = 0.f;
+        row_sums[i * S_N + 7] = 0.f;
+    }
+}
+
 int check_args(const char* fn, const float* lp, const float* ref, const float* adv, const void* mask, int mask_dtype,
                const void* lens, int length_dtype, int64_t batch, int64_t width, int kl_penalty, int seq_mean) {
     MRL_REQUIRE(batch >= 0 && width >= 0, MRL_ERR_INVALID_ARG, "%s: batch=%lld width=%lld", fn, (long long)batch,
@@ -293,5 +321,80 @@ extern "C" int mrl_policy_loss_bwd(const float* log_prob, const float* old_log_p
     hipLaunchKernelGGL(policy_loss_bwd_kernel, dim3(blocks), dim3(kBlock), 0, mrl::as_stream(stream), log_prob,
                        old_log_prob, ref_log_prob, advantages, mask, mask_dtype, response_length, length_dtype, batch,
                        width, p, row_sums, out, upstream, g_log_prob, g_entropy);
+    return mrl::check_launch(fn);
+}
+
+extern "C" int mrl_fused_loss_prepare(int layout, int64_t batch, int64_t width, int64_t n_rows, const int32_t* seqlens,
+                                      const int32_t* cu_seqlens_padded, int64_t padded_seq_len,
+                                      const void* prompt_length, int prompt_dtype, const void* response_length,
+                                      int response_dtype, const float* old_log_prob, const float* ref_log_prob,
+                                      const float* advantages, const void* mask, int mask_dtype, int seq_mean,
+                                      int64_t* row_start, int32_t* row_count, float* seq_mask_sum, float* row_ops,
+                                      void* stream) {
+    const char* fn = "mrl_fused_loss_prepare";
+    MRL_REQUIRE(layout == 0 || layout == 1, MRL_ERR_INVALID_ARG, "%s: layout=%d (0 packed, 1 padded)", fn, layout);
+    MRL_REQUIRE(batch >= 0 && batch <= (1LL << 20) && width >= 0 && n_rows >= 0, MRL_ERR_INVALID_ARG,
+                "%s: batch=%lld width=%lld n_rows=%lld", fn, (long long)batch, (long long)width, (long long)n_rows);
+    MRL_REQUIRE((n_rows + kBlock - 1) / kBlock <= 0x7fffffffLL, MRL_ERR_UNSUPPORTED, "%s: n_rows exceeds the grid limit",
+                fn);
+    MRL_REQUIRE(seq_mean == 0 || seq_mean == 1, MRL_ERR_INVALID_ARG, "%s: seq_mean=%d", fn, seq_mean);
+    MRL_REQUIRE(mask == nullptr || mrl::mask_dtype_bytes(mask_dtype) != 0, MRL_ERR_UNSUPPORTED, "%s: mask dtype %d", fn,
+                mask_dtype);
+    MRL_REQUIRE(prompt_length == nullptr || mrl::int_dtype_bytes(prompt_dtype) != 0, MRL_ERR_UNSUPPORTED,
+                "%s: prompt_length dtype %d (want I32 or I64)", fn, prompt_dtype);
+    MRL_REQUIRE(response_length == nullptr || mrl::int_dtype_bytes(response_dtype) != 0, MRL_ERR_UNSUPPORTED,
+                "%s: response_length dtype %d (want I32 or I64)", fn, response_dtype);
+    MRL_REQUIRE(n_rows == 0 || row_ops != nullptr, MRL_ERR_INVALID_ARG, "%s: row_ops is NULL", fn);
+    if (batch > 0) {
+        MRL_REQUIRE(row_start && row_count && seq_mask_sum && advantages, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+        MRL_REQUIRE(mask != nullptr || response_length != nullptr, MRL_ERR_INVALID_ARG,
+                    "%s: need a mask or response lengths", fn);
+        if (layout == 0) {
+            MRL_REQUIRE(seqlens && cu_seqlens_padded, MRL_ERR_INVALID_ARG, "%s: packed layout needs seqlens and cu", fn);
+        } else {
+            MRL_REQUIRE(prompt_length && response_length && padded_seq_len >= 0, MRL_ERR_INVALID_ARG,
+                        "%s: padded layout needs prompt_length, response_length and the padded length", fn);
+        }
+    }
+    hipStream_t s = mrl::as_stream(stream);
+    if (batch > 0) {
+        hipLaunchKernelGGL(fused_seq_kernel, dim3((unsigned)batch), dim3(kBlock), 0, s, layout, width, seqlens,
+                           cu_seqlens_padded, padded_seq_len, prompt_length, prompt_dtype, response_length,
+                           response_dtype, mask, mask_dtype, row_start, row_count, seq_mask_sum);
+        int rc = mrl::check_launch(fn);
+        if (rc != MRL_OK) return rc;
+    }
+    if (n_rows > 0) {
+        hipLaunchKernelGGL(fused_row_ops_kernel, dim3((unsigned)((n_rows + kBlock - 1) / kBlock)), dim3(kBlock), 0, s,
+                           batch, width, n_rows, (const int64_t*)row_start, (const int32_t*)row_count,
+                           (const float*)seq_mask_sum, old_log_prob, ref_log_prob, advantages, mask, mask_dtype,
+                           response_length, response_dtype, seq_mean, row_ops);
+        return mrl::check_launch(fn);
+    }
+    return MRL_OK;
+}
+
+extern "C" int mrl_fused_loss_reduce(const float* row_terms, const int64_t* row_start, const int32_t* row_count,
+                                     int64_t batch, int64_t width, const float* old_log_prob,
+                                     const float* ref_log_prob, const float* advantages, const void* mask,
+                                     int mask_dtype, const void* response_length, int response_dtype, float clip_lo,
+                                     float clip_hi, int kl_penalty, float kl_coef, float entropy_coeff, int seq_mean,
+                                     float loss_scale, float* row_sums, float* out, void* stream) {
+    const char* fn = "mrl_fused_loss_reduce";
+    int rc = check_args(fn, (const float*)row_terms, ref_log_prob, advantages, mask, mask_dtype, response_length,
+                        response_dtype, batch, width, kl_penalty, seq_mean);
+    if (rc != MRL_OK) return rc;
+    MRL_REQUIRE(out != nullptr && (batch == 0 || (row_sums && row_start && row_count)), MRL_ERR_INVALID_ARG,
+                "%s: NULL pointer", fn);
+    const Params p = {clip_lo, clip_hi, kl_coef, entropy_coeff, loss_scale, kl_penalty, seq_mean};
+    hipStream_t s = mrl::as_stream(stream);
+    if (batch > 0) {
+        hipLaunchKernelGGL(fused_seq_reduce_kernel, dim3((unsigned)batch), dim3(kBlock), 0, s, row_terms, row_start,
+                           row_count, width, old_log_prob, ref_log_prob, advantages, mask, mask_dtype, response_length,
+                           response_dtype, p, row_sums);
+        rc = mrl::check_launch(fn);
+        if (rc != MRL_OK) return rc;
+    }
+    hipLaunchKernelGGL(policy_loss_finalize_kernel, dim3(1), dim3(kBlock), 0, s, (const float*)row_sums, batch, p, out);
     return mrl::check_launch(fn);
 }

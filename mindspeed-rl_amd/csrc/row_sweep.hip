@@ -1,0 +1,440 @@
+// Row-in-registers vocabulary sweeps for gfx950.
+//
+// One workgroup of 1024 threads (16 wavefronts, one workgroup per CU) owns one logits row and
+// keeps ALL of it in registers: up to 19 16-byte vectors per thread = 311 296 bytes, enough for a
+// 152 064-entry bf16 row.  The row is loaded once (every load issued before the first use), the
+// softmax statistics and the token's loss gradient are computed from registers, and dlogits are
+// written from the same registers - one HBM read and one HBM write per element for the whole
+// forward + backward of the log-prob / policy-loss path.  Reads and writes of a workgroup are
+// separated in time, which is also the access pattern that the HBM system serves best for a
+// read+write stream.
+//
+// Two kernels share the skeleton:
+//   fused_sweep_kernel   forward statistics + policy-loss gradient + dlogits (eager gradient)
+//   bwd_regs_kernel      dlogits from a saved logsumexp (the autograd backward of the split path)
+#include "mrl_internal.h"
+#include "policy_terms.h"
+#include "row_sweep.h"
+#include "vocab_common.h"
+
+namespace {
+
+using namespace mrl_vocab;
+using namespace mrl_loss;
+
+constexpr int kBlock = 1024;
+constexpr int kWaves = kBlock / 64;
+
+// Two-level reduction for 16 wavefronts: shuffles inside each wavefront, then the first
+// wavefront combines the 16 partials with shuffles again (a serial combine by every thread
+// would cost more ALU time than a sixth of the row).
+template <bool kEntropy>
+__device__ __forceinline__ Stats block_reduce_1024(Stats st, float k, Stats* lds) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        Stats o;
+        o.m = __shfl_xor(st.m, off, 64);
+        o.s = __shfl_xor(st.s, off, 64);
+        o.u = kEntropy ? __shfl_xor(st.u, off, 64) : 0.f;
+        st = merge<kEntropy>(st, o, k);
+    }
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) lds[wave] = st;
+    __syncthreads();
+    if (wave == 0) {
+        Stats x = lds[lane & (kWaves - 1)];
+#pragma unroll
+        for (int off = kWaves / 2; off >= 1; off >>= 1) {
+            Stats o;
+            o.m = __shfl_xor(x.m, off, 64);
+            o.s = __shfl_xor(x.s, off, 64);
+            o.u = kEntropy ? __shfl_xor(x.u, off, 64) : 0.f;
+            x = merge<kEntropy>(x, o, k);
+        }
+        if (lane == 0) lds[kWaves] = x;
+    }
+    __syncthreads();
+    return lds[kWaves];
+}
+
+__device__ __forceinline__ int64_t load_label(const void* labels, int dtype, int64_t r) {
+    return dtype == MRL_I32 ? (int64_t) reinterpret_cast<const int32_t*>(labels)[r]
+                            : reinterpret_cast<const int64_t*>(labels)[r];
+}
+
+struct RowGrad {
+    float k;        // inv_t * log2(e)
+    float lse2;     // lse * log2(e)
+    float c0, c1;   // dlogit = 2^(z k - lse2) * (c0 + c1 z)
+    float onehot;   // added at the label
+};
+
+template <bool kEntropy>
+__device__ __forceinline__ float grad_elem(const RowGrad& g, float z) {
+    const float e = fast_exp2(__builtin_fmaf(z, g.k, -g.lse2));
+    const float w = kEntropy ? __builtin_fmaf(g.c1, z, g.c0) : g.c0;
+    return e * w;
+}
+
+// Writes dlogits for the vectors this thread holds.
+template <int DT, int NV, bool kEntropy>
+__device__ __forceinline__ void store_grads(const u32x4 (&v)[NV], int n_vec, const RowGrad& g, int y_vec, int y_lane,
+                                            u32x4* __restrict__ ovec) {
+    using E = Elem<DT>;
+    constexpr int kVec = E::kVec;
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int q = 0; q < NV; ++q) {
+        const int idx = q * kBlock + tid;
+        if (idx < n_vec) {
+            float z[kVec], d[kVec];
+            E::unpack(v[q], z);
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) d[i] = grad_elem<kEntropy>(g, z[i]);
+            if (idx == y_vec) {
+#pragma unroll
+                for (int i = 0; i < kVec; ++i)
+                    if (i == y_lane) d[i] += g.onehot;
+            }
+            __builtin_nontemporal_store(E::pack(d), ovec + idx);
+        }
+    }
+}
+
+__device__ __forceinline__ void zero_row(u32x4* __restrict__ ovec, int n_vec) {
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    for (int idx = threadIdx.x; idx < n_vec; idx += kBlock) __builtin_nontemporal_store(zero, ovec + idx);
+}
+
+template <int DT, int NV, bool kEntropy>
+__global__ __launch_bounds__(kBlock) void fused_sweep_kernel(
+    const typename Elem<DT>::T* logits, int64_t row_stride, int vocab, const void* __restrict__ labels,
+    int labels_dtype, float inv_t, const float* __restrict__ row_ops, int has_old, Params p, float grad_scale,
+    typename Elem<DT>::T* dlogits, int64_t d_stride, float* __restrict__ logp, float* __restrict__ entropy,
+    float* __restrict__ row_terms) {
+    using E = Elem<DT>;
+    using T = typename E::T;
+    constexpr int kVec = E::kVec;
+    __shared__ Stats lds[kWaves + 1];
+
+    const int64_t r = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int n_vec = vocab / kVec;
+    const T* row = logits + r * row_stride;
+    u32x4* ovec = reinterpret_cast<u32x4*>(dlogits + r * d_stride);
+    const u32x4* ivec = reinterpret_cast<const u32x4*>(row);
+
+    const float* ops = row_ops + r * MRL_ROW_OPS;
+    const float m = ops[MRL_OP_MASK];
+    if (m == 0.f) {                       // not a response token: no gradient, nothing to read
+        zero_row(ovec, n_vec);
+        if (tid == 0) {
+            if (logp) logp[r] = 0.f;
+            if (entropy) entropy[r] = 0.f;
+#pragma unroll
+            for (int q = 0; q < S_N; ++q) row_terms[r * S_N + q] = 0.f;
+        }
+        return;
+    }
+
+    // the whole row: every load is in flight before the first use
+    u32x4 v[NV];
+#pragma unroll
+    for (int q = 0; q < NV; ++q) {
+        const int idx = q * kBlock + tid;
+        if (idx < n_vec) v[q] = __builtin_nontemporal_load(ivec + idx);
+    }
+    const int64_t y = load_label(labels, labels_dtype, r);
+    const bool y_ok = (y >= 0) && (y < (int64_t)vocab);
+    const float z_y = y_ok ? E::load(row + y) : 0.f;
+    const float old_lp = ops[MRL_OP_OLD], ref_lp = ops[MRL_OP_REF], adv = ops[MRL_OP_ADV];
+    const float w_pg = ops[MRL_OP_WPG], inv_tok = ops[MRL_OP_INVTOK];
+
+    const float k = inv_t * kLog2e;
+    Stats st = {kMaxInit, 0.f, 0.f};
+#pragma unroll
+    for (int q = 0; q < NV; ++q) {
+        const int idx = q * kBlock + tid;
+        if (idx < n_vec) {
+            float z[kVec];
+            E::unpack(v[q], z);
+            float vmax = st.m;
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) vmax = fmaxf(vmax, z[i]);
+            grow_max<kEntropy>(st, vmax, k);
+            const float mk = st.m * k;
+#pragma unroll
+            for (int i = 0; i < kVec; ++i) add_one<kEntropy>(st, z[i], k, mk);
+        }
+    }
+    const Stats tot = block_reduce_1024<kEntropy>(st, k, lds);
+
+    // row scalars, computed redundantly by every thread (uniform values)
+    const float lse = (tot.m * k + fast_log2(tot.s)) * kLn2;
+    const float lp = (y_ok ? z_y * inv_t : tot.m * inv_t) - lse;
+    const float ent = kEntropy ? lse - (tot.u / tot.s) * inv_t : 0.f;
+    const Token t = token_terms<true>(lp, old_lp, has_old != 0, ref_lp, adv, p);
+    const float g_lp = grad_scale * m * (w_pg * t.d_pg + p.kl_coef * inv_tok * t.d_kl);
+    const float g_h = kEntropy ? grad_scale * m * (-p.entropy_coeff * inv_tok) : 0.f;
+
+    if (g_lp == 0.f && g_h == 0.f) {
+        zero_row(ovec, n_vec);
+    } else {
+        RowGrad g;
+        g.k = k;
+        g.lse2 = lse * kLog2e;
+        g.c0 = kEntropy ? inv_t * (-g_lp + g_h * (lse - ent)) : -g_lp * inv_t;
+        g.c1 = kEntropy ? -g_h * inv_t * inv_t : 0.f;
+        g.onehot = g_lp * inv_t;
+        store_grads<DT, NV, kEntropy>(v, n_vec, g, y_ok ? (int)(y / kVec) : -1, y_ok ? (int)(y % kVec) : 0, ovec);
+    }
+    if (tid == 0) {
+        if (logp) logp[r] = lp;
+        if (entropy) entropy[r] = ent;
+        float* out = row_terms + r * S_N;
+        out[S_PG] = t.pg * m;
+        out[S_CLIP] = t.clipped * m;
+        out[S_PPOKL] = t.neg_logr * m;
+        out[S_KL] = t.kl * m;
+        out[S_ENT] = ent * m;
+        out[S_MASK] = m;
+        out[6] = 0.f;
+        out[7] = 0.f;
+    }
+}
+
+template <int DT, int NV, bool kEntropy>
+__global__ __launch_bounds__(kBlock) void bwd_regs_kernel(
+    const typename Elem<DT>::T* logits, int64_t row_stride, int vocab, const void* __restrict__ labels,
+    int labels_dtype, float inv_t, const float* __restrict__ lse_in, const float* __restrict__ ent_in,
+    const float* __restrict__ g_logp, const float* __restrict__ g_entropy, typename Elem<DT>::T* dlogits,
+    int64_t d_stride) {
+    using E = Elem<DT>;
+    using T = typename E::T;
+    constexpr int kVec = E::kVec;
+    const int64_t r = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int n_vec = vocab / kVec;
+    const T* row = logits + r * row_stride;
+    u32x4* ovec = reinterpret_cast<u32x4*>(dlogits + r * d_stride);
+    const u32x4* ivec = reinterpret_cast<const u32x4*>(row);
+
+    const float g_lp = g_logp ? g_logp[r] : 0.f;
+    const float g_h = (kEntropy && g_entropy) ? g_entropy[r] : 0.f;
+    if (g_lp == 0.f && g_h == 0.f) {
+        zero_row(ovec, n_vec);
+        return;
+    }
+    u32x4 v[NV];
+#pragma unroll
+    for (int q = 0; q < NV; ++q) {
+        const int idx = q * kBlock + tid;
+        if (idx < n_vec) v[q] = __builtin_nontemporal_load(ivec + idx);
+    }
+    const float lse = lse_in[r];
+    RowGrad g;
+    g.k = inv_t * kLog2e;
+    g.lse2 = lse * kLog2e;
+    g.c0 = kEntropy ? inv_t * (-g_lp + g_h * (lse - ent_in[r])) : -g_lp * inv_t;
+    g.c1 = kEntropy ? -g_h * inv_t * inv_t : 0.f;
+    g.onehot = g_lp * inv_t;
+    const int64_t y = load_label(labels, labels_dtype, r);
+    const bool y_ok = (y >= 0) && (y < (int64_t)vocab);
+    store_grads<DT, NV, kEntropy>(v, n_vec, g, y_ok ? (int)(y / kVec) : -1, y_ok ? (int)(y % kVec) : 0, ovec);
+}
+
+// Conditional in-place rescale: multiplies every row by upstream/assumed unless that ratio is 1.
+template <int DT>
+__global__ __launch_bounds__(256) void scale_rows_kernel(typename Elem<DT>::T* x, int64_t row_stride, int vocab,
+                                                         const float* __restrict__ upstream, float assumed) {
+    using E = Elem<DT>;
+    constexpr int kVec = E::kVec;
+    const float ratio = *upstream / assumed;
+    if (ratio == 1.f) return;
+    u32x4* vec = reinterpret_cast<u32x4*>(x + (int64_t)blockIdx.x * row_stride);
+    const int n_vec = vocab / kVec;
+    for (int idx = threadIdx.x; idx < n_vec; idx += 256) {
+        float z[kVec];
+        E::unpack(vec[idx], z);
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) z[i] *= ratio;
+        vec[idx] = E::pack(z);
+    }
+}
+
+// ----------------------------------------------------------------------------- host dispatch
+constexpr int kMaxVecPerThread = 19;
+
+inline int pick_nv(int64_t n_vec) {
+    const int64_t need = (n_vec + kBlock - 1) / kBlock;
+    const int sizes[] = {4, 8, 12, 16, 19};
+    for (int s : sizes)
+        if (need <= s) return s;
+    return 0;
+}
+
+template <int DT, int NV>
+int launch_fused(const mrl::FusedArgs& a) {
+    using T = typename Elem<DT>::T;
+    const dim3 grid((unsigned)a.n_rows), block(kBlock);
+    const Params p = {a.clip_lo, a.clip_hi, a.kl_coef, a.entropy_coeff, 1.f, a.kl_penalty, 0};
+#define MRL_FUSED_LAUNCH(ENT)                                                                                  \
+    hipLaunchKernelGGL((fused_sweep_kernel<DT, NV, ENT>), grid, block, 0, a.stream, (const T*)a.logits,        \
+                       a.row_stride, (int)a.vocab, a.labels, a.labels_dtype, a.inv_t, a.row_ops, a.has_old, p, \
+                       a.grad_scale, (T*)a.dlogits, a.d_stride, a.logp, a.entropy, a.row_terms)
+    if (a.with_entropy) MRL_FUSED_LAUNCH(true);
+    else MRL_FUSED_LAUNCH(false);
+#undef MRL_FUSED_LAUNCH
+    return mrl::check_launch("mrl_fused_logprob_loss");
+}
+
+template <int DT, int NV>
+int launch_bwd_regs(const mrl::BwdRegsArgs& a) {
+    using T = typename Elem<DT>::T;
+    const dim3 grid((unsigned)a.n_rows), block(kBlock);
+#define MRL_BWDR_LAUNCH(ENT)                                                                              \
+    hipLaunchKernelGGL((bwd_regs_kernel<DT, NV, ENT>), grid, block, 0, a.stream, (const T*)a.logits,      \
+                       a.row_stride, (int)a.vocab, a.labels, a.labels_dtype, a.inv_t, a.lse, a.entropy,   \
+                       a.g_logp, a.g_entropy, (T*)a.dlogits, a.d_stride)
+    if (a.g_entropy) MRL_BWDR_LAUNCH(true);
+    else MRL_BWDR_LAUNCH(false);
+#undef MRL_BWDR_LAUNCH
+    return mrl::check_launch("mrl_vocab_logprob_bwd");
+}
+
+#define MRL_NV_SWITCH(FUNC, DT, nv, a)      \
+    switch (nv) {                           \
+        case 4: return FUNC<DT, 4>(a);      \
+        case 8: return FUNC<DT, 8>(a);      \
+        case 12: return FUNC<DT, 12>(a);    \
+        case 16: return FUNC<DT, 16>(a);    \
+        default: return FUNC<DT, 19>(a);    \
+    }
+
+template <int DT>
+int fused_by_nv(int nv, const mrl::FusedArgs& a) { MRL_NV_SWITCH(launch_fused, DT, nv, a) }
+// the 8-vector instantiation of the backward kernel is left out: the compiler spills it heavily
+// for fp32, and 12 vectors per thread cost nothing extra (unused slots are predicated off)
+template <int DT>
+int bwd_by_nv(int nv, const mrl::BwdRegsArgs& a) {
+    switch (nv) {
+        case 4: return launch_bwd_regs<DT, 4>(a);
+        case 8:
+        case 12: return launch_bwd_regs<DT, 12>(a);
+        case 16: return launch_bwd_regs<DT, 16>(a);
+        default: return launch_bwd_regs<DT, 19>(a);
+    }
+}
+
+}  // namespace
+
+namespace mrl {
+
+bool row_sweep_supported(int dtype, int64_t vocab, const void* in, int64_t in_stride, const void* out,
+                         int64_t out_stride, int64_t n_rows) {
+    const int eb = float_dtype_bytes(dtype);
+    if (eb == 0) return false;
+    const int64_t per_vec = 16 / eb;
+    if (vocab % per_vec != 0) return false;
+    if (pick_nv(vocab / per_vec) == 0) return false;
+    if (!aligned(in, 16) || !aligned(out, 16)) return false;
+    if (n_rows > 1 && ((in_stride * eb) % 16 != 0 || (out_stride * eb) % 16 != 0)) return false;
+    return true;
+}
+
+int bwd_regs_launch(const BwdRegsArgs& a) {
+    const int nv = pick_nv(a.vocab / (16 / float_dtype_bytes(a.dtype)));
+    switch (a.dtype) {
+        case MRL_F32: return bwd_by_nv<MRL_F32>(nv, a);
+        case MRL_BF16: return bwd_by_nv<MRL_BF16>(nv, a);
+        default: return bwd_by_nv<MRL_F16>(nv, a);
+    }
+}
+
+}  // namespace mrl
+
+extern "C" int64_t mrl_fused_max_vocab(int logits_dtype) {
+    const int eb = mrl::float_dtype_bytes(logits_dtype);
+    if (eb == 0) return 0;
+    return (int64_t)kMaxVecPerThread * kBlock * (16 / eb);
+}
+
+extern "C" int mrl_fused_logprob_loss(const void* logits, int logits_dtype, int64_t n_rows, int64_t vocab,
+                                      int64_t row_stride, const void* labels, int labels_dtype,
+                                      float inv_temperature, const float* row_ops, int has_old, float clip_lo,
+                                      float clip_hi, int kl_penalty, float kl_coef, float entropy_coeff,
+                                      float grad_scale, void* dlogits, int64_t dlogits_row_stride, float* logp,
+                                      float* entropy, float* row_terms, void* stream) {
+    const char* fn = "mrl_fused_logprob_loss";
+    MRL_REQUIRE(n_rows >= 0 && vocab > 0 && n_rows <= 0x7fffffffLL, MRL_ERR_INVALID_ARG, "%s: n_rows=%lld vocab=%lld",
+                fn, (long long)n_rows, (long long)vocab);
+    const int eb = mrl::float_dtype_bytes(logits_dtype);
+    MRL_REQUIRE(eb != 0, MRL_ERR_UNSUPPORTED, "%s: logits dtype %d (want F32, BF16 or F16)", fn, logits_dtype);
+    MRL_REQUIRE(mrl::int_dtype_bytes(labels_dtype) != 0, MRL_ERR_UNSUPPORTED, "%s: labels dtype %d (want I32 or I64)",
+                fn, labels_dtype);
+    MRL_REQUIRE(row_stride >= vocab && dlogits_row_stride >= vocab, MRL_ERR_INVALID_ARG, "%s: row stride below vocab",
+                fn);
+    MRL_REQUIRE(kl_penalty >= MRL_KL_NONE && kl_penalty <= MRL_KL_LOW_VAR, MRL_ERR_INVALID_ARG, "%s: kl_penalty=%d", fn,
+                kl_penalty);
+    MRL_REQUIRE(inv_temperature > 0.f && inv_temperature < 1.0e6f, MRL_ERR_INVALID_ARG,
+                "%s: inv_temperature=%g must be in (0, 1e6)", fn, (double)inv_temperature);
+    if (n_rows == 0) return MRL_OK;
+    MRL_REQUIRE(logits && labels && row_ops && dlogits && row_terms, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+    MRL_REQUIRE(mrl::row_sweep_supported(logits_dtype, vocab, logits, row_stride, dlogits, dlogits_row_stride, n_rows),
+                MRL_ERR_UNSUPPORTED,
+                "%s: needs 16-byte aligned rows, vocab %% %d == 0 and vocab <= %lld for this dtype (got vocab=%lld)", fn,
+                16 / eb, (long long)mrl_fused_max_vocab(logits_dtype), (long long)vocab);
+    if (dlogits != logits) {
+        const char* x = (const char*)logits;
+        const char* y = (const char*)dlogits;
+        const int64_t xb = ((n_rows - 1) * row_stride + vocab) * eb, yb = ((n_rows - 1) * dlogits_row_stride + vocab) * eb;
+        MRL_REQUIRE(x + xb <= y || y + yb <= x, MRL_ERR_INVALID_ARG, "%s: dlogits partially overlaps logits", fn);
+    } else {
+        MRL_REQUIRE(dlogits_row_stride == row_stride, MRL_ERR_INVALID_ARG, "%s: in-place needs identical strides", fn);
+    }
+    mrl::FusedArgs a;
+    a.logits = logits; a.dtype = logits_dtype; a.n_rows = n_rows; a.vocab = vocab; a.row_stride = row_stride;
+    a.labels = labels; a.labels_dtype = labels_dtype; a.inv_t = inv_temperature; a.row_ops = row_ops;
+    a.has_old = has_old; a.clip_lo = clip_lo; a.clip_hi = clip_hi; a.kl_penalty = kl_penalty; a.kl_coef = kl_coef;
+    a.entropy_coeff = entropy_coeff; a.grad_scale = grad_scale; a.dlogits = dlogits; a.d_stride = dlogits_row_stride;
+    a.logp = logp; a.entropy = entropy; a.row_terms = row_terms; a.with_entropy = (entropy != nullptr);
+    a.stream = mrl::as_stream(stream);
+    const int nv = pick_nv(vocab / (16 / eb));
+    switch (logits_dtype) {
+        case MRL_F32: return fused_by_nv<MRL_F32>(nv, a);
+        case MRL_BF16: return fused_by_nv<MRL_BF16>(nv, a);
+        default: return fused_by_nv<MRL_F16>(nv, a);
+    }
+}
+
+extern "C" int mrl_scale_rows(void* x, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                              const float* upstream, float assumed, void* stream) {
+    const char* fn = "mrl_scale_rows";
+    const int eb = mrl::float_dtype_bytes(dtype);
+    MRL_REQUIRE(eb != 0, MRL_ERR_UNSUPPORTED, "%s: dtype %d (want F32, BF16 or F16)", fn, dtype);
+    MRL_REQUIRE(n_rows >= 0 && n_rows <= 0x7fffffffLL && vocab > 0 && row_stride >= vocab, MRL_ERR_INVALID_ARG,
+                "%s: n_rows=%lld vocab=%lld row_stride=%lld", fn, (long long)n_rows, (long long)vocab,
+                (long long)row_stride);
+    MRL_REQUIRE(assumed != 0.f, MRL_ERR_INVALID_ARG, "%s: assumed scale is zero", fn);
+    if (n_rows == 0) return MRL_OK;
+    MRL_REQUIRE(x && upstream, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+    MRL_REQUIRE(vocab % (16 / eb) == 0 && mrl::aligned(x, 16) && (n_rows == 1 || (row_stride * eb) % 16 == 0),
+                MRL_ERR_UNSUPPORTED, "%s: needs 16-byte aligned rows", fn);
+    hipStream_t s = mrl::as_stream(stream);
+    const dim3 grid((unsigned)n_rows), block(256);
+    switch (dtype) {
+        case MRL_F32:
+            hipLaunchKernelGGL(scale_rows_kernel<MRL_F32>, grid, block, 0, s, (float*)x, row_stride, (int)vocab,
+                               upstream, assumed);
+            break;
+        case MRL_BF16:
+            hipLaunchKernelGGL(scale_rows_kernel<MRL_BF16>, grid, block, 0, s, (uint16_t*)x, row_stride, (int)vocab,
+                               upstream, assumed);
+            break;
+        default:
+            hipLaunchKernelGGL(scale_rows_kernel<MRL_F16>, grid, block, 0, s, (uint16_t*)x, row_stride, (int)vocab,
+                               upstream, assumed);
+            break;
+    }
+    return mrl::check_launch(fn);
+}

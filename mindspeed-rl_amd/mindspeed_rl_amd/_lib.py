@@ -45,8 +45,17 @@ SIGNATURES = {
                             _int, _f32, _vp, _vp, _vp],
     "mrl_policy_loss_bwd": [_vp, _vp, _vp, _vp, _vp, _int, _vp, _int, _i64, _i64, _f32, _f32, _int, _f32, _f32, _int,
                             _f32, _vp, _vp, _vp, _vp, _vp, _vp],
+    "mrl_fused_max_vocab": [_int],
+    "mrl_fused_loss_prepare": [_int, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _int, _vp, _int, _vp, _vp, _vp, _vp, _int,
+                               _int, _vp, _vp, _vp, _vp, _vp],
+    "mrl_fused_logprob_loss": [_vp, _int, _i64, _i64, _i64, _vp, _int, _f32, _vp, _int, _f32, _f32, _int, _f32, _f32,
+                               _f32, _vp, _i64, _vp, _vp, _vp, _vp],
+    "mrl_fused_loss_reduce": [_vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _int, _vp, _int, _f32, _f32, _int, _f32,
+                              _f32, _int, _f32, _vp, _vp, _vp],
+    "mrl_scale_rows": [_vp, _int, _i64, _i64, _i64, _vp, _f32, _vp],
     "mrl_copy_bytes": [_vp, _vp, _i64, _vp],
 }
+_RESTYPES = {"mrl_last_error": ctypes.c_char_p, "mrl_fused_max_vocab": ctypes.c_int64}
 
 _lib = None
 
@@ -77,7 +86,7 @@ def load():
     for name, argtypes in SIGNATURES.items():
         fn = getattr(lib, name)       # AttributeError if the library lacks a declared symbol
         fn.argtypes = argtypes
-        fn.restype = ctypes.c_char_p if name == "mrl_last_error" else ctypes.c_int
+        fn.restype = _RESTYPES.get(name, ctypes.c_int)
     _lib = lib
     return lib
 

@@ -8,12 +8,13 @@ text-only log-prob strategy (``logprob_computer.py:73-145``), ``GRPOActorLossFun
 signatures, keyword arguments, return values and error behaviour are the reference's; the work
 is done by the HIP kernels of libmrl_hip.so.
 """
+import os
 from abc import ABC, abstractmethod
 from typing import Dict, Tuple
 
 import torch
 
-from . import _lib
+from . import _lib, vocab_ops
 from .packing import (generate_mask, postprocess_packed_seqs, response_window, truncate_middle_and_pad,
                       truncate_prompt_and_pad)
 from .vocab_ops import compute_log_probs, vocab_logprob_entropy, vocab_parallel_entropy
@@ -134,6 +135,140 @@ def policy_loss(log_prob, entropy, old_log_prob, ref_log_prob, advantages, mask=
                kl_coef=float(kl_coef), entropy_coeff=float(entropy_coeff), seq_mean=0 if token_level_loss else 1,
                loss_scale=float(loss_scale))
     return _PolicyLoss.apply(log_prob, entropy, old_log_prob, ref_log_prob, advantages, mask_t, lens_t, cfg)
+
+
+# ------------------------------------------------------------------------------------ fused sweep
+def fused_supported(output):
+    """True if the row-in-registers kernel can take these logits: a floating dtype it knows,
+    16-byte aligned dense rows and a vocabulary that fits the register file."""
+    if output.dtype not in (torch.float32, torch.bfloat16, torch.float16) or not output.is_cuda:
+        return False
+    vocab = output.shape[-1]
+    per_vec = 16 // output.element_size()
+    if vocab % per_vec != 0 or vocab > _lib.load().mrl_fused_max_vocab(_lib.dtype_code(output)):
+        return False
+    return output.is_contiguous() and output.data_ptr() % 16 == 0
+
+
+class _FusedLogprobLoss(torch.autograd.Function):
+    """logits -> (loss, out[8]) with dlogits produced in the same sweep (one read, one write of
+    the [T, V] tensor for forward + backward).  The backward only rescales the stored dlogits if
+    the upstream gradient differs from the scale assumed in the forward."""
+
+    @staticmethod
+    def forward(ctx, output, labels, batch, cfg):
+        dev = _lib.require_device(output, labels)
+        vocab = output.shape[-1]
+        flat = output.reshape(-1, vocab)
+        n_rows = flat.shape[0]
+        lab = labels.reshape(-1)
+        if lab.dtype not in (torch.int32, torch.int64):
+            lab = lab.to(torch.int64)
+        lab = lab.contiguous()
+        n_seq, width = batch["responses"].shape[0], batch["responses"].shape[-1]
+
+        def f32(t):
+            return None if t is None else t.to(dev).to(torch.float32).contiguous()
+
+        def idx(t):
+            if t is None:
+                return None
+            if t.dtype not in (torch.int32, torch.int64):
+                t = t.to(torch.int64)
+            return t.to(dev).reshape(-1).contiguous()
+
+        old, ref, adv = f32(batch.get("old_log_prob")), f32(cfg["ref_log_prob"]), f32(batch.get("advantages"))
+        mask_t, lens_t = _mask_args(cfg["mask"], batch["response_length"], dev)
+        prompt, resp = idx(batch["prompt_length"]), idx(batch["response_length"])
+        if cfg["packed"]:
+            layout, padded_s = 0, 0
+            seqlens = cfg["seqlens"].to(dev).to(torch.int32).contiguous()
+            cu = cfg["cu"].to(dev).to(torch.int32).contiguous()
+        else:
+            layout, padded_s = 1, output.shape[1]
+            seqlens = cu = None
+        row_start = torch.empty(n_seq, dtype=torch.int64, device=dev)
+        row_count = torch.empty(n_seq, dtype=torch.int32, device=dev)
+        seq_msum = torch.empty(n_seq, dtype=torch.float32, device=dev)
+        row_ops = torch.empty(n_rows * 8, dtype=torch.float32, device=dev)
+        row_terms = torch.empty(n_rows * 8, dtype=torch.float32, device=dev)
+        row_sums = torch.empty(max(n_seq, 1) * 8, dtype=torch.float32, device=dev)
+        out = torch.empty(8, dtype=torch.float32, device=dev)
+        ent = torch.empty(n_rows, dtype=torch.float32, device=dev) if cfg["entropy_coeff"] != 0 else None
+        dlogits = flat if cfg["grad_inplace"] else torch.empty_like(flat)
+        stream = _lib.stream(dev)
+        mdt = _lib.dtype_code(mask_t) if mask_t is not None else _lib.F32
+        pdt = _lib.dtype_code(prompt)
+        rdt = _lib.dtype_code(resp)
+        _lib.call("mrl_fused_loss_prepare", layout, n_seq, width, n_rows, _lib.ptr(seqlens), _lib.ptr(cu), padded_s,
+                  _lib.ptr(prompt), pdt, _lib.ptr(resp), rdt, _lib.ptr(old), _lib.ptr(ref), _lib.ptr(adv),
+                  _lib.ptr(mask_t), mdt, cfg["seq_mean"], _lib.ptr(row_start), _lib.ptr(row_count),
+                  _lib.ptr(seq_msum), _lib.ptr(row_ops), stream)
+        grad_scale = cfg["loss_scale"] * cfg["expected_upstream"]
+        vocab_ops._timed_call("mrl_fused_logprob_loss", n_rows, dev, _lib.ptr(flat), _lib.dtype_code(flat), n_rows,
+                              vocab, vocab, _lib.ptr(lab), _lib.dtype_code(lab), cfg["inv_temperature"],
+                              _lib.ptr(row_ops), 0 if old is None else 1, cfg["clip_lo"], cfg["clip_hi"],
+                              cfg["kl_penalty"], cfg["kl_coef"], cfg["entropy_coeff"], grad_scale, _lib.ptr(dlogits),
+                              vocab, None, _lib.ptr(ent), _lib.ptr(row_terms), stream)
+        _lib.call("mrl_fused_loss_reduce", _lib.ptr(row_terms), _lib.ptr(row_start), _lib.ptr(row_count), n_seq, width,
+                  _lib.ptr(old), _lib.ptr(ref), _lib.ptr(adv), _lib.ptr(mask_t), mdt, _lib.ptr(resp), rdt,
+                  cfg["clip_lo"], cfg["clip_hi"], cfg["kl_penalty"], cfg["kl_coef"], cfg["entropy_coeff"],
+                  cfg["seq_mean"], cfg["loss_scale"], _lib.ptr(row_sums), _lib.ptr(out), stream)
+        ctx.save_for_backward(dlogits)
+        ctx.meta = (tuple(output.shape), cfg["expected_upstream"])
+        ctx.mark_non_differentiable(out)
+        return out[0].clone(), out
+
+    @staticmethod
+    def backward(ctx, g_loss, _g_out):
+        (dlogits,) = ctx.saved_tensors
+        shape, expected = ctx.meta
+        dev = dlogits.device
+        n_rows, vocab = dlogits.shape
+        upstream = g_loss.to(torch.float32).reshape(1).contiguous()
+        _lib.call("mrl_scale_rows", _lib.ptr(dlogits), _lib.dtype_code(dlogits), n_rows, vocab, vocab,
+                  _lib.ptr(upstream), float(expected), _lib.stream(dev))
+        return dlogits.view(shape), None, None, None
+
+
+def fused_logprob_policy_loss(output, batch, *, packed, seqlens=None, cu_seqlens=None, mask=None, ref_log_prob=None,
+                              clip_low, clip_high, kl_penalty=None, kl_coef=0.0, entropy_coeff=0.0,
+                              token_level_loss=True, loss_scale=1.0, inv_temperature=1.0, grad_inplace=False,
+                              expected_upstream=1.0):
+    """Log-prob, entropy, policy loss AND dlogits in one sweep over the logits.
+
+    ``output`` is the packed ``[1, T, V]`` (``packed=True``, with ``seqlens`` / ``cu_seqlens``) or
+    padded ``[B, S, V]`` logits; ``batch`` holds ``labels, responses, response_length,
+    prompt_length, advantages`` and optionally ``old_log_prob``.  Returns ``(loss, out)`` like
+    :func:`policy_loss`.  ``expected_upstream`` is the scalar the caller will multiply the loss by
+    before ``backward()`` (1 unless known otherwise); any other value is honoured by a rescale."""
+    if kl_penalty is None:
+        kl_code = _lib.KL_NONE
+    elif kl_penalty in _lib.KL_BY_NAME:
+        kl_code = _lib.KL_BY_NAME[kl_penalty]
+    else:
+        raise NotImplementedError
+    cfg = dict(packed=bool(packed), seqlens=seqlens, cu=cu_seqlens, mask=mask, ref_log_prob=ref_log_prob,
+               clip_lo=float(1.0 - clip_low), clip_hi=float(1.0 + clip_high), kl_penalty=kl_code,
+               kl_coef=float(kl_coef), entropy_coeff=float(entropy_coeff), seq_mean=0 if token_level_loss else 1,
+               loss_scale=float(loss_scale), inv_temperature=float(inv_temperature), grad_inplace=bool(grad_inplace),
+               expected_upstream=float(expected_upstream))
+    return _FusedLogprobLoss.apply(output, batch["labels"], batch, cfg)
+
+
+def _use_fused(output, kwargs):
+    """The fused sweep is the default for a training step; ``fused=False`` (or the environment
+    variable MRL_FUSED=0) selects the split forward / backward kernels."""
+    if not kwargs.get("fused", os.environ.get("MRL_FUSED", "1") != "0"):
+        return False
+    return torch.is_grad_enabled() and output.requires_grad and fused_supported(output)
+
+
+def _fused_kwargs(kwargs):
+    return dict(packed=kwargs.get("use_remove_padding", False), seqlens=kwargs.get("seqlens_in_batch"),
+                cu_seqlens=kwargs.get("cu_seqlens_padded"), inv_temperature=float(kwargs.get("inv_temperature", 1.0)),
+                grad_inplace=bool(kwargs.get("grad_inplace", False)),
+                expected_upstream=float(kwargs.get("expected_grad_scale", 1.0)))
 
 
 # ------------------------------------------------------------------------------------ log-prob strategy
@@ -274,6 +409,13 @@ class GRPOActorLossFunc(BaseLossFunc):
         if forward_only:
             log_probs, _ = super().compute_log_probs(output=output, batch=batch, **kwargs)
             return log_probs
+        if _use_fused(output, kwargs):
+            loss, out = fused_logprob_policy_loss(
+                output, batch, ref_log_prob=batch.get("ref_log_prob"), clip_low=self.clip_ratio,
+                clip_high=self.clip_ratio, kl_penalty=self.kl_penalty, kl_coef=self.kl_ctrl.value,
+                entropy_coeff=self.entropy_coeff, token_level_loss=True,
+                loss_scale=_dynamic_scale(batch, forward_only, kwargs), **_fused_kwargs(kwargs))
+            return _finish(loss, out)
         log_probs, entropy = super().compute_log_probs(output=output, batch=batch,
                                                        skip_entropy=(self.entropy_coeff == 0), **kwargs)
         # batch['response_mask'] is ignored here, as in the reference: the mask is j < response_length
@@ -329,12 +471,18 @@ class DAPOActorLossFunc(BaseLossFunc):
         if forward_only:
             log_probs, _ = super().compute_log_probs(output=output, batch=batch, **kwargs)
             return log_probs
-        log_probs, entropy = super().compute_log_probs(output=output, batch=batch,
-                                                       skip_entropy=(self.entropy_coeff == 0), **kwargs)
         if not self.clip_higher_enable:
             self.clip_ratio_low = self.clip_ratio
             self.clip_ratio_high = self.clip_ratio
         mask = batch["response_mask"] if "response_mask" in batch else None
+        if _use_fused(output, kwargs):
+            loss, out = fused_logprob_policy_loss(
+                output, batch, mask=mask, clip_low=self.clip_ratio_low, clip_high=self.clip_ratio_high,
+                kl_penalty=None, entropy_coeff=self.entropy_coeff, token_level_loss=self.token_level_loss,
+                loss_scale=_dynamic_scale(batch, forward_only, kwargs), **_fused_kwargs(kwargs))
+            return _finish(loss, out)
+        log_probs, entropy = super().compute_log_probs(output=output, batch=batch,
+                                                       skip_entropy=(self.entropy_coeff == 0), **kwargs)
         loss, out = policy_loss(log_probs, entropy if self.entropy_coeff != 0 else None, batch.get("old_log_prob"),
                                 None, batch.get("advantages"), mask=mask,
                                 response_length=None if mask is not None else batch["response_length"],

@@ -515,8 +515,9 @@ def _to_dev(d, dev):
     return {k: (v.to(dev) if isinstance(v, torch.Tensor) else v) for k, v in d.items()}
 
 
+@pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("entropy_coeff", [0.0, 0.001])
-def test_grpo_compute_loss_config0_packed(dev, entropy_coeff):
+def test_grpo_compute_loss_config0_packed(dev, entropy_coeff, fused):
     """configs[0]: 4 prompts x G=4, R in [64,256], V=32000 fp32 logits ~N(0,2), eps 0.2, k3 KL 0.001."""
     gen = torch.Generator().manual_seed(0)
     logits, b, kw, rewards, _ = _make_batch(gen, 4, 4, 64, 256, 32000, torch.float32, 2.0, 1, prompt_hi=1)
@@ -530,6 +531,7 @@ def test_grpo_compute_loss_config0_packed(dev, entropy_coeff):
                           "entropy_coeff": entropy_coeff})
     zd = logits.to(dev).requires_grad_()
     bd, kwd = _to_dev(b, dev), _to_dev(kw, dev)
+    kwd["fused"] = fused        # one-sweep eager gradient, or the split forward / backward kernels
     # advantages computed on the device from the rewards agree with the oracle's
     rmask = mrl.generate_mask(bd["responses"], bd["response_length"])
     adv_d, _ = mrl.compute_group_norm_advantage_return(rewards.to(dev), rmask, bd["response_length"], 4)
@@ -561,7 +563,8 @@ def test_grpo_compute_loss_config0_packed(dev, entropy_coeff):
                        **{k: v for k, v in kwd.items() if k != "use_remove_padding"})
 
 
-def test_padded_vs_packed_and_dapo_bf16(dev):
+@pytest.mark.parametrize("fused", [True, False])
+def test_padded_vs_packed_and_dapo_bf16(dev, fused):
     """configs[2]/[4] in small: the same responses as a padded [B,S] batch and packed with
     alignment 8, bf16 logits, an empty-response group, DAPO clip-higher with sequence mean."""
     gen = torch.Generator().manual_seed(2)
@@ -578,6 +581,7 @@ def test_padded_vs_packed_and_dapo_bf16(dev):
     f.add_loss_meta_info({"entropy_coeff": 0.002, "token_level_loss": True, "clip_higher_enable": True,
                           "clip_ratio_low": 0.2, "clip_ratio_high": 0.28, "clip_ratio": 0.2})
     bd, kwd = _to_dev(b, dev), _to_dev(kw, dev)
+    kwd["fused"] = fused
     zo = logits.float().requires_grad_()
     want_loss, want_stats = o_loss.dapo_compute_loss(zo, b, meta, **kw)
     (dz_o,) = torch.autograd.grad(want_loss, zo)
@@ -592,7 +596,7 @@ def test_padded_vs_packed_and_dapo_bf16(dev):
     # padded layout through the same loss object: same loss, same statistics
     bp = dict(bd, labels=labels.to(dev))
     zp = padded.to(dev).requires_grad_()
-    loss_p, stats_p = f.compute_loss(zp, bp)
+    loss_p, stats_p = f.compute_loss(zp, bp, fused=fused)
     assert loss_p.item() == pytest.approx(loss.item(), rel=1e-6)
     for k in stats:
         assert stats_p[k] == pytest.approx(stats[k], rel=1e-6, abs=1e-9)
@@ -607,10 +611,101 @@ def test_padded_vs_packed_and_dapo_bf16(dev):
     rm[:, ::3] = 0
     rm[:, 0] = 1
     b2["response_mask"] = rm
-    want_loss, want_stats = o_loss.dapo_compute_loss(logits.float(), b2, meta, **kw)
+    zo2 = logits.float().requires_grad_()
+    want_loss, want_stats = o_loss.dapo_compute_loss(zo2, b2, meta, **kw)
+    (dz_o2,) = torch.autograd.grad(want_loss, zo2)
     loss, stats = f.compute_loss(zd, _to_dev(b2, dev), **kwd)
     assert abs(loss.item() - want_loss.item()) <= TOL_LOSS_REL * abs(want_loss.item()) + 1e-7
     assert stats["actor/pg_clipfrac"] == 0.0 and stats["actor/kl_loss"] == 0.0
+    (dz2,) = torch.autograd.grad(loss, zd)
+    assert (dz2.float().cpu() - dz_o2).abs().max().item() < TOL_DLOGITS
+    assert (dz2.float().cpu() - dz_o2).abs().max().item() < 1e-2 * dz_o2.abs().max().item()
+
+
+def test_fused_sweep_specifics(dev):
+    """The one-sweep path: agreement with the split kernels, an upstream scale that differs from
+    the expected one (rescale kernel), in-place gradients, tokens whose mask reaches past the
+    logits window, and the automatic fall-back for a vocabulary the registers cannot hold."""
+    gen = torch.Generator().manual_seed(7)
+    logits, b, kw, _, _ = _make_batch(gen, 2, 4, 6, 30, 8192, torch.bfloat16, 3.0, 2, prompt_hi=3)
+    f = mrl.LossFuncFactory.get_instance("ray_grpo", "actor")
+    f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.01), "kl_penalty": "low_var_kl",
+                          "entropy_coeff": 0.003})
+    bd, kwd = _to_dev(b, dev), _to_dev(kw, dev)
+    assert mrl.fused_supported(logits.to(dev))
+    zd = logits.to(dev).requires_grad_()
+    loss_s, stats_s = f.compute_loss(zd, bd, fused=False, **kwd)
+    (dz_s,) = torch.autograd.grad(loss_s, zd)
+    loss_f, stats_f = f.compute_loss(zd, bd, fused=True, **kwd)
+    (dz_f,) = torch.autograd.grad(loss_f, zd)
+    # the two paths sum the row in a different order, and the surrogate is a cancelling sum of +-A*r
+    assert loss_f.item() == pytest.approx(loss_s.item(), rel=5e-5)
+    for k in stats_s:
+        assert stats_f[k] == pytest.approx(stats_s[k], rel=5e-5, abs=1e-8)
+    assert (dz_f.float() - dz_s.float()).abs().max().item() <= 2 ** -8 * dz_s.float().abs().max().item()
+    # upstream 1/16 while 1 was expected: the stored gradient is rescaled; expected 1/16: no rescale needed
+    (dz_16,) = torch.autograd.grad(f.compute_loss(zd, bd, fused=True, **kwd)[0] / 16.0, zd)
+    assert torch.equal(dz_16.float() * 16.0, dz_f.float())
+    (dz_16b,) = torch.autograd.grad(f.compute_loss(zd, bd, fused=True, expected_grad_scale=1 / 16.0, **kwd)[0] / 16.0, zd)
+    assert torch.equal(dz_16b, dz_16)
+    # in place: the gradient lands in the logits buffer
+    z_in = logits.to(dev).requires_grad_()
+    loss_i, _ = f.compute_loss(z_in, bd, fused=True, grad_inplace=True, **kwd)
+    (dz_i,) = torch.autograd.grad(loss_i, z_in)
+    assert dz_i.data_ptr() == z_in.data_ptr() and torch.equal(dz_i, dz_f)
+    # a mask that reaches past the window (response_length larger than what the packed rows hold)
+    b2 = dict(b, response_length=b["response_length"] + 2)
+    width = b["responses"].shape[1]
+    b2["response_length"] = torch.clamp(b2["response_length"], max=width)
+    want, want_stats = o_loss.grpo_compute_loss(logits.float(), b2, dict(clip_ratio=0.2, kl_coef=0.01,
+                                                kl_penalty="low_var_kl", entropy_coeff=0.003), **kw)
+    got, got_stats = f.compute_loss(zd, _to_dev(b2, dev), fused=True, **kwd)
+    assert abs(got.item() - want.item()) <= TOL_LOSS_REL * abs(want.item()) + 1e-7
+    for k in want_stats:
+        assert abs(got_stats[k] - want_stats[k]) <= TOL_LOSS_REL * abs(want_stats[k]) + 1e-6, k
+    # no old_log_prob: ratio 1
+    b3 = {k: v for k, v in b.items() if k != "old_log_prob"}
+    zo = logits.float().requires_grad_()
+    want, _ = o_loss.grpo_compute_loss(zo, b3, dict(clip_ratio=0.2, kl_coef=0.01, kl_penalty="low_var_kl",
+                                                    entropy_coeff=0.003), **kw)
+    (dz_o,) = torch.autograd.grad(want, zo)
+    got, _ = f.compute_loss(zd, _to_dev(b3, dev), fused=True, **kwd)
+    (dz_g,) = torch.autograd.grad(got, zd)
+    assert abs(got.item() - want.item()) <= TOL_LOSS_REL * abs(want.item()) + 1e-7
+    assert (dz_g.float().cpu() - dz_o).abs().max().item() < TOL_DLOGITS
+    # a vocabulary that is not a multiple of the vector width falls back to the split kernels
+    odd = torch.randn(1, logits.shape[1], 1003, generator=gen).to(torch.bfloat16).to(dev).requires_grad_()
+    assert not mrl.fused_supported(odd)
+    bd_odd = dict(bd, labels=bd["labels"] % 1003)
+    loss_o, _ = f.compute_loss(odd, bd_odd, fused=True, **kwd)
+    (dz_odd,) = torch.autograd.grad(loss_o, odd)
+    assert dz_odd.shape == odd.shape and torch.isfinite(loss_o).item()
+    assert _lib.load().mrl_fused_max_vocab(_lib.BF16) == 19 * 1024 * 8
+    assert _lib.load().mrl_fused_max_vocab(_lib.F32) == 19 * 1024 * 4
+
+
+@pytest.mark.parametrize("dtype,vocab", [(torch.bfloat16, 152064), (torch.bfloat16, 129280), (torch.float32, 32000),
+                                         (torch.float16, 65536), (torch.float32, 77824), (torch.bfloat16, 64)])
+def test_fused_sweep_vocab_sizes(dev, dtype, vocab):
+    """Every register-tile size of the fused kernel (4, 8, 12, 16, 19 vectors per thread)."""
+    gen = torch.Generator().manual_seed(vocab)
+    logits, b, kw, _, _ = _make_batch(gen, 1, 4, 3, 9, vocab, dtype, 3.0, 1, prompt_hi=2)
+    meta = dict(clip_ratio=0.2, kl_coef=0.02, kl_penalty="low_var_kl", entropy_coeff=0.002)
+    zo = logits.float().requires_grad_()
+    want, want_stats = o_loss.grpo_compute_loss(zo, b, meta, **kw)
+    (dz_o,) = torch.autograd.grad(want, zo)
+    f = mrl.LossFuncFactory.get_instance("ray_grpo", "actor")
+    f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.02), "kl_penalty": "low_var_kl",
+                          "entropy_coeff": 0.002})
+    zd = logits.to(dev).requires_grad_()
+    assert mrl.fused_supported(zd)
+    got, got_stats = f.compute_loss(zd, _to_dev(b, dev), fused=True, **_to_dev(kw, dev))
+    (dz,) = torch.autograd.grad(got, zd)
+    assert abs(got.item() - want.item()) <= TOL_LOSS_REL * abs(want.item()) + 1e-7
+    for k in want_stats:
+        assert abs(got_stats[k] - want_stats[k]) <= TOL_LOSS_REL * abs(want_stats[k]) + 1e-6, k
+    assert (dz.float().cpu() - dz_o).abs().max().item() < TOL_DLOGITS
+    assert (dz.float().cpu() - dz_o).abs().max().item() <= 2 ** -8 * dz_o.abs().max().item() + 1e-9
 
 
 def test_copy_kernel_moves_bytes(dev):
