@@ -199,8 +199,10 @@ def main():
         step()
     torch.cuda.synchronize()
     vocab_ops.kernel_events = []
+    dz = None
     t0 = time.perf_counter()
     for _ in range(args.steps):
+        del dz                      # the previous gradient is released before the next one is allocated
         loss, stats, dz = step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
@@ -221,8 +223,8 @@ def main():
         "mrl_vocab_logprob_bwd": live_rows * 2 * row_bytes + dead_rows * row_bytes,
         "mrl_fused_logprob_loss": live_rows * 2 * row_bytes + dead_rows * row_bytes,
     }
-    kernel_symbol = {"mrl_vocab_logprob_fwd": "vocab_fwd_kernel", "mrl_vocab_logprob_bwd": "bwd_regs_kernel",
-                     "mrl_fused_logprob_loss": "fused_sweep_kernel"}
+    kernel_symbol = {"mrl_vocab_logprob_fwd": "vocab_fwd_kernel", "mrl_vocab_logprob_bwd": "vocab_bwd_kernel",
+                     "mrl_fused_logprob_loss": "fused_sweep_persistent_kernel"}
     kernels = {}
     for name, nbytes in kernel_bytes.items():
         ms = avg_ms(name)

@@ -26,19 +26,8 @@ struct FusedArgs {
     hipStream_t stream;
 };
 
-struct BwdRegsArgs {
-    const void* logits; int dtype; int64_t n_rows, vocab, row_stride;
-    const void* labels; int labels_dtype; float inv_t;
-    const float* lse; const float* entropy; const float* g_logp; const float* g_entropy;
-    void* dlogits; int64_t d_stride;
-    hipStream_t stream;
-};
-
 // True if rows of this dtype / vocab / alignment fit the row-in-registers kernels.
 bool row_sweep_supported(int dtype, int64_t vocab, const void* in, int64_t in_stride, const void* out,
                          int64_t out_stride, int64_t n_rows);
-
-// Backward from a saved logsumexp with the row-in-registers access pattern (same dtype in/out).
-int bwd_regs_launch(const BwdRegsArgs& a);
 
 }  // namespace mrl

@@ -9,9 +9,11 @@
 // separated in time, which is also the access pattern that the HBM system serves best for a
 // read+write stream.
 //
-// Two kernels share the skeleton:
-//   fused_sweep_kernel   forward statistics + policy-loss gradient + dlogits (eager gradient)
-//   bwd_regs_kernel      dlogits from a saved logsumexp (the autograd backward of the split path)
+// fused_sweep_kernel launches one workgroup per row; fused_sweep_persistent_kernel (the default
+// for large batches) launches one workgroup per CU that walks its rows, which removes the
+// workgroup launch gap between rows.
+#include <stdlib.h>
+
 #include "mrl_internal.h"
 #include "policy_terms.h"
 #include "row_sweep.h"
@@ -203,44 +205,144 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_kernel(
     }
 }
 
-template <int DT, int NV, bool kEntropy>
-__global__ __launch_bounds__(kBlock) void bwd_regs_kernel(
-    const typename Elem<DT>::T* logits, int64_t row_stride, int vocab, const void* __restrict__ labels,
-    int labels_dtype, float inv_t, const float* __restrict__ lse_in, const float* __restrict__ ent_in,
-    const float* __restrict__ g_logp, const float* __restrict__ g_entropy, typename Elem<DT>::T* dlogits,
-    int64_t d_stride) {
+// Persistent variant of the fused sweep: one workgroup per CU walks rows r, r + grid, ... and, while
+// it turns the registers of row r into dlogits, refills each register with the same vector of its
+// NEXT row as soon as the store has been issued.  The loads of row r+grid are therefore in flight
+// during the gradient pass of row r, and the statistics pass of the next row starts on data that
+// has already arrived - the register file never has to hold two rows.
+template <int DT, int NV, bool kEntropy, bool kInterleave>
+__global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
+    const typename Elem<DT>::T* logits, int64_t row_stride, int vocab, int64_t n_rows,
+    const void* __restrict__ labels, int labels_dtype, float inv_t, const float* __restrict__ row_ops, int has_old,
+    Params p, float grad_scale, typename Elem<DT>::T* dlogits, int64_t d_stride, float* __restrict__ logp,
+    float* __restrict__ entropy, float* __restrict__ row_terms) {
     using E = Elem<DT>;
     using T = typename E::T;
     constexpr int kVec = E::kVec;
-    const int64_t r = blockIdx.x;
+    __shared__ Stats lds[kWaves + 1];
+
     const int tid = threadIdx.x;
     const int n_vec = vocab / kVec;
-    const T* row = logits + r * row_stride;
-    u32x4* ovec = reinterpret_cast<u32x4*>(dlogits + r * d_stride);
-    const u32x4* ivec = reinterpret_cast<const u32x4*>(row);
+    const float k = inv_t * kLog2e;
+    const int64_t step = gridDim.x;
 
-    const float g_lp = g_logp ? g_logp[r] : 0.f;
-    const float g_h = (kEntropy && g_entropy) ? g_entropy[r] : 0.f;
-    if (g_lp == 0.f && g_h == 0.f) {
-        zero_row(ovec, n_vec);
-        return;
-    }
     u32x4 v[NV];
+    int64_t r = blockIdx.x;
+    bool loaded = false;                    // v holds row r
+    if (r < n_rows && row_ops[r * MRL_ROW_OPS + MRL_OP_MASK] != 0.f) {
+        const u32x4* ivec = reinterpret_cast<const u32x4*>(logits + r * row_stride);
 #pragma unroll
-    for (int q = 0; q < NV; ++q) {
-        const int idx = q * kBlock + tid;
-        if (idx < n_vec) v[q] = __builtin_nontemporal_load(ivec + idx);
+        for (int q = 0; q < NV; ++q) {
+            const int idx = q * kBlock + tid;
+            if (idx < n_vec) v[q] = __builtin_nontemporal_load(ivec + idx);
+        }
+        loaded = true;
     }
-    const float lse = lse_in[r];
-    RowGrad g;
-    g.k = inv_t * kLog2e;
-    g.lse2 = lse * kLog2e;
-    g.c0 = kEntropy ? inv_t * (-g_lp + g_h * (lse - ent_in[r])) : -g_lp * inv_t;
-    g.c1 = kEntropy ? -g_h * inv_t * inv_t : 0.f;
-    g.onehot = g_lp * inv_t;
-    const int64_t y = load_label(labels, labels_dtype, r);
-    const bool y_ok = (y >= 0) && (y < (int64_t)vocab);
-    store_grads<DT, NV, kEntropy>(v, n_vec, g, y_ok ? (int)(y / kVec) : -1, y_ok ? (int)(y % kVec) : 0, ovec);
+    for (; r < n_rows; r += step) {
+        const T* row = logits + r * row_stride;
+        u32x4* ovec = reinterpret_cast<u32x4*>(dlogits + r * d_stride);
+        const float* ops = row_ops + r * MRL_ROW_OPS;
+        const float m = ops[MRL_OP_MASK];
+        const int64_t r2 = r + step;
+        const bool next_live = (r2 < n_rows) && (row_ops[r2 * MRL_ROW_OPS + MRL_OP_MASK] != 0.f);
+        const u32x4* nvec = reinterpret_cast<const u32x4*>(logits + (next_live ? r2 : r) * row_stride);
+
+        bool wrote = false;                 // dlogits of row r written (and the next row prefetched) in the gradient pass
+        if (m != 0.f) {
+            const int64_t y = load_label(labels, labels_dtype, r);
+            const bool y_ok = (y >= 0) && (y < (int64_t)vocab);
+            const float z_y = y_ok ? E::load(row + y) : 0.f;
+            Stats st = {kMaxInit, 0.f, 0.f};
+#pragma unroll
+            for (int q = 0; q < NV; ++q) {
+                const int idx = q * kBlock + tid;
+                if (idx < n_vec) {
+                    float z[kVec];
+                    E::unpack(v[q], z);
+                    float vmax = st.m;
+#pragma unroll
+                    for (int i = 0; i < kVec; ++i) vmax = fmaxf(vmax, z[i]);
+                    grow_max<kEntropy>(st, vmax, k);
+                    const float mk = st.m * k;
+#pragma unroll
+                    for (int i = 0; i < kVec; ++i) add_one<kEntropy>(st, z[i], k, mk);
+                }
+            }
+            const Stats tot = block_reduce_1024<kEntropy>(st, k, lds);
+            const float lse = (tot.m * k + fast_log2(tot.s)) * kLn2;
+            const float lp = (y_ok ? z_y * inv_t : tot.m * inv_t) - lse;
+            const float ent = kEntropy ? lse - (tot.u / tot.s) * inv_t : 0.f;
+            const Token t = token_terms<true>(lp, ops[MRL_OP_OLD], has_old != 0, ops[MRL_OP_REF], ops[MRL_OP_ADV], p);
+            const float inv_tok = ops[MRL_OP_INVTOK];
+            const float g_lp = grad_scale * m * (ops[MRL_OP_WPG] * t.d_pg + p.kl_coef * inv_tok * t.d_kl);
+            const float g_h = kEntropy ? grad_scale * m * (-p.entropy_coeff * inv_tok) : 0.f;
+            if (g_lp != 0.f || g_h != 0.f) {
+                RowGrad g;
+                g.k = k;
+                g.lse2 = lse * kLog2e;
+                g.c0 = kEntropy ? inv_t * (-g_lp + g_h * (lse - ent)) : -g_lp * inv_t;
+                g.c1 = kEntropy ? -g_h * inv_t * inv_t : 0.f;
+                g.onehot = g_lp * inv_t;
+                const int y_vec = y_ok ? (int)(y / kVec) : -1;
+                const int y_lane = y_ok ? (int)(y % kVec) : 0;
+#pragma unroll
+                for (int q = 0; q < NV; ++q) {
+                    const int idx = q * kBlock + tid;
+                    if (idx < n_vec) {
+                        float z[kVec], d[kVec];
+                        E::unpack(v[q], z);
+#pragma unroll
+                        for (int i = 0; i < kVec; ++i) d[i] = grad_elem<kEntropy>(g, z[i]);
+                        if (idx == y_vec) {
+#pragma unroll
+                            for (int i = 0; i < kVec; ++i)
+                                if (i == y_lane) d[i] += g.onehot;
+                        }
+                        __builtin_nontemporal_store(E::pack(d), ovec + idx);
+                        if (kInterleave && next_live) v[q] = __builtin_nontemporal_load(nvec + idx);   // refill
+                    }
+                }
+                if (!kInterleave && next_live) {
+#pragma unroll
+                    for (int q = 0; q < NV; ++q) {
+                        const int idx = q * kBlock + tid;
+                        if (idx < n_vec) v[q] = __builtin_nontemporal_load(nvec + idx);
+                    }
+                }
+                wrote = true;
+            }
+            if (tid == 0) {
+                if (logp) logp[r] = lp;
+                if (entropy) entropy[r] = ent;
+                float* out = row_terms + r * S_N;
+                out[S_PG] = t.pg * m;
+                out[S_CLIP] = t.clipped * m;
+                out[S_PPOKL] = t.neg_logr * m;
+                out[S_KL] = t.kl * m;
+                out[S_ENT] = ent * m;
+                out[S_MASK] = m;
+                out[6] = 0.f;
+                out[7] = 0.f;
+            }
+        } else if (tid == 0) {
+            if (logp) logp[r] = 0.f;
+            if (entropy) entropy[r] = 0.f;
+#pragma unroll
+            for (int q = 0; q < S_N; ++q) row_terms[r * S_N + q] = 0.f;
+        }
+        if (!wrote) {                       // no gradient for this row: zeros, then fetch the next row plainly
+            zero_row(ovec, n_vec);
+            if (next_live) {
+#pragma unroll
+                for (int q = 0; q < NV; ++q) {
+                    const int idx = q * kBlock + tid;
+                    if (idx < n_vec) v[q] = __builtin_nontemporal_load(nvec + idx);
+                }
+            }
+        }
+        loaded = next_live;
+    }
+    (void)loaded;
 }
 
 // Conditional in-place rescale: multiplies every row by upstream/assumed unless that ratio is 1.
@@ -273,11 +375,41 @@ inline int pick_nv(int64_t n_vec) {
     return 0;
 }
 
+// Number of CUs of the current device (one persistent workgroup each); 0 if the query fails.
+int cu_count() {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    return n;
+}
+
+// MRL_SWEEP_PERSISTENT=0 selects the one-workgroup-per-row launch (a tuning / debugging switch).
+bool persistent_enabled() {
+    static const bool on = [] {
+        const char* e = getenv("MRL_SWEEP_PERSISTENT");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
 template <int DT, int NV>
 int launch_fused(const mrl::FusedArgs& a) {
     using T = typename Elem<DT>::T;
-    const dim3 grid((unsigned)a.n_rows), block(kBlock);
+    const dim3 block(kBlock);
     const Params p = {a.clip_lo, a.clip_hi, a.kl_coef, a.entropy_coeff, 1.f, a.kl_penalty, 0};
+    const int cus = persistent_enabled() ? cu_count() : 0;
+    if (cus > 0 && a.n_rows > 2 * (int64_t)cus) {
+        const dim3 pgrid((unsigned)cus);
+#define MRL_FUSEDP_LAUNCH(ENT)                                                                                     \
+    hipLaunchKernelGGL((fused_sweep_persistent_kernel<DT, NV, ENT, false>), pgrid, block, 0, a.stream, (const T*)a.logits, \
+                       a.row_stride, (int)a.vocab, a.n_rows, a.labels, a.labels_dtype, a.inv_t, a.row_ops,         \
+                       a.has_old, p, a.grad_scale, (T*)a.dlogits, a.d_stride, a.logp, a.entropy, a.row_terms)
+        if (a.with_entropy) MRL_FUSEDP_LAUNCH(true);
+        else MRL_FUSEDP_LAUNCH(false);
+#undef MRL_FUSEDP_LAUNCH
+        return mrl::check_launch("mrl_fused_logprob_loss");
+    }
+    const dim3 grid((unsigned)a.n_rows);
 #define MRL_FUSED_LAUNCH(ENT)                                                                                  \
     hipLaunchKernelGGL((fused_sweep_kernel<DT, NV, ENT>), grid, block, 0, a.stream, (const T*)a.logits,        \
                        a.row_stride, (int)a.vocab, a.labels, a.labels_dtype, a.inv_t, a.row_ops, a.has_old, p, \
@@ -286,20 +418,6 @@ int launch_fused(const mrl::FusedArgs& a) {
     else MRL_FUSED_LAUNCH(false);
 #undef MRL_FUSED_LAUNCH
     return mrl::check_launch("mrl_fused_logprob_loss");
-}
-
-template <int DT, int NV>
-int launch_bwd_regs(const mrl::BwdRegsArgs& a) {
-    using T = typename Elem<DT>::T;
-    const dim3 grid((unsigned)a.n_rows), block(kBlock);
-#define MRL_BWDR_LAUNCH(ENT)                                                                              \
-    hipLaunchKernelGGL((bwd_regs_kernel<DT, NV, ENT>), grid, block, 0, a.stream, (const T*)a.logits,      \
-                       a.row_stride, (int)a.vocab, a.labels, a.labels_dtype, a.inv_t, a.lse, a.entropy,   \
-                       a.g_logp, a.g_entropy, (T*)a.dlogits, a.d_stride)
-    if (a.g_entropy) MRL_BWDR_LAUNCH(true);
-    else MRL_BWDR_LAUNCH(false);
-#undef MRL_BWDR_LAUNCH
-    return mrl::check_launch("mrl_vocab_logprob_bwd");
 }
 
 #define MRL_NV_SWITCH(FUNC, DT, nv, a)      \
@@ -313,19 +431,6 @@ int launch_bwd_regs(const mrl::BwdRegsArgs& a) {
 
 template <int DT>
 int fused_by_nv(int nv, const mrl::FusedArgs& a) { MRL_NV_SWITCH(launch_fused, DT, nv, a) }
-// the 8-vector instantiation of the backward kernel is left out: the compiler spills it heavily
-// for fp32, and 12 vectors per thread cost nothing extra (unused slots are predicated off)
-template <int DT>
-int bwd_by_nv(int nv, const mrl::BwdRegsArgs& a) {
-    switch (nv) {
-        case 4: return launch_bwd_regs<DT, 4>(a);
-        case 8:
-        case 12: return launch_bwd_regs<DT, 12>(a);
-        case 16: return launch_bwd_regs<DT, 16>(a);
-        default: return launch_bwd_regs<DT, 19>(a);
-    }
-}
-
 }  // namespace
 
 namespace mrl {
@@ -340,15 +445,6 @@ bool row_sweep_supported(int dtype, int64_t vocab, const void* in, int64_t in_st
     if (!aligned(in, 16) || !aligned(out, 16)) return false;
     if (n_rows > 1 && ((in_stride * eb) % 16 != 0 || (out_stride * eb) % 16 != 0)) return false;
     return true;
-}
-
-int bwd_regs_launch(const BwdRegsArgs& a) {
-    const int nv = pick_nv(a.vocab / (16 / float_dtype_bytes(a.dtype)));
-    switch (a.dtype) {
-        case MRL_F32: return bwd_by_nv<MRL_F32>(nv, a);
-        case MRL_BF16: return bwd_by_nv<MRL_BF16>(nv, a);
-        default: return bwd_by_nv<MRL_F16>(nv, a);
-    }
 }
 
 }  // namespace mrl

@@ -9,7 +9,6 @@
 // state costs one convert, one FMA and one v_exp_f32 per element.  Wavefront reduction uses
 // cross-lane shuffles, the four wavefronts combine through LDS.
 #include "mrl_internal.h"
-#include "row_sweep.h"
 #include "vocab_common.h"
 
 namespace {
@@ -416,16 +415,6 @@ extern "C" int mrl_vocab_logprob_bwd(const void* logits, int logits_dtype, int64
         vector_ok = out_aligned_at_head && (strides_ok || n_rows == 1);
     }
     hipStream_t s = mrl::as_stream(stream);
-    // same dtype in and out, aligned rows that fit the register file: the row-in-registers kernel
-    // (reads and writes of a workgroup separated in time) serves the read+write stream best
-    if (dlogits_dtype == logits_dtype &&
-        mrl::row_sweep_supported(logits_dtype, vocab, logits, row_stride, dlogits, dlogits_row_stride, n_rows)) {
-        mrl::BwdRegsArgs a;
-        a.logits = logits; a.dtype = logits_dtype; a.n_rows = n_rows; a.vocab = vocab; a.row_stride = row_stride;
-        a.labels = labels; a.labels_dtype = labels_dtype; a.inv_t = inv_temperature; a.lse = lse; a.entropy = entropy;
-        a.g_logp = g_logp; a.g_entropy = g_entropy; a.dlogits = dlogits; a.d_stride = dlogits_row_stride; a.stream = s;
-        return mrl::bwd_regs_launch(a);
-    }
     const int v = (int)vocab;
 #define MRL_BWD(DI, DO)                                                                                      \
     (labels_dtype == MRL_I32                                                                                 \
