@@ -345,22 +345,26 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
     (void)loaded;
 }
 
-// Conditional in-place rescale: multiplies every row by upstream/assumed unless that ratio is 1.
+// Conditional in-place rescale: multiplies every row by upstream/assumed unless that ratio is 1
+// (then every workgroup exits at once; the grid is kept small so that this costs microseconds).
 template <int DT>
 __global__ __launch_bounds__(256) void scale_rows_kernel(typename Elem<DT>::T* x, int64_t row_stride, int vocab,
-                                                         const float* __restrict__ upstream, float assumed) {
+                                                         int64_t n_rows, const float* __restrict__ upstream,
+                                                         float assumed) {
     using E = Elem<DT>;
     constexpr int kVec = E::kVec;
     const float ratio = *upstream / assumed;
     if (ratio == 1.f) return;
-    u32x4* vec = reinterpret_cast<u32x4*>(x + (int64_t)blockIdx.x * row_stride);
     const int n_vec = vocab / kVec;
-    for (int idx = threadIdx.x; idx < n_vec; idx += 256) {
-        float z[kVec];
-        E::unpack(vec[idx], z);
+    for (int64_t r = blockIdx.x; r < n_rows; r += gridDim.x) {
+        u32x4* vec = reinterpret_cast<u32x4*>(x + r * row_stride);
+        for (int idx = threadIdx.x; idx < n_vec; idx += 256) {
+            float z[kVec];
+            E::unpack(vec[idx], z);
 #pragma unroll
-        for (int i = 0; i < kVec; ++i) z[i] *= ratio;
-        vec[idx] = E::pack(z);
+            for (int i = 0; i < kVec; ++i) z[i] *= ratio;
+            vec[idx] = E::pack(z);
+        }
     }
 }
 
@@ -517,19 +521,19 @@ extern "C" int mrl_scale_rows(void* x, int dtype, int64_t n_rows, int64_t vocab,
     MRL_REQUIRE(vocab % (16 / eb) == 0 && mrl::aligned(x, 16) && (n_rows == 1 || (row_stride * eb) % 16 == 0),
                 MRL_ERR_UNSUPPORTED, "%s: needs 16-byte aligned rows", fn);
     hipStream_t s = mrl::as_stream(stream);
-    const dim3 grid((unsigned)n_rows), block(256);
+    const dim3 grid((unsigned)(n_rows < 4096 ? n_rows : 4096)), block(256);
     switch (dtype) {
         case MRL_F32:
             hipLaunchKernelGGL(scale_rows_kernel<MRL_F32>, grid, block, 0, s, (float*)x, row_stride, (int)vocab,
-                               upstream, assumed);
+                               n_rows, upstream, assumed);
             break;
         case MRL_BF16:
             hipLaunchKernelGGL(scale_rows_kernel<MRL_BF16>, grid, block, 0, s, (uint16_t*)x, row_stride, (int)vocab,
-                               upstream, assumed);
+                               n_rows, upstream, assumed);
             break;
         default:
             hipLaunchKernelGGL(scale_rows_kernel<MRL_F16>, grid, block, 0, s, (uint16_t*)x, row_stride, (int)vocab,
-                               upstream, assumed);
+                               n_rows, upstream, assumed);
             break;
     }
     return mrl::check_launch(fn);

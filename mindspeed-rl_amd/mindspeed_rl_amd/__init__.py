@@ -9,7 +9,7 @@ from .advantage import (FixedKLController, compute_group_norm_advantage_return, 
                         dynamic_sampling_keep_mask)
 from .functional import masked_mean, masked_sum
 from .loss import (BaseLossFunc, DAPOActorLossFunc, GRPOActorLossFunc, LossFuncFactory, LossRegister,
-                   MultimodalLogProbComputer, ReferenceLossFunc, StandardLogProbComputer, fused_logprob_policy_loss, fused_supported,
+                   MultimodalLogProbComputer, PPOActorLossFunc, ReferenceLossFunc, StandardLogProbComputer, fused_logprob_policy_loss, fused_supported,
                    policy_loss)
 from .packing import (generate_mask, pack_index, postprocess_packed_seqs, preprocess_packed_seqs, response_window,
                       truncate_middle_and_pad, truncate_prompt_and_pad)

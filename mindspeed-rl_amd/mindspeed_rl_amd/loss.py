@@ -502,6 +502,63 @@ class DAPOActorLossFunc(BaseLossFunc):
         return loss, out[2], out[3], out[4], out[5]
 
 
+@LossFuncFactory.register_loss("ray_ppo", "actor")
+class PPOActorLossFunc(BaseLossFunc):
+    """Reference: ``ppo_actor_loss_func.py:13-133``: the GRPO surrogate without the KL term; four
+    statistics (no ``actor/kl_loss``)."""
+
+    def __init__(self):
+        super().__init__()
+        self.clip_ratio = 0.2
+        self.entropy_coeff = 0.0
+
+    def add_loss_meta_info(self, meta_info: Dict):
+        if meta_info is None:
+            return
+        if "clip_ratio" in meta_info.keys():
+            self.clip_ratio = float(meta_info["clip_ratio"])
+        for key in ("kl_ctrl", "entropy_coeff"):
+            if key in meta_info.keys():
+                setattr(self, key, meta_info[key])
+
+    @staticmethod
+    def _get_policy_loss_input(batch: Dict[str, torch.Tensor]):
+        if "responses" not in batch:
+            raise ValueError("The responses is None")
+        response_mask = generate_mask(batch["responses"], batch["response_length"])
+        return (response_mask, batch.get("old_log_prob"), batch.get("advantages"), batch.get("ref_log_prob"))
+
+    def compute_loss(self, output: torch.Tensor, batch: Dict[str, torch.Tensor], forward_only=False,
+                     non_loss_data=True, **kwargs) -> Tuple[torch.Tensor, Dict]:
+        if "responses" not in batch:
+            raise ValueError("The responses is None")
+        if forward_only:
+            log_probs, _ = super().compute_log_probs(output=output, batch=batch, **kwargs)
+            return log_probs
+        common = dict(clip_low=self.clip_ratio, clip_high=self.clip_ratio, kl_penalty=None,
+                      entropy_coeff=self.entropy_coeff, token_level_loss=True,
+                      loss_scale=_dynamic_scale(batch, forward_only, kwargs))
+        if _use_fused(output, kwargs):
+            loss, out = fused_logprob_policy_loss(output, batch, **common, **_fused_kwargs(kwargs))
+        else:
+            log_probs, entropy = super().compute_log_probs(output=output, batch=batch,
+                                                           skip_entropy=(self.entropy_coeff == 0), **kwargs)
+            loss, out = policy_loss(log_probs, entropy if self.entropy_coeff != 0 else None,
+                                    batch.get("old_log_prob"), None, batch.get("advantages"),
+                                    response_length=batch["response_length"], **common)
+        loss, stats = _finish(loss, out)
+        del stats[STAT_KEYS[3]]                  # PPO reports no actor/kl_loss
+        return loss, stats
+
+    @staticmethod
+    def _compute_ppo_policy_loss(old_log_prob, log_prob, advantages, eos_mask, cliprange, entropy, entropy_coeff):
+        """Reference: ``ppo_actor_loss_func.py:91-133``: ``(pg_loss, pg_clipfrac, ppo_kl, entropy_loss)``."""
+        loss, out = policy_loss(log_prob, entropy, old_log_prob, None, advantages, mask=eos_mask, clip_low=cliprange,
+                                clip_high=cliprange, kl_penalty=None, entropy_coeff=entropy_coeff,
+                                token_level_loss=True)
+        return loss, out[2], out[3], out[5]
+
+
 @LossFuncFactory.register_loss("ray_grpo", "reference")
 @LossFuncFactory.register_loss("ray_ppo", "reference")
 class ReferenceLossFunc(BaseLossFunc):

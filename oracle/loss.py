@@ -8,6 +8,7 @@ Restates with stock torch ops (so that autograd supplies the backward the refere
 * ``mindspeed_rl/models/loss/dapo_actor_loss_func.py:105-152``     ``_compute_dapo_policy_loss``
 * ``mindspeed_rl/models/loss/grpo_actor_loss_func.py:43-98`` and
   ``dapo_actor_loss_func.py:47-102``                                ``compute_loss`` tail (scale + stats)
+* ``mindspeed_rl/models/loss/ppo_actor_loss_func.py:39-133``       PPO actor (the GRPO surrogate without KL)
 * ``mindspeed_rl/models/loss/logprob_computer.py:94-145``          ``StandardLogProbComputer.compute``
 
 Pinned by ``tests/ut/utils/test_compute_utils.py:92-108`` (KL vectors),
@@ -61,6 +62,21 @@ def grpo_policy_loss(old_log_prob, log_prob, ref_log_prob, advantages, entropy, 
     kl_mean = masked_mean(compute_kl_penalty(log_prob, ref_log_prob, kl_penalty), eos_mask)
     pg_loss = pg_mean + kl_mean * kl_coef - entropy_coeff * entropy_loss
     return pg_loss, clipfrac, ppo_kl, kl_mean, entropy_loss
+
+
+def ppo_policy_loss(old_log_prob, log_prob, advantages, eos_mask, cliprange, entropy, entropy_coeff):
+    """``ppo_actor_loss_func.py:91-133``: the GRPO surrogate without the KL term."""
+    if old_log_prob is None:
+        old_log_prob = log_prob.detach().clone()
+    log_ratio = log_prob - old_log_prob
+    ratio = torch.exp(log_ratio)
+    ppo_kl = masked_mean(-log_ratio, eos_mask)
+    entropy_loss = masked_mean(entropy, eos_mask)
+    surr1 = -advantages * ratio
+    surr2 = -advantages * torch.clamp(ratio, 1.0 - cliprange, 1.0 + cliprange)
+    pg_mean = masked_mean(torch.max(surr1, surr2), eos_mask)
+    clipfrac = masked_mean(torch.gt(surr2, surr1).float(), eos_mask)
+    return pg_mean - entropy_coeff * entropy_loss, clipfrac, ppo_kl, entropy_loss
 
 
 def dapo_policy_loss(old_log_prob, log_prob, entropy, entropy_coeff, advantages, eos_mask,
@@ -166,3 +182,19 @@ def dapo_compute_loss(output, batch, meta, forward_only=False, **kwargs):
     out = dapo_policy_loss(batch.get("old_log_prob"), log_probs, entropy, entropy_coeff,
                            batch.get("advantages"), mask, lo, hi, meta["token_level_loss"])
     return _finish(*out, batch, forward_only, kwargs)
+
+
+def ppo_compute_loss(output, batch, meta, forward_only=False, **kwargs):
+    """``ppo_actor_loss_func.py:39-89``: four statistics, no ``actor/kl_loss``."""
+    if forward_only:
+        return logprob_computer(output, batch, True, **kwargs)[0]
+    entropy_coeff = meta.get("entropy_coeff", 0.0)
+    log_probs, entropy = logprob_computer(output, batch, entropy_coeff == 0, **kwargs)
+    if "responses" not in batch:
+        raise ValueError("The responses is None")
+    mask = packing.generate_mask(batch["responses"], batch["response_length"])
+    pg_loss, clipfrac, ppo_kl, ent = ppo_policy_loss(batch.get("old_log_prob"), log_probs, batch.get("advantages"),
+                                                     mask, meta.get("clip_ratio", 0.2), entropy, entropy_coeff)
+    policy_loss, stats = _finish(pg_loss, clipfrac, ppo_kl, torch.zeros(()), ent, batch, forward_only, kwargs)
+    del stats["actor/kl_loss"]
+    return policy_loss, stats

@@ -622,6 +622,35 @@ def test_padded_vs_packed_and_dapo_bf16(dev, fused):
     assert (dz2.float().cpu() - dz_o2).abs().max().item() < 1e-2 * dz_o2.abs().max().item()
 
 
+@pytest.mark.parametrize("fused", [True, False])
+def test_ppo_actor_loss_parity(dev, fused):
+    """PPO actor (the GRPO surrogate without KL, four statistics), end to end and as a stand-alone op."""
+    gen = torch.Generator().manual_seed(17)
+    logits, b, kw, _, _ = _make_batch(gen, 2, 3, 4, 20, 4096, torch.bfloat16, 3.0, 1)
+    meta = dict(clip_ratio=0.25, entropy_coeff=0.004)
+    zo = logits.float().requires_grad_()
+    want, want_stats = o_loss.ppo_compute_loss(zo, b, meta, **kw)
+    (dz_o,) = torch.autograd.grad(want, zo)
+    f = mrl.LossFuncFactory.get_instance("ray_ppo", "actor")
+    assert isinstance(f, mrl.PPOActorLossFunc)
+    f.add_loss_meta_info({"clip_ratio": 0.25, "entropy_coeff": 0.004, "kl_ctrl": mrl.FixedKLController(0.1)})
+    zd = logits.to(dev).requires_grad_()
+    got, got_stats = f.compute_loss(zd, _to_dev(b, dev), fused=fused, **_to_dev(kw, dev))
+    assert set(got_stats) == set(want_stats) == {"actor/pg_loss", "actor/pg_clipfrac", "actor/ppo_kl", "actor/entropy"}
+    assert abs(got.item() - want.item()) <= TOL_LOSS_REL * abs(want.item()) + 1e-7
+    for k in want_stats:
+        assert abs(got_stats[k] - want_stats[k]) <= TOL_LOSS_REL * abs(want_stats[k]) + 1e-6, k
+    (dz,) = torch.autograd.grad(got, zd)
+    assert (dz.float().cpu() - dz_o).abs().max().item() < TOL_DLOGITS
+    lp, old, _, adv, ent, lens = _loss_case(gen, 8, 33)
+    mask = o_pack.generate_mask(lp, lens)
+    want4 = o_loss.ppo_policy_loss(old, lp, adv, mask, 0.2, ent, 0.01)
+    got4 = mrl.PPOActorLossFunc._compute_ppo_policy_loss(old.to(dev), lp.to(dev), adv.to(dev), mask.to(dev), 0.2,
+                                                         ent.to(dev), 0.01)
+    assert len(got4) == 4
+    _check_loss(got4, want4, [], [])
+
+
 def test_fused_sweep_specifics(dev):
     """The one-sweep path: agreement with the split kernels, an upstream scale that differs from
     the expected one (rescale kernel), in-place gradients, tokens whose mask reaches past the

@@ -98,6 +98,7 @@ def test_registry_contract(reference_vectors):
     assert isinstance(mrl.LossFuncFactory.get_instance("ray_grpo", "actor"), mrl.GRPOActorLossFunc)
     key = reference_vectors["dapo_defaults"]["registry_key"]
     assert isinstance(mrl.LossFuncFactory.get_instance(*key), mrl.DAPOActorLossFunc)
+    assert isinstance(mrl.LossFuncFactory.get_instance("ray_ppo", "actor"), mrl.PPOActorLossFunc)
     assert isinstance(mrl.LossFuncFactory.get_instance("ray_grpo", "reference"), mrl.ReferenceLossFunc)
     assert isinstance(mrl.LossFuncFactory.get_instance("ray_ppo", "reference"), mrl.ReferenceLossFunc)
     assert mrl.LossFuncFactory.get_instance("nope", "actor") is None
