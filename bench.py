@@ -43,7 +43,9 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS) + ["c3fwd"],
+                    help="c3fwd: the fused lm_head + log-prob forward of configs[3] (bf16 MFMA, logits never stored)")
+    ap.add_argument("--tokens", type=int, default=163840, help="rows of the c3fwd workload")
     ap.add_argument("--entropy-coeff", type=float, default=0.001,
                     help="non-zero so that the forward computes entropy and the backward its gradient")
     ap.add_argument("--path", default="fused", choices=["fused", "split"],
@@ -163,6 +165,53 @@ def cpu_baseline(torch, w, rows_target, entropy_coeff, seed):
     }
 
 
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def run_lmhead(args):
+    """configs[3], forward part: hidden [T, 3584] ~N(0,1), W [152064, 3584] ~N(0,0.02), bf16; one step =
+    log-prob + entropy + logsumexp of every token without materialising the logits."""
+    import torch
+    import mindspeed_rl_amd as mrl
+    from mindspeed_rl_amd import lmhead
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    tokens, vocab, hdim = args.tokens, 152064, 3584
+    g = torch.Generator(device=dev).manual_seed(args.seed)
+    hidden = torch.randn(tokens, hdim, generator=g, device=dev).to(torch.bfloat16)
+    weight = (torch.randn(vocab, hdim, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    labels = torch.randint(0, vocab, (tokens,), generator=g, device=dev)
+    for _ in range(args.warmup):
+        mrl.lmhead_logprob(hidden, weight, labels)
+    torch.cuda.synchronize()
+    lmhead.kernel_events = []
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        lp, ent, lse = mrl.lmhead_logprob(hidden, weight, labels)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    events, lmhead.kernel_events = lmhead.kernel_events, None
+    ms = sum(s.elapsed_time(e) for (_, s, e, _) in events) / len(events)
+    flops = 2.0 * tokens * vocab * hdim
+    tflops = flops / (ms * 1e-3) / 1e12
+    # spot check against a plain GEMM on a slice of the rows
+    ref = torch.log_softmax(torch.nn.functional.linear(hidden[:256].float(), weight.float()), -1)
+    err = (lp[:256] - ref.gather(-1, labels[:256, None]).squeeze(-1)).abs().max().item()
+    result = {
+        "metric": "tokens/sec for fused lm_head+logprob forward; MFMA TFLOP/s as % of bf16 dense peak",
+        "value": tokens / (elapsed / args.steps), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": elapsed * 1e3 / args.steps, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "configs[3] forward: hidden [%d,3584] x W [152064,3584]^T, online logsumexp, logits never "
+                               "stored" % tokens, "accumulate": "f32"},
+        "roofline": {"kernel": "lmhead_fwd_kernel + lmhead_finish_kernel (mrl_lmhead_logprob_fwd)", "bound": "mfma",
+                     "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "flops_per_launch": flops, "avg_ms": ms},
+        "max_abs_err_vs_fp32_gemm_256_rows": err,
+    }
+    print(json.dumps(result), flush=True)
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -176,6 +225,9 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     _lib.load()
+    if args.workload == "c3fwd":
+        run_lmhead(args)
+        return
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     w = WORKLOADS[args.workload]

@@ -294,6 +294,27 @@ int mrl_scale_rows(void* x, int dtype, int64_t n_rows, int64_t vocab, int64_t ro
                    const float* upstream, float assumed, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Fused lm_head + log-prob, forward (no counterpart in the reference, which always materialises
+ * the [T, V] logits in GPTModel.output_layer and then runs compute_log_probs on them,
+ * utils/compute.py:29-51): logits[t, v] = sum_k hidden[t, k] * weight[v, k] are produced tile by
+ * tile on the bf16 matrix cores with fp32 accumulation and consumed by an online log-sum-exp,
+ * so they never reach memory.  The statistics use the fp32 logits (the reference rounds the
+ * materialised logits to bf16 first).
+ *
+ * hidden: [n_tokens, hidden_dim] bf16, weight: [vocab, hidden_dim] bf16 (the layout of a
+ * torch.nn.Linear weight), both dense and 16-byte aligned; hidden_dim % 64 == 0.  labels
+ * [n_tokens] I32 / I64.  Outputs as mrl_vocab_logprob_fwd (entropy, lse nullable).  workspace:
+ * mrl_lmhead_workspace_bytes(n_tokens, vocab) bytes of device memory, 16-byte aligned, holding
+ * the per-vocabulary-group partial statistics (MRL_LMHEAD_GROUPS x n_tokens x 16 bytes).
+ */
+#define MRL_LMHEAD_GROUPS 8
+int64_t mrl_lmhead_workspace_bytes(int64_t n_tokens, int64_t vocab);
+int mrl_lmhead_logprob_fwd(const void* hidden, const void* weight, int64_t n_tokens, int64_t vocab,
+                           int64_t hidden_dim, const void* labels, int labels_dtype,
+                           float inv_temperature, float* logp, float* entropy, float* lse,
+                           void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Plain device-to-device copy kernel of n_bytes (multiple of 16, 16-byte aligned pointers);
  * used to calibrate the rocprofv3 FETCH_SIZE / WRITE_SIZE counters and as the measured
  * bandwidth ceiling next to the 8 TB/s vendor peak.  No counterpart in the reference. */

@@ -1,0 +1,283 @@
+// Fused lm_head + log-prob for gfx950: streams hidden x W_vocab^T tiles through bf16 MFMA and
+// keeps an online log-sum-exp per token, so the [T, V] logits are never written to memory.
+//
+//   logits[t, v] = sum_k hidden[t, k] * W[v, k]        (bf16 operands, fp32 accumulate)
+//   lse, logp[label], entropy exactly as the vocabulary sweep computes them, on the fp32 logits
+//
+// Mapping.  The product is computed TRANSPOSED, S^T = W_tile x hidden_tile^T with
+// v_mfma_f32_32x32x16_bf16: vocabulary rows are the MFMA's M, tokens its N.  In the 32x32 result
+// layout a lane then owns ONE token column and 16 vocabulary rows, so the softmax statistics of a
+// token accumulate inside a lane; only the two lane halves and the two vocabulary wavefronts have
+// to be combined once, at the very end.  A workgroup (256 threads = 2x2 wavefronts) owns 128 tokens
+// and walks over the 256-row vocabulary tiles of its vocabulary group; each wavefront computes a
+// 128 (vocab) x 64 (token) sub-tile = 4x2 MFMA blocks per 16-wide k-step, operands staged through
+// LDS (rows padded to 144 bytes), the next k-step's global loads in flight during the MFMAs.
+// Vocabulary groups (gridDim = token tiles x groups, group = blockIdx % groups so that the
+// workgroups of one XCD read the same W rows) leave per-group partial statistics that a small
+// second kernel merges, together with the label logit (one fp32 dot product per token).
+#include "mrl_internal.h"
+#include "vocab_common.h"
+
+namespace {
+
+using namespace mrl_vocab;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kThreads = 256;
+constexpr int BV = 256;            // vocabulary rows per macro tile
+constexpr int BT = 128;            // tokens per macro tile
+constexpr int BK = 64;             // k elements per LDS stage
+constexpr int kLdsStride = BK + 8; // bf16 elements per LDS row: 144 bytes, breaks the bank pattern
+constexpr int kChunksPerRow = BK / 8;                          // 16-byte chunks per row and stage
+constexpr int kALoads = BV * kChunksPerRow / kThreads;         // 8 chunks per thread
+constexpr int kBLoads = BT * kChunksPerRow / kThreads;         // 4 chunks per thread
+
+__global__ __launch_bounds__(kThreads, 2) void lmhead_fwd_kernel(
+    const uint16_t* __restrict__ hidden, const uint16_t* __restrict__ weight, int64_t n_tokens, int vocab, int hdim,
+    int n_groups, int tiles_per_group, float k_scale, float* __restrict__ partial) {
+    __shared__ __attribute__((aligned(16))) uint16_t As[BV * kLdsStride];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[BT * kLdsStride];
+    __shared__ Stats comb[2][2][64];   // [token half][token block][lane % 32 (+32 unused)]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wv = wave >> 1, wt = wave & 1;
+    const int group = blockIdx.x % n_groups;
+    const int64_t t0 = (int64_t)(blockIdx.x / n_groups) * BT;
+    const int n_vtiles = (vocab + BV - 1) / BV;
+    const int tile_begin = group * tiles_per_group;
+    const int tile_end = min(tile_begin + tiles_per_group, n_vtiles);
+
+    // global -> LDS staging: chunk c = tid + i*256 covers row c/8, 16-byte column c%8
+    const int ld_row = tid >> 3, ld_col = tid & 7;
+    // token rows of this workgroup as 32-bit element offsets from the tile base, clamped so that
+    // tail rows read valid memory (they are masked on output)
+    const uint16_t* b_base = hidden + t0 * hdim;
+    int b_off[kBLoads];
+#pragma unroll
+    for (int i = 0; i < kBLoads; ++i) {
+        int64_t r = ld_row + 32 * i;
+        if (t0 + r >= n_tokens) r = n_tokens - 1 - t0;
+        b_off[i] = (int)r * hdim + ld_col * 8;
+    }
+
+    Stats st[2];
+#pragma unroll
+    for (int tb = 0; tb < 2; ++tb) st[tb] = {kMaxInit, 0.f, 0.f};
+
+    for (int tile = tile_begin; tile < tile_end; ++tile) {
+        const int v0 = tile * BV;
+        const uint16_t* a_base = weight + (int64_t)v0 * hdim;
+        int a_off[kALoads];
+#pragma unroll
+        for (int i = 0; i < kALoads; ++i) {
+            int r = ld_row + 32 * i;
+            if (v0 + r >= vocab) r = vocab - 1 - v0;
+            a_off[i] = r * hdim + ld_col * 8;
+        }
+        floatx16 acc[4][2];
+#pragma unroll
+        for (int vb = 0; vb < 4; ++vb)
+#pragma unroll
+            for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc[vb][tb][i] = 0.f;
+
+        u32x4 a_reg[kALoads], b_reg[kBLoads];
+#pragma unroll
+        for (int i = 0; i < kALoads; ++i) a_reg[i] = *reinterpret_cast<const u32x4*>(a_base + a_off[i]);
+#pragma unroll
+        for (int i = 0; i < kBLoads; ++i) b_reg[i] = *reinterpret_cast<const u32x4*>(b_base + b_off[i]);
+
+        const int n_ksteps = hdim / BK;
+        for (int kstep = 0; kstep < n_ksteps; ++kstep) {
+            __syncthreads();                               // the previous stage has been consumed
+#pragma unroll
+            for (int i = 0; i < kALoads; ++i)
+                *reinterpret_cast<u32x4*>(&As[(ld_row + 32 * i) * kLdsStride + ld_col * 8]) = a_reg[i];
+#pragma unroll
+            for (int i = 0; i < kBLoads; ++i)
+                *reinterpret_cast<u32x4*>(&Bs[(ld_row + 32 * i) * kLdsStride + ld_col * 8]) = b_reg[i];
+            __syncthreads();
+            if (kstep + 1 < n_ksteps) {                    // next stage's loads fly during the MFMAs
+                const int off = (kstep + 1) * BK;
+#pragma unroll
+                for (int i = 0; i < kALoads; ++i) a_reg[i] = *reinterpret_cast<const u32x4*>(a_base + off + a_off[i]);
+#pragma unroll
+                for (int i = 0; i < kBLoads; ++i) b_reg[i] = *reinterpret_cast<const u32x4*>(b_base + off + b_off[i]);
+            }
+#pragma unroll
+            for (int ks = 0; ks < BK / 16; ++ks) {
+                const int koff = ks * 16 + (lane >> 5) * 8;
+                bf16x8 af[4], bfr[2];
+#pragma unroll
+                for (int vb = 0; vb < 4; ++vb)
+                    af[vb] = *reinterpret_cast<const bf16x8*>(&As[(wv * 128 + vb * 32 + (lane & 31)) * kLdsStride + koff]);
+#pragma unroll
+                for (int tb = 0; tb < 2; ++tb)
+                    bfr[tb] = *reinterpret_cast<const bf16x8*>(&Bs[(wt * 64 + tb * 32 + (lane & 31)) * kLdsStride + koff]);
+#pragma unroll
+                for (int vb = 0; vb < 4; ++vb)
+#pragma unroll
+                    for (int tb = 0; tb < 2; ++tb)
+                        acc[vb][tb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[vb], bfr[tb], acc[vb][tb], 0, 0, 0);
+            }
+        }
+
+        // online softmax statistics of this tile: a lane holds 64 vocabulary rows of each token column
+        const bool ragged = (v0 + BV > vocab);
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb) {
+            if (ragged) {
+#pragma unroll
+                for (int vb = 0; vb < 4; ++vb)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const int v = v0 + wv * 128 + vb * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
+                        if (v >= vocab) acc[vb][tb][i] = kMaxInit;
+                    }
+            }
+            float vmax = st[tb].m;
+#pragma unroll
+            for (int vb = 0; vb < 4; ++vb)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) vmax = fmaxf(vmax, acc[vb][tb][i]);
+            grow_max<true>(st[tb], vmax, k_scale);
+            const float mk = st[tb].m * k_scale;
+#pragma unroll
+            for (int vb = 0; vb < 4; ++vb)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) add_one<true>(st[tb], acc[vb][tb][i], k_scale, mk);
+        }
+    }
+
+    // combine the two lane halves (same token, other vocabulary rows), then the two vocabulary wavefronts
+#pragma unroll
+    for (int tb = 0; tb < 2; ++tb) {
+        Stats o;
+        o.m = __shfl_xor(st[tb].m, 32, 64);
+        o.s = __shfl_xor(st[tb].s, 32, 64);
+        o.u = __shfl_xor(st[tb].u, 32, 64);
+        st[tb] = merge<true>(st[tb], o, k_scale);
+    }
+    __syncthreads();
+    if (wv == 1 && lane < 32) {
+        comb[wt][0][lane] = st[0];
+        comb[wt][1][lane] = st[1];
+    }
+    __syncthreads();
+    if (wv == 0 && lane < 32) {
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb) {
+            const Stats r = merge<true>(st[tb], comb[wt][tb][lane], k_scale);
+            const int64_t t = t0 + wt * 64 + tb * 32 + lane;
+            if (t < n_tokens) {
+                float* p = partial + ((int64_t)group * n_tokens + t) * 4;
+                p[0] = r.m;
+                p[1] = r.s;
+                p[2] = r.u;
+                p[3] = 0.f;
+            }
+        }
+    }
+}
+
+// One wavefront per token: merges the per-group partial statistics and computes the label logit
+// as an fp32 dot product of the token's hidden row with the label's weight row.
+template <typename LabelT>
+__global__ __launch_bounds__(256) void lmhead_finish_kernel(
+    const uint16_t* __restrict__ hidden, const uint16_t* __restrict__ weight, const LabelT* __restrict__ labels,
+    const float* __restrict__ partial, int64_t n_tokens, int vocab, int hdim, int n_groups, float inv_t,
+    float* __restrict__ logp, float* __restrict__ entropy, float* __restrict__ lse_out) {
+    const int lane = threadIdx.x & 63;
+    const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= n_tokens) return;
+    const float k = inv_t * kLog2e;
+    const int64_t y = (int64_t)labels[t];
+    const bool y_ok = (y >= 0) && (y < (int64_t)vocab);
+    float dot = 0.f;
+    if (y_ok) {
+        const uint16_t* hrow = hidden + t * hdim;
+        const uint16_t* wrow = weight + y * hdim;
+        for (int j = lane * 8; j < hdim; j += 64 * 8) {
+            const u32x4 hv = *reinterpret_cast<const u32x4*>(hrow + j);
+            const u32x4 wv = *reinterpret_cast<const u32x4*>(wrow + j);
+            float a[8], b[8];
+            Elem<MRL_BF16>::unpack(hv, a);
+            Elem<MRL_BF16>::unpack(wv, b);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) dot = __builtin_fmaf(a[i], b[i], dot);
+        }
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) dot += __shfl_xor(dot, off, 64);
+    if (lane == 0) {
+        Stats r = {kMaxInit, 0.f, 0.f};
+        for (int g = 0; g < n_groups; ++g) {
+            const float* p = partial + ((int64_t)g * n_tokens + t) * 4;
+            const Stats o = {p[0], p[1], p[2]};
+            r = merge<true>(r, o, k);
+        }
+        const float lse = (r.m * k + fast_log2(r.s)) * kLn2;
+        logp[t] = (y_ok ? dot * inv_t : r.m * inv_t) - lse;
+        if (entropy) entropy[t] = lse - (r.u / r.s) * inv_t;
+        if (lse_out) lse_out[t] = lse;
+    }
+}
+
+}  // namespace
+
+extern "C" int64_t mrl_lmhead_workspace_bytes(int64_t n_tokens, int64_t vocab) {
+    if (n_tokens < 0 || vocab <= 0) return 0;
+    return (int64_t)MRL_LMHEAD_GROUPS * n_tokens * 4 * (int64_t)sizeof(float);
+}
+
+extern "C" int mrl_lmhead_logprob_fwd(const void* hidden, const void* weight, int64_t n_tokens, int64_t vocab,
+                                      int64_t hidden_dim, const void* labels, int labels_dtype,
+                                      float inv_temperature, float* logp, float* entropy, float* lse,
+                                      void* workspace, int64_t workspace_bytes, void* stream) {
+    const char* fn = "mrl_lmhead_logprob_fwd";
+    MRL_REQUIRE(n_tokens >= 0 && vocab > 0 && hidden_dim > 0, MRL_ERR_INVALID_ARG,
+                "%s: n_tokens=%lld vocab=%lld hidden_dim=%lld", fn, (long long)n_tokens, (long long)vocab,
+                (long long)hidden_dim);
+    MRL_REQUIRE(hidden_dim % BK == 0, MRL_ERR_UNSUPPORTED, "%s: hidden_dim=%lld must be a multiple of %d", fn,
+                (long long)hidden_dim, BK);
+    MRL_REQUIRE(vocab <= (1LL << 30) && hidden_dim <= (1LL << 20), MRL_ERR_UNSUPPORTED, "%s: size out of range", fn);
+    MRL_REQUIRE(mrl::int_dtype_bytes(labels_dtype) != 0, MRL_ERR_UNSUPPORTED, "%s: labels dtype %d (want I32 or I64)",
+                fn, labels_dtype);
+    MRL_REQUIRE(inv_temperature > 0.f && inv_temperature < 1.0e6f, MRL_ERR_INVALID_ARG,
+                "%s: inv_temperature=%g must be in (0, 1e6)", fn, (double)inv_temperature);
+    if (n_tokens == 0) return MRL_OK;
+    MRL_REQUIRE(hidden && weight && labels && logp && workspace, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+    MRL_REQUIRE(mrl::aligned(hidden, 16) && mrl::aligned(weight, 16) && mrl::aligned(workspace, 16), MRL_ERR_MISALIGNED,
+                "%s: hidden, weight and workspace must be 16-byte aligned", fn);
+    MRL_REQUIRE(workspace_bytes >= mrl_lmhead_workspace_bytes(n_tokens, vocab), MRL_ERR_INVALID_ARG,
+                "%s: workspace of %lld bytes, need %lld", fn, (long long)workspace_bytes,
+                (long long)mrl_lmhead_workspace_bytes(n_tokens, vocab));
+    const int n_groups = MRL_LMHEAD_GROUPS;
+    const int n_vtiles = (int)((vocab + BV - 1) / BV);
+    const int tiles_per_group = (n_vtiles + n_groups - 1) / n_groups;
+    const int64_t n_ttiles = (n_tokens + BT - 1) / BT;
+    MRL_REQUIRE(n_ttiles * n_groups <= 0x7fffffffLL, MRL_ERR_UNSUPPORTED, "%s: grid too large", fn);
+    hipStream_t s = mrl::as_stream(stream);
+    float* partial = (float*)workspace;
+    // a group without tiles (tiny vocabularies) still writes its neutral partials
+    hipLaunchKernelGGL(lmhead_fwd_kernel, dim3((unsigned)(n_ttiles * n_groups)), dim3(kThreads), 0, s,
+                       (const uint16_t*)hidden, (const uint16_t*)weight, n_tokens, (int)vocab, (int)hidden_dim,
+                       n_groups, tiles_per_group, inv_temperature * kLog2e, partial);
+    int rc = mrl::check_launch(fn);
+    if (rc != MRL_OK) return rc;
+    const dim3 fgrid((unsigned)((n_tokens + 3) / 4)), fblock(256);
+    if (labels_dtype == MRL_I32) {
+        hipLaunchKernelGGL(lmhead_finish_kernel<int32_t>, fgrid, fblock, 0, s, (const uint16_t*)hidden,
+                           (const uint16_t*)weight, (const int32_t*)labels, (const float*)partial, n_tokens, (int)vocab,
+                           (int)hidden_dim, n_groups, inv_temperature, logp, entropy, lse);
+    } else {
+        hipLaunchKernelGGL(lmhead_finish_kernel<int64_t>, fgrid, fblock, 0, s, (const uint16_t*)hidden,
+                           (const uint16_t*)weight, (const int64_t*)labels, (const float*)partial, n_tokens, (int)vocab,
+                           (int)hidden_dim, n_groups, inv_temperature, logp, entropy, lse);
+    }
+    return mrl::check_launch(fn);
+}

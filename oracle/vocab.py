@@ -111,3 +111,13 @@ def logprob_entropy_fp64(logits, labels):
     p = torch.softmax(z, dim=-1)
     ent = lse - (p * z).sum(-1)
     return logp, ent, lse
+
+
+def lmhead_logprob_entropy(hidden, weight, labels, inv_temperature=1.0):
+    """Oracle of the fused lm_head path: the logits are the fp32 product of the bf16 operands
+    (``F.linear`` on the up-cast tensors, no rounding of the logits to bf16), followed by the two
+    functions above.  The reference materialises bf16 logits in ``GPTModel.output_layer`` (external
+    Megatron code) before ``compute_log_probs`` up-casts them; a kernel that never stores the logits
+    has no reason to round them, so the comparison is made on the fp32 product."""
+    logits = torch.nn.functional.linear(hidden.float(), weight.float()) * inv_temperature
+    return compute_log_probs(logits, labels), vocab_parallel_entropy(logits), torch.logsumexp(logits, -1)

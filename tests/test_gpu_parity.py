@@ -737,6 +737,30 @@ def test_fused_sweep_vocab_sizes(dev, dtype, vocab):
     assert (dz.float().cpu() - dz_o).abs().max().item() <= 2 ** -8 * dz_o.abs().max().item() + 1e-9
 
 
+@pytest.mark.parametrize("tokens,vocab,hdim", [(300, 1000, 128), (129, 256, 64), (64, 4096 + 24, 256),
+                                               (517, 2 * 2048 + 256, 3584)])
+def test_lmhead_logprob_forward(dev, tokens, vocab, hdim):
+    """Fused lm_head + log-prob on the bf16 matrix cores against F.linear (fp32) + the vocabulary oracle:
+    ragged token and vocabulary tiles, labels outside the vocabulary, temperature."""
+    gen = torch.Generator().manual_seed(tokens + vocab)
+    h = torch.randn(tokens, hdim, generator=gen).to(torch.bfloat16)
+    w = (torch.randn(vocab, hdim, generator=gen) * (2.0 / hdim ** 0.5)).to(torch.bfloat16)
+    y = torch.randint(0, vocab, (tokens,), generator=gen)
+    y[1] = -1
+    y[2] = vocab
+    for inv_t in (1.0, 1.0 / 0.7):
+        lp_o, h_o, lse_o = o_vocab.lmhead_logprob_entropy(h, w, y, inv_t)
+        lp, ent, lse = mrl.lmhead_logprob(h.to(dev), w.to(dev), y.to(dev), inv_temperature=inv_t)
+        assert lp.shape == (tokens,) and lp.dtype == torch.float32
+        assert (lse.cpu() - lse_o).abs().max().item() < 1e-4
+        assert (lp.cpu() - lp_o).abs().max().item() < 2e-4
+        assert (ent.cpu() - h_o).abs().max().item() < 2e-4
+    lp2, ent2, _ = mrl.lmhead_logprob(h.to(dev).view(1, tokens, hdim), w.to(dev), y.to(dev).view(1, tokens).int(),
+                                      want_entropy=False)
+    assert lp2.shape == (1, tokens) and ent2.abs().sum().item() == 0
+    assert torch.allclose(lp2.view(-1).cpu(), o_vocab.lmhead_logprob_entropy(h, w, y)[0], atol=2e-4)
+
+
 def test_copy_kernel_moves_bytes(dev):
     src = torch.randint(0, 255, (1 << 20,), dtype=torch.uint8, device=dev)
     dst = torch.zeros_like(src)
