@@ -43,8 +43,9 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS) + ["c3fwd"],
-                    help="c3fwd: the fused lm_head + log-prob forward of configs[3] (bf16 MFMA, logits never stored)")
+    ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS) + ["c3fwd", "c3"],
+                    help="c3fwd: the fused lm_head + log-prob forward of configs[3] (bf16 MFMA, logits never stored); "
+                         "c3: configs[3] forward + backward from the hidden states (chunked GEMM -> fused sweep -> GEMMs)")
     ap.add_argument("--tokens", type=int, default=163840, help="rows of the c3fwd workload")
     ap.add_argument("--entropy-coeff", type=float, default=0.001,
                     help="non-zero so that the forward computes entropy and the backward its gradient")
@@ -212,6 +213,78 @@ def run_lmhead(args):
     print(json.dumps(result), flush=True)
 
 
+def run_lmhead_train(args):
+    """configs[3]: GRPO loss as in configs[1] but from hidden [T, 3584] and W [152064, 3584]; backward yields
+    dHidden and dW.  Logits exist for 8192 rows at a time."""
+    import torch
+    import mindspeed_rl_amd as mrl
+    from mindspeed_rl_amd import vocab_ops
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    w = WORKLOADS["c1"]
+    vocab, hdim = w["vocab"], 3584
+    plen, rlen, rewards = make_lengths(torch, w, args.seed)
+    batch = plen.shape[0]
+    seqlens = (plen + rlen).flatten().to(torch.int32)
+    cu = torch.zeros(batch + 1, dtype=torch.int32)
+    cu[1:] = torch.cumsum(seqlens, 0)
+    total, tokens, resp_w = int(cu[-1]), int(rlen.sum()), int(rlen.max())
+    g = torch.Generator(device=dev).manual_seed(args.seed)
+    hidden = torch.randn(1, total, hdim, generator=g, device=dev).to(torch.bfloat16)
+    weight = (torch.randn(vocab, hdim, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    labels = torch.randint(0, vocab, (1, total), generator=g, device=dev)
+    b = {"labels": labels, "responses": torch.zeros(batch, resp_w, dtype=torch.int32, device=dev),
+         "response_length": rlen.to(dev), "prompt_length": plen.to(dev)}
+    seqlens_d, cu_d = seqlens.to(dev), cu.to(dev)
+    rmask = mrl.generate_mask(b["responses"], b["response_length"])
+    b["advantages"], _ = mrl.compute_group_norm_advantage_return(rewards.to(dev), rmask, b["response_length"], w["group"])
+    lp_rows, _, _ = mrl.lmhead_logprob(hidden, weight, labels, want_entropy=False)
+    lp0 = mrl.postprocess_packed_seqs(lp_rows, seqlens_d, cu_d, resp_w, prompt_length=b["prompt_length"])
+    maskf = rmask.to(torch.float32)
+    b["old_log_prob"] = (lp0 + torch.randn(lp0.shape, generator=g, device=dev) * 0.05) * maskf
+    ref_lp = (lp0 + torch.randn(lp0.shape, generator=g, device=dev) * 0.05) * maskf
+
+    def step():
+        h = hidden.detach().requires_grad_()
+        wt = weight.detach().requires_grad_()
+        loss, out = mrl.fused_lmhead_policy_loss(h, wt, b, packed=True, seqlens=seqlens_d, cu_seqlens=cu_d,
+                                                 ref_log_prob=ref_lp, clip_low=0.2, clip_high=0.2,
+                                                 kl_penalty="low_var_kl", kl_coef=0.001,
+                                                 entropy_coeff=args.entropy_coeff)
+        stats = out.cpu().tolist()
+        dh, dw = torch.autograd.grad(loss, [h, wt])
+        return loss, stats, dh, dw
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    vocab_ops.kernel_events = []
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss, stats, dh, dw = step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    events, vocab_ops.kernel_events = vocab_ops.kernel_events, None
+    sweep_ms = sum(s.elapsed_time(e) for (_, s, e, _) in events) / args.steps
+    ms = elapsed * 1e3 / args.steps
+    flops = 6.0 * total * vocab * hdim                       # forward GEMM + dHidden GEMM + dW GEMM
+    tflops = flops / (ms * 1e-3) / 1e12
+    result = {
+        "metric": "tokens/sec for fused lm_head + logprob + GRPO loss fwd+bwd (dHidden, dW); TFLOP/s as % of bf16 dense peak",
+        "value": tokens / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "configs[3]: hidden [%d,3584] x W [152064,3584], GRPO loss as configs[1], logits only for "
+                               "8192 rows at a time" % total, "response_tokens": tokens, "accumulate": "f32",
+                   "gemm": "library (hipBLASLt via torch.mm)", "sweep": "fused_sweep_persistent_kernel in place"},
+        "roofline": {"kernel": "whole step (3 library GEMMs + fused sweeps)", "bound": "mfma", "achieved": tflops,
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
+                     "traffic": None, "flops_per_step": flops, "fused_sweeps_ms_per_step": sweep_ms},
+        "loss": float(loss.detach()), "stats": stats[1:6],
+    }
+    print(json.dumps(result), flush=True)
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -227,6 +300,9 @@ def main():
     _lib.load()
     if args.workload == "c3fwd":
         run_lmhead(args)
+        return
+    if args.workload == "c3":
+        run_lmhead_train(args)
         return
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)

@@ -27,19 +27,21 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int kThreads = 256;
 constexpr int BV = 256;            // vocabulary rows per macro tile
-constexpr int BT = 128;            // tokens per macro tile
+// tokens per macro tile = 64 * kTB: each of the two token wavefronts owns kTB 32-token MFMA blocks
 constexpr int BK = 64;             // k elements per LDS stage
 constexpr int kLdsStride = BK + 8; // bf16 elements per LDS row: 144 bytes, breaks the bank pattern
 constexpr int kChunksPerRow = BK / 8;                          // 16-byte chunks per row and stage
 constexpr int kALoads = BV * kChunksPerRow / kThreads;         // 8 chunks per thread
-constexpr int kBLoads = BT * kChunksPerRow / kThreads;         // 4 chunks per thread
 
-__global__ __launch_bounds__(kThreads, 2) void lmhead_fwd_kernel(
+template <int kTB>
+__global__ __launch_bounds__(kThreads, (kTB <= 2 ? 2 : 1)) void lmhead_fwd_kernel(
     const uint16_t* __restrict__ hidden, const uint16_t* __restrict__ weight, int64_t n_tokens, int vocab, int hdim,
     int n_groups, int tiles_per_group, float k_scale, float* __restrict__ partial) {
     __shared__ __attribute__((aligned(16))) uint16_t As[BV * kLdsStride];
+    constexpr int BT = 64 * kTB;
+    constexpr int kBLoads = BT * kChunksPerRow / kThreads;
     __shared__ __attribute__((aligned(16))) uint16_t Bs[BT * kLdsStride];
-    __shared__ Stats comb[2][2][64];   // [token half][token block][lane % 32 (+32 unused)]
+    __shared__ Stats comb[2][kTB][32];   // [token half][token block][lane % 32]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -63,9 +65,9 @@ __global__ __launch_bounds__(kThreads, 2) void lmhead_fwd_kernel(
         b_off[i] = (int)r * hdim + ld_col * 8;
     }
 
-    Stats st[2];
+    Stats st[kTB];
 #pragma unroll
-    for (int tb = 0; tb < 2; ++tb) st[tb] = {kMaxInit, 0.f, 0.f};
+    for (int tb = 0; tb < kTB; ++tb) st[tb] = {kMaxInit, 0.f, 0.f};
 
     for (int tile = tile_begin; tile < tile_end; ++tile) {
         const int v0 = tile * BV;
@@ -77,11 +79,11 @@ __global__ __launch_bounds__(kThreads, 2) void lmhead_fwd_kernel(
             if (v0 + r >= vocab) r = vocab - 1 - v0;
             a_off[i] = r * hdim + ld_col * 8;
         }
-        floatx16 acc[4][2];
+        floatx16 acc[4][kTB];
 #pragma unroll
         for (int vb = 0; vb < 4; ++vb)
 #pragma unroll
-            for (int tb = 0; tb < 2; ++tb)
+            for (int tb = 0; tb < kTB; ++tb)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) acc[vb][tb][i] = 0.f;
 
@@ -111,17 +113,17 @@ __global__ __launch_bounds__(kThreads, 2) void lmhead_fwd_kernel(
 #pragma unroll
             for (int ks = 0; ks < BK / 16; ++ks) {
                 const int koff = ks * 16 + (lane >> 5) * 8;
-                bf16x8 af[4], bfr[2];
+                bf16x8 af[4], bfr[kTB];
 #pragma unroll
                 for (int vb = 0; vb < 4; ++vb)
                     af[vb] = *reinterpret_cast<const bf16x8*>(&As[(wv * 128 + vb * 32 + (lane & 31)) * kLdsStride + koff]);
 #pragma unroll
-                for (int tb = 0; tb < 2; ++tb)
-                    bfr[tb] = *reinterpret_cast<const bf16x8*>(&Bs[(wt * 64 + tb * 32 + (lane & 31)) * kLdsStride + koff]);
+                for (int tb = 0; tb < kTB; ++tb)
+                    bfr[tb] = *reinterpret_cast<const bf16x8*>(&Bs[(wt * 32 * kTB + tb * 32 + (lane & 31)) * kLdsStride + koff]);
 #pragma unroll
                 for (int vb = 0; vb < 4; ++vb)
 #pragma unroll
-                    for (int tb = 0; tb < 2; ++tb)
+                    for (int tb = 0; tb < kTB; ++tb)
                         acc[vb][tb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[vb], bfr[tb], acc[vb][tb], 0, 0, 0);
             }
         }
@@ -129,7 +131,7 @@ __global__ __launch_bounds__(kThreads, 2) void lmhead_fwd_kernel(
         // online softmax statistics of this tile: a lane holds 64 vocabulary rows of each token column
         const bool ragged = (v0 + BV > vocab);
 #pragma unroll
-        for (int tb = 0; tb < 2; ++tb) {
+        for (int tb = 0; tb < kTB; ++tb) {
             if (ragged) {
 #pragma unroll
                 for (int vb = 0; vb < 4; ++vb)
@@ -155,7 +157,7 @@ __global__ __launch_bounds__(kThreads, 2) void lmhead_fwd_kernel(
 
     // combine the two lane halves (same token, other vocabulary rows), then the two vocabulary wavefronts
 #pragma unroll
-    for (int tb = 0; tb < 2; ++tb) {
+    for (int tb = 0; tb < kTB; ++tb) {
         Stats o;
         o.m = __shfl_xor(st[tb].m, 32, 64);
         o.s = __shfl_xor(st[tb].s, 32, 64);
@@ -164,15 +166,15 @@ __global__ __launch_bounds__(kThreads, 2) void lmhead_fwd_kernel(
     }
     __syncthreads();
     if (wv == 1 && lane < 32) {
-        comb[wt][0][lane] = st[0];
-        comb[wt][1][lane] = st[1];
+#pragma unroll
+        for (int tb = 0; tb < kTB; ++tb) comb[wt][tb][lane] = st[tb];
     }
     __syncthreads();
     if (wv == 0 && lane < 32) {
 #pragma unroll
-        for (int tb = 0; tb < 2; ++tb) {
+        for (int tb = 0; tb < kTB; ++tb) {
             const Stats r = merge<true>(st[tb], comb[wt][tb][lane], k_scale);
-            const int64_t t = t0 + wt * 64 + tb * 32 + lane;
+            const int64_t t = t0 + wt * 32 * kTB + tb * 32 + lane;
             if (t < n_tokens) {
                 float* p = partial + ((int64_t)group * n_tokens + t) * 4;
                 p[0] = r.m;
@@ -259,12 +261,15 @@ extern "C" int mrl_lmhead_logprob_fwd(const void* hidden, const void* weight, in
     const int n_groups = MRL_LMHEAD_GROUPS;
     const int n_vtiles = (int)((vocab + BV - 1) / BV);
     const int tiles_per_group = (n_vtiles + n_groups - 1) / n_groups;
-    const int64_t n_ttiles = (n_tokens + BT - 1) / BT;
+    // 128-token tiles (4x2 MFMA blocks per wavefront, two workgroups per CU); a 256-token tile with the
+    // accumulators in AGPRs measured slower (758 vs 916 TFLOP/s at 32k tokens) and is not instantiated
+    constexpr int kTokenBlocks = 2;
+    const int64_t n_ttiles = (n_tokens + 64 * kTokenBlocks - 1) / (64 * kTokenBlocks);
     MRL_REQUIRE(n_ttiles * n_groups <= 0x7fffffffLL, MRL_ERR_UNSUPPORTED, "%s: grid too large", fn);
     hipStream_t s = mrl::as_stream(stream);
     float* partial = (float*)workspace;
     // a group without tiles (tiny vocabularies) still writes its neutral partials
-    hipLaunchKernelGGL(lmhead_fwd_kernel, dim3((unsigned)(n_ttiles * n_groups)), dim3(kThreads), 0, s,
+    hipLaunchKernelGGL(lmhead_fwd_kernel<kTokenBlocks>, dim3((unsigned)(n_ttiles * n_groups)), dim3(kThreads), 0, s,
                        (const uint16_t*)hidden, (const uint16_t*)weight, n_tokens, (int)vocab, (int)hidden_dim,
                        n_groups, tiles_per_group, inv_temperature * kLog2e, partial);
     int rc = mrl::check_launch(fn);

@@ -8,7 +8,7 @@ from . import _lib
 from .advantage import (FixedKLController, compute_group_norm_advantage_return, dynamic_sampling_keep,
                         dynamic_sampling_keep_mask)
 from .functional import masked_mean, masked_sum
-from .lmhead import lmhead_logprob
+from .lmhead import fused_lmhead_policy_loss, lmhead_logprob
 from .loss import (BaseLossFunc, DAPOActorLossFunc, GRPOActorLossFunc, LossFuncFactory, LossRegister,
                    MultimodalLogProbComputer, PPOActorLossFunc, ReferenceLossFunc, StandardLogProbComputer, fused_logprob_policy_loss, fused_supported,
                    policy_loss)

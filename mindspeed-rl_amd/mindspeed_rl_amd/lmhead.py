@@ -8,7 +8,7 @@ vocabulary sweeps of a GRPO iteration).
 """
 import torch
 
-from . import _lib
+from . import _lib, vocab_ops
 
 # (name, start, end, rows) appended per call when set to a list, like vocab_ops.kernel_events
 kernel_events = None
@@ -53,3 +53,128 @@ def lmhead_logprob(hidden, weight, labels, inv_temperature=1.0, want_entropy=Tru
         kernel_events.append(("mrl_lmhead_logprob_fwd", start, end, n_tokens))
     ent_out = ent.view(lead) if want_entropy else torch.zeros(lead, dtype=torch.float32, device=dev)
     return logp.view(lead), ent_out, lse.view(lead)
+
+
+class _FusedLmHeadLoss(torch.autograd.Function):
+    """(hidden, weight) -> (loss, out[8]) with dHidden and dWeight produced during the forward.
+
+    The rows are processed in chunks: ``logits_c = hidden_c @ weight^T`` (a plain library GEMM),
+    the fused sweep turns the chunk into dlogits in place (one read, one write), then
+    ``dHidden_c = dlogits_c @ weight`` and ``dWeight += dlogits_c^T @ hidden_c`` (library GEMMs,
+    fp32 accumulation across chunks).  Only ``chunk_rows x V`` logits exist at any time."""
+
+    @staticmethod
+    def forward(ctx, hidden, weight, labels, batch, cfg):
+        from .loss import _mask_args
+        dev = _lib.require_device(hidden, weight, labels)
+        hdim = hidden.shape[-1]
+        h2d = hidden.detach().reshape(-1, hdim).contiguous()
+        w = weight.detach().contiguous()
+        n_rows, vocab = h2d.shape[0], w.shape[0]
+        lab = labels.reshape(-1)
+        if lab.dtype not in (torch.int32, torch.int64):
+            lab = lab.to(torch.int64)
+        lab = lab.contiguous()
+        n_seq, width = batch["responses"].shape[0], batch["responses"].shape[-1]
+
+        def f32(t):
+            return None if t is None else t.to(dev).to(torch.float32).contiguous()
+
+        def idx(t):
+            if t.dtype not in (torch.int32, torch.int64):
+                t = t.to(torch.int64)
+            return t.to(dev).reshape(-1).contiguous()
+
+        old, ref, adv = f32(batch.get("old_log_prob")), f32(cfg["ref_log_prob"]), f32(batch.get("advantages"))
+        mask_t, _ = _mask_args(cfg["mask"], batch["response_length"], dev)
+        prompt, resp = idx(batch["prompt_length"]), idx(batch["response_length"])
+        if cfg["packed"]:
+            layout, padded_s = 0, 0
+            seqlens = cfg["seqlens"].to(dev).to(torch.int32).contiguous()
+            cu = cfg["cu"].to(dev).to(torch.int32).contiguous()
+        else:
+            layout, padded_s = 1, hidden.shape[1]
+            seqlens = cu = None
+        row_start = torch.empty(n_seq, dtype=torch.int64, device=dev)
+        row_count = torch.empty(n_seq, dtype=torch.int32, device=dev)
+        seq_msum = torch.empty(n_seq, dtype=torch.float32, device=dev)
+        row_ops = torch.empty(n_rows * 8, dtype=torch.float32, device=dev)
+        row_terms = torch.empty(n_rows * 8, dtype=torch.float32, device=dev)
+        row_sums = torch.empty(max(n_seq, 1) * 8, dtype=torch.float32, device=dev)
+        out = torch.empty(8, dtype=torch.float32, device=dev)
+        want_ent = cfg["entropy_coeff"] != 0
+        ent = torch.empty(n_rows, dtype=torch.float32, device=dev) if want_ent else None
+        stream = _lib.stream(dev)
+        mdt = _lib.dtype_code(mask_t) if mask_t is not None else _lib.F32
+        pdt, rdt = _lib.dtype_code(prompt), _lib.dtype_code(resp)
+        _lib.call("mrl_fused_loss_prepare", layout, n_seq, width, n_rows, _lib.ptr(seqlens), _lib.ptr(cu), padded_s,
+                  _lib.ptr(prompt), pdt, _lib.ptr(resp), rdt, _lib.ptr(old), _lib.ptr(ref), _lib.ptr(adv),
+                  _lib.ptr(mask_t), mdt, cfg["seq_mean"], _lib.ptr(row_start), _lib.ptr(row_count),
+                  _lib.ptr(seq_msum), _lib.ptr(row_ops), stream)
+        grad_scale = cfg["loss_scale"] * cfg["expected_upstream"]
+        chunk = max(1, min(int(cfg["chunk_rows"]), n_rows))
+        logits = torch.empty((chunk, vocab), dtype=h2d.dtype, device=dev)
+        d_hidden = torch.empty_like(h2d)
+        d_weight32 = torch.zeros((vocab, hdim), dtype=torch.float32, device=dev)
+        w_t = w.t()
+        for c0 in range(0, n_rows, chunk):
+            c1 = min(n_rows, c0 + chunk)
+            rows = c1 - c0
+            z = logits[:rows]
+            torch.mm(h2d[c0:c1], w_t, out=z)                      # plain GEMM (hipBLASLt)
+            vocab_ops._timed_call(
+                "mrl_fused_logprob_loss", rows, dev, _lib.ptr(z), _lib.dtype_code(z), rows, vocab, vocab,
+                lab.data_ptr() + c0 * lab.element_size(), _lib.dtype_code(lab), cfg["inv_temperature"],
+                row_ops.data_ptr() + c0 * 32, 0 if old is None else 1, cfg["clip_lo"], cfg["clip_hi"], cfg["kl_penalty"],
+                cfg["kl_coef"], cfg["entropy_coeff"], grad_scale, _lib.ptr(z), vocab, None,
+                (ent.data_ptr() + c0 * 4) if want_ent else None, row_terms.data_ptr() + c0 * 32, stream)
+            torch.mm(z, w, out=d_hidden[c0:c1])                   # dHidden_c = dlogits_c @ W
+            d_weight32.addmm_(z.t().float(), h2d[c0:c1].float()) if cfg["fp32_dw_gemm"] else \
+                d_weight32.add_(torch.mm(z.t(), h2d[c0:c1]))      # dW += dlogits_c^T @ hidden_c
+        _lib.call("mrl_fused_loss_reduce", _lib.ptr(row_terms), _lib.ptr(row_start), _lib.ptr(row_count), n_seq, width,
+                  _lib.ptr(old), _lib.ptr(ref), _lib.ptr(adv), _lib.ptr(mask_t), mdt, _lib.ptr(resp), rdt,
+                  cfg["clip_lo"], cfg["clip_hi"], cfg["kl_penalty"], cfg["kl_coef"], cfg["entropy_coeff"],
+                  cfg["seq_mean"], cfg["loss_scale"], _lib.ptr(row_sums), _lib.ptr(out), stream)
+        d_weight = d_weight32.to(w.dtype)
+        ctx.save_for_backward(d_hidden, d_weight)
+        ctx.meta = (tuple(hidden.shape), cfg["expected_upstream"])
+        ctx.mark_non_differentiable(out)
+        return out[0].clone(), out
+
+    @staticmethod
+    def backward(ctx, g_loss, _g_out):
+        d_hidden, d_weight = ctx.saved_tensors
+        shape, expected = ctx.meta
+        dev = d_hidden.device
+        upstream = g_loss.to(torch.float32).reshape(1).contiguous()
+        for t in (d_hidden, d_weight):
+            _lib.call("mrl_scale_rows", _lib.ptr(t), _lib.dtype_code(t), t.shape[0], t.shape[1], t.shape[1],
+                      _lib.ptr(upstream), float(expected), _lib.stream(dev))
+        return d_hidden.view(shape), d_weight, None, None, None
+
+
+def fused_lmhead_policy_loss(hidden, weight, batch, *, packed, seqlens=None, cu_seqlens=None, mask=None,
+                             ref_log_prob=None, clip_low, clip_high, kl_penalty=None, kl_coef=0.0, entropy_coeff=0.0,
+                             token_level_loss=True, loss_scale=1.0, inv_temperature=1.0, expected_upstream=1.0,
+                             chunk_rows=8192, fp32_dw_gemm=False):
+    """Policy loss straight from the hidden states: ``hidden`` is packed ``[1, T, H]`` (or padded
+    ``[B, S, H]``) bf16, ``weight`` the ``[V, H]`` bf16 lm_head weight; ``batch`` as for
+    :func:`mindspeed_rl_amd.fused_logprob_policy_loss` (``labels, responses, response_length,
+    prompt_length, advantages``, optional ``old_log_prob``).  Returns ``(loss, out)``; ``backward()``
+    yields dHidden and dWeight.  Full ``[T, V]`` logits are never materialised: at most
+    ``chunk_rows x V`` exist at a time.  ``hidden_dim`` and ``V`` must make 16-byte rows and
+    ``V <= mrl_fused_max_vocab``."""
+    if kl_penalty is None:
+        kl_code = _lib.KL_NONE
+    elif kl_penalty in _lib.KL_BY_NAME:
+        kl_code = _lib.KL_BY_NAME[kl_penalty]
+    else:
+        raise NotImplementedError
+    if hidden.dtype not in (torch.bfloat16, torch.float16) or weight.dtype != hidden.dtype:
+        raise TypeError("hidden and weight must both be bfloat16 (or float16)")
+    cfg = dict(packed=bool(packed), seqlens=seqlens, cu=cu_seqlens, mask=mask, ref_log_prob=ref_log_prob,
+               clip_lo=float(1.0 - clip_low), clip_hi=float(1.0 + clip_high), kl_penalty=kl_code,
+               kl_coef=float(kl_coef), entropy_coeff=float(entropy_coeff), seq_mean=0 if token_level_loss else 1,
+               loss_scale=float(loss_scale), inv_temperature=float(inv_temperature),
+               expected_upstream=float(expected_upstream), chunk_rows=int(chunk_rows), fp32_dw_gemm=bool(fp32_dw_gemm))
+    return _FusedLmHeadLoss.apply(hidden, weight, batch["labels"], batch, cfg)

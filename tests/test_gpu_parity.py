@@ -761,6 +761,41 @@ def test_lmhead_logprob_forward(dev, tokens, vocab, hdim):
     assert torch.allclose(lp2.view(-1).cpu(), o_vocab.lmhead_logprob_entropy(h, w, y)[0], atol=2e-4)
 
 
+@pytest.mark.parametrize("chunk_rows", [64, 8192])
+def test_fused_lmhead_policy_loss(dev, chunk_rows):
+    """Loss and gradients straight from the hidden states (chunked: GEMM -> fused sweep -> two GEMMs).
+    The oracle is fed the SAME bf16 logits the device GEMM produced, so that the comparison is about
+    this pipeline and not about where two GEMM implementations round a logit differently."""
+    gen = torch.Generator().manual_seed(23)
+    vocab, hdim = 2048, 128
+    _, b, kw, _, _ = _make_batch(gen, 2, 4, 5, 24, vocab, torch.bfloat16, 1.0, 2)
+    total = b["labels"].shape[1]
+    h = torch.randn(1, total, hdim, generator=gen).to(torch.bfloat16)
+    w = (torch.randn(vocab, hdim, generator=gen) * (3.0 / hdim ** 0.5)).to(torch.bfloat16)
+    hd, wd = h.to(dev).requires_grad_(), w.to(dev).requires_grad_()
+    logits = torch.mm(hd.detach()[0], wd.detach().t()).cpu()            # what the pipeline's first GEMM yields
+    meta = dict(clip_ratio=0.2, kl_coef=0.01, kl_penalty="low_var_kl", entropy_coeff=0.002)
+    zo = logits.float().view(1, total, vocab).requires_grad_()
+    want, want_stats = o_loss.grpo_compute_loss(zo, b, meta, **kw)
+    (dz,) = torch.autograd.grad(want, zo)
+    dz16 = dz[0].to(torch.bfloat16).float()
+    dh_want = dz16 @ w.float()
+    dw_want = dz16.t() @ h[0].float()
+    bd, kwd = _to_dev(b, dev), _to_dev(kw, dev)
+    loss, out = mrl.fused_lmhead_policy_loss(hd, wd, bd, packed=True, seqlens=kwd["seqlens_in_batch"],
+                                             cu_seqlens=kwd["cu_seqlens_padded"], ref_log_prob=bd["ref_log_prob"],
+                                             clip_low=0.2, clip_high=0.2, kl_penalty="low_var_kl", kl_coef=0.01,
+                                             entropy_coeff=0.002, chunk_rows=chunk_rows)
+    assert abs(loss.item() - want.item()) <= TOL_LOSS_REL * abs(want.item()) + 1e-7
+    host = out.cpu().tolist()
+    for k, v in zip(("actor/pg_clipfrac", "actor/ppo_kl", "actor/kl_loss", "actor/entropy"), host[2:6]):
+        assert abs(v - want_stats[k]) <= TOL_LOSS_REL * abs(want_stats[k]) + 1e-6, k
+    dh, dw = torch.autograd.grad(loss * 0.5, [hd, wd])
+    assert dh.shape == hd.shape and dw.shape == wd.shape and dh.dtype == torch.bfloat16
+    assert (dh.float().cpu()[0] * 2 - dh_want).abs().max().item() <= 2e-2 * dh_want.abs().max().item()
+    assert (dw.float().cpu() * 2 - dw_want).abs().max().item() <= 2e-2 * dw_want.abs().max().item()
+
+
 def test_copy_kernel_moves_bytes(dev):
     src = torch.randint(0, 255, (1 << 20,), dtype=torch.uint8, device=dev)
     dst = torch.zeros_like(src)
