@@ -33,8 +33,9 @@ WORKLOADS = {
                desc="configs[1]: Qwen2.5-7B-shaped GRPO actor step, 16x8 responses, R~U[512,2048], V=152064 bf16"),
     "c0": dict(prompts=4, group=4, r_lo=64, r_hi=256, vocab=32000, dtype="f32", sigma=2.0,
                desc="configs[0]: 4x4 responses, R~U[64,256], V=32000 fp32"),
-    "c4chunk": dict(prompts=1, group=4, r_lo=8192, r_hi=24576, vocab=129280, dtype="bf16", sigma=3.0,
-                    desc="one ~64k-row chunk of configs[4]: V=129280 bf16, DAPO-length responses"),
+    "c4chunk": dict(prompts=1, group=4, r_lo=8192, r_hi=24576, vocab=129280, dtype="bf16", sigma=3.0, loss="dapo",
+                    desc="one ~64k-row chunk of configs[4]: 4 of a kept group's 16 responses, R~U[8192,24576], "
+                         "V=129280 bf16, DAPO clip-higher 0.2/0.28, no KL, token-level loss"),
 }
 
 
@@ -100,7 +101,22 @@ def build_device_batch(torch, mrl, w, plen, rlen, rewards, dev, seed):
     kw = dict(use_remove_padding=True, seqlens_in_batch=seqlens.to(dev), cu_seqlens_padded=cu.to(dev),
               seq_len=int(seqlens.max()))
     rmask = mrl.generate_mask(b["responses"], b["response_length"])
-    adv, _ = mrl.compute_group_norm_advantage_return(rewards.to(dev), rmask, b["response_length"], w["group"])
+    if w.get("loss") == "dapo":
+        # configs[4]: the chunk holds the first rows of a 16-response group; rewards Bernoulli(p), p~Beta(.5,.5);
+        # groups whose rewards are all equal are dropped by the dynamic-sampling filter before the loss
+        full = 16
+        gcpu = torch.Generator().manual_seed(seed + 7)
+        while True:
+            # Beta(1/2, 1/2) is the arcsine law: sin^2(pi u / 2) of a uniform u
+            p = float(torch.sin(torch.rand(1, generator=gcpu) * (3.141592653589793 / 2)) ** 2)
+            group_rewards = torch.bernoulli(torch.full((full, 1), p), generator=gcpu)
+            if mrl.dynamic_sampling_keep_mask(group_rewards.to(dev), full).any().item():
+                break
+        ones = torch.ones(full, 1, device=dev)
+        adv_group, _ = mrl.compute_group_norm_advantage_return(group_rewards.to(dev), ones, ones, full)
+        adv = adv_group[:batch].repeat(1, resp_w) * rmask.to(torch.float32)
+    else:
+        adv, _ = mrl.compute_group_norm_advantage_return(rewards.to(dev), rmask, b["response_length"], w["group"])
     b["advantages"] = adv
     # behaviour / reference log-probs: current + N(0, 0.05)
     ref_fn = mrl.LossFuncFactory.get_instance("ray_grpo", "reference")
@@ -313,9 +329,14 @@ def main():
     vocab = w["vocab"]
     ebytes = logits.element_size()
 
-    f = mrl.LossFuncFactory.get_instance("ray_grpo", "actor")
-    f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.001), "kl_penalty": "low_var_kl",
-                          "entropy_coeff": args.entropy_coeff})
+    if w.get("loss") == "dapo":
+        f = mrl.LossFuncFactory.get_instance("ray_dapo", "actor")
+        f.add_loss_meta_info({"clip_ratio": 0.2, "clip_higher_enable": True, "clip_ratio_low": 0.2,
+                              "clip_ratio_high": 0.28, "token_level_loss": True, "entropy_coeff": args.entropy_coeff})
+    else:
+        f = mrl.LossFuncFactory.get_instance("ray_grpo", "actor")
+        f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.001),
+                              "kl_penalty": "low_var_kl", "entropy_coeff": args.entropy_coeff})
 
     def step():
         z = logits.detach().requires_grad_()
@@ -383,7 +404,7 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": w["desc"], "responses": int(plen.shape[0]), "packed_rows": total, "response_tokens": tokens,
-            "vocab": vocab, "accumulate": "f32", "clip": 0.2, "kl": "low_var_kl 0.001",
+            "vocab": vocab, "accumulate": "f32", "loss_kind": w.get("loss", "grpo: clip 0.2, low_var_kl 0.001"),
             "entropy_coeff": args.entropy_coeff, "loss": "token-mean", "path": args.path,
         },
         "roofline": {

@@ -162,6 +162,32 @@ int mrl_generate_mask(const void* lengths, int lengths_dtype, int64_t batch, int
                       int64_t* out, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Ragged <-> padded experience columns: the wire format either side of the path.  Replace the
+ * per-row Python loops of unpack_pad_experience (mindspeed_rl/trainer/utils/transfer_dock.py:
+ * 1092-1198) and truncate_rows (mindspeed_rl/utils/pad_process.py:144-166).  Bit-exact copies.
+ *
+ * mrl_ragged_layout: cu[0] = 0, cu[i+1] = cu[i] + len_i (int32 [batch+1]); info[0] = cu[batch],
+ * info[1] = max_i len_i rounded up to `multiple` (int64 [2]).  len_i = lengths[i] (I32 / I64), < 0
+ * counts as 0.  With width > 0, len_i follows truncate_rows for rows of that width: clamped to
+ * width; with left_pad a zero length keeps the whole row (python's x[-0:]); and if `rows`
+ * ([batch, width] integers, elem_bytes 4 or 8) is given, 0 where lengths[i] == 0 and
+ * rows[i, 0] == -1.  eff_len (nullable int32 [batch]) receives the len_i.  One workgroup;
+ * batch <= 2^20. */
+int mrl_ragged_layout(const void* lengths, int lengths_dtype, int64_t batch, int64_t multiple,
+                      const void* rows, int elem_bytes, int64_t width, int left_pad, int32_t* eff_len,
+                      int32_t* cu, int64_t* info, void* stream);
+
+/* out[i, d, j] = flat[d * flat_stride + cu[i] + j] for j < cu[i+1] - cu[i], else pad_bits; out is
+ * [batch, first_dim, width] (first_dim = 1 for ordinary columns, 3 for mrope position ids). */
+int mrl_ragged_to_padded(const void* flat, int elem_bytes, int64_t first_dim, int64_t flat_stride,
+                         const int32_t* cu, int64_t batch, int64_t width, uint64_t pad_bits, void* out,
+                         void* stream);
+
+/* flat[cu[i] + j] = padded[i, j] (left_pad = 0) or padded[i, width - len_i + j] (left_pad = 1). */
+int mrl_padded_to_ragged(const void* padded, int elem_bytes, int64_t batch, int64_t width,
+                         const int32_t* cu, int left_pad, int64_t total, void* flat, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Group-relative advantages.  Replaces compute_group_norm_advantage_return
  * (mindspeed_rl/trainer/utils/compute_utils.py:152-191): rows i*group .. (i+1)*group-1 form one
  * group; in fp64, score = (r - mean) / (unbiased_std + 1e-6); cast to fp32; advantages[i, j] =

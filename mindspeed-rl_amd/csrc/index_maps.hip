@@ -234,6 +234,104 @@ __global__ __launch_bounds__(kBlock) void generate_mask_kernel(const void* __res
     out[e] = (j < load_index(lengths, dtype, i)) ? 1 : 0;
 }
 
+
+// ----------------------------------------------------------------------------- ragged <-> padded
+// Exclusive scan of clamped row lengths plus their maximum, by one workgroup:
+//   cu[0] = 0, cu[i+1] = cu[i] + len_i;  info[0] = cu[batch];  info[1] = max_i len_i rounded up to `multiple`.
+// With width > 0, len_i follows truncate_rows: clamped to [0, width]; with left_pad a zero index keeps the
+// whole row (python's x[-0:]); and, if `rows` is given, 0 where index_i == 0 and rows[i, 0] == -1.
+template <typename T>
+__global__ __launch_bounds__(kScanBlock) void ragged_layout_kernel(const void* __restrict__ lengths, int ldtype,
+                                                                   int64_t batch, int64_t multiple,
+                                                                   const T* __restrict__ rows, int64_t width,
+                                                                   int left_pad, int32_t* __restrict__ eff_len,
+                                                                   int32_t* __restrict__ cu, int64_t* __restrict__ info) {
+    __shared__ uint32_t wave_sum[kScanBlock / 64];
+    __shared__ int32_t wave_max[kScanBlock / 64];
+    __shared__ uint32_t carry_s;
+    __shared__ int32_t max_s;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    if (tid == 0) {
+        carry_s = 0;
+        max_s = 0;
+        cu[0] = 0;
+    }
+    __syncthreads();
+    for (int64_t base = 0; base < batch; base += kScanBlock) {
+        const int64_t i = base + tid;
+        int32_t len = 0;
+        if (i < batch) {
+            int64_t n = load_index(lengths, ldtype, i);
+            if (width > 0) {
+                if (rows != nullptr && n == 0 && rows[i * width] == (T)-1) n = 0;
+                else if (left_pad && n == 0) n = width;
+                if (n > width) n = width;
+            }
+            if (n < 0) n = 0;
+            len = (int32_t)n;
+            if (eff_len) eff_len[i] = len;
+        }
+        uint32_t x = (uint32_t)len;
+        int32_t mx = len;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const uint32_t o = __shfl_up(x, off, 64);
+            if (lane >= off) x += o;
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) mx = max(mx, __shfl_xor(mx, off, 64));
+        if (lane == 63) wave_sum[wave] = x;
+        if (lane == 0) wave_max[wave] = mx;
+        __syncthreads();
+        uint32_t prefix = carry_s;
+        for (int w = 0; w < wave; ++w) prefix += wave_sum[w];
+        if (i < batch) cu[i + 1] = (int32_t)(prefix + x);
+        __syncthreads();
+        if (tid == kScanBlock - 1) carry_s = prefix + x;
+        if (tid == 0) {
+            int32_t m = max_s;
+            for (int w = 0; w < kScanBlock / 64; ++w) m = max(m, wave_max[w]);
+            max_s = m;
+        }
+        __syncthreads();
+    }
+    if (tid == 0) {
+        info[0] = (int64_t)(int32_t)carry_s;
+        int64_t m = max_s;
+        if (multiple > 1) m = (m + multiple - 1) / multiple * multiple;
+        info[1] = m;
+    }
+}
+
+// out[i, d, j] = flat[d, cu[i] + j] for j < len_i, pad elsewhere (unpack_pad_experience)
+template <typename T>
+__global__ __launch_bounds__(kBlock) void ragged_to_padded_kernel(const T* __restrict__ flat, int64_t first_dim,
+                                                                  int64_t flat_stride, const int32_t* __restrict__ cu,
+                                                                  int64_t width, T pad, int64_t n_out,
+                                                                  T* __restrict__ out) {
+    const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (e >= n_out) return;
+    const int64_t j = e % width;
+    const int64_t d = (e / width) % first_dim;
+    const int64_t i = e / (width * first_dim);
+    const int64_t lo = cu[i], n = (int64_t)cu[i + 1] - lo;
+    out[e] = j < n ? flat[d * flat_stride + lo + j] : pad;
+}
+
+// flat[cu[i] + j] = padded[i, j] (or padded[i, width - len_i + j] when the rows are left-padded)
+template <typename T>
+__global__ __launch_bounds__(kBlock) void padded_to_ragged_kernel(const T* __restrict__ padded, int batch,
+                                                                  int64_t width, const int32_t* __restrict__ cu,
+                                                                  int left_pad, int64_t total, T* __restrict__ flat) {
+    const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (t >= total) return;
+    const int i = find_sequence(cu, batch, t);
+    const int64_t j = t - cu[i];
+    const int64_t n = (int64_t)cu[i + 1] - cu[i];
+    flat[t] = padded[(int64_t)i * width + (left_pad ? width - n + j : j)];
+}
+
 inline unsigned blocks_for(int64_t n) { return (unsigned)((n + kBlock - 1) / kBlock); }
 
 int check_elems(const char* fn, int64_t n) {
@@ -415,5 +513,79 @@ extern "C" int mrl_generate_mask(const void* lengths, int lengths_dtype, int64_t
     MRL_REQUIRE(mrl::aligned(out, 8), MRL_ERR_MISALIGNED, "%s: out misaligned", fn);
     hipLaunchKernelGGL(generate_mask_kernel, dim3(blocks_for(n_out)), dim3(kBlock), 0, mrl::as_stream(stream),
                        lengths, lengths_dtype, width, n_out, out);
+    return mrl::check_launch(fn);
+}
+
+extern "C" int mrl_ragged_layout(const void* lengths, int lengths_dtype, int64_t batch, int64_t multiple,
+                                 const void* rows, int elem_bytes, int64_t width, int left_pad, int32_t* eff_len,
+                                 int32_t* cu, int64_t* info, void* stream) {
+    const char* fn = "mrl_ragged_layout";
+    MRL_REQUIRE(batch >= 0 && batch <= (1LL << 20), MRL_ERR_INVALID_ARG, "%s: batch=%lld out of [0, 2^20]", fn,
+                (long long)batch);
+    MRL_REQUIRE(multiple >= 1, MRL_ERR_INVALID_ARG, "%s: multiple=%lld", fn, (long long)multiple);
+    MRL_REQUIRE(mrl::int_dtype_bytes(lengths_dtype) != 0, MRL_ERR_UNSUPPORTED, "%s: lengths dtype %d (want I32 or I64)",
+                fn, lengths_dtype);
+    MRL_REQUIRE(cu != nullptr && info != nullptr && (batch == 0 || lengths != nullptr), MRL_ERR_INVALID_ARG,
+                "%s: NULL pointer", fn);
+    MRL_REQUIRE(width >= 0, MRL_ERR_INVALID_ARG, "%s: width=%lld", fn, (long long)width);
+    MRL_REQUIRE(rows == nullptr || ((elem_bytes == 4 || elem_bytes == 8) && width >= 1), MRL_ERR_UNSUPPORTED,
+                "%s: rows need 4- or 8-byte elements and width >= 1", fn);
+    hipStream_t s = mrl::as_stream(stream);
+    if (rows != nullptr && elem_bytes == 8) {
+        hipLaunchKernelGGL(ragged_layout_kernel<int64_t>, dim3(1), dim3(kScanBlock), 0, s, lengths, lengths_dtype, batch,
+                           multiple, (const int64_t*)rows, width, left_pad, eff_len, cu, info);
+    } else {
+        hipLaunchKernelGGL(ragged_layout_kernel<int32_t>, dim3(1), dim3(kScanBlock), 0, s, lengths, lengths_dtype, batch,
+                           multiple, (const int32_t*)rows, width, left_pad, eff_len, cu, info);
+    }
+    return mrl::check_launch(fn);
+}
+
+extern "C" int mrl_ragged_to_padded(const void* flat, int elem_bytes, int64_t first_dim, int64_t flat_stride,
+                                    const int32_t* cu, int64_t batch, int64_t width, uint64_t pad_bits, void* out,
+                                    void* stream) {
+    const char* fn = "mrl_ragged_to_padded";
+    MRL_REQUIRE(elem_bytes == 2 || elem_bytes == 4 || elem_bytes == 8, MRL_ERR_UNSUPPORTED,
+                "%s: elem_bytes=%d (want 2, 4 or 8)", fn, elem_bytes);
+    MRL_REQUIRE(batch >= 0 && width >= 0 && first_dim >= 1 && flat_stride >= 0, MRL_ERR_INVALID_ARG,
+                "%s: batch=%lld width=%lld first_dim=%lld", fn, (long long)batch, (long long)width,
+                (long long)first_dim);
+    const int64_t n_out = batch * first_dim * width;
+    int rc = check_elems(fn, n_out);
+    if (rc != MRL_OK) return rc;
+    if (n_out == 0) return MRL_OK;
+    MRL_REQUIRE(out && cu && (flat || flat_stride == 0), MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+    hipStream_t s = mrl::as_stream(stream);
+    const dim3 grid(blocks_for(n_out)), block(kBlock);
+#define MRL_R2P(T)                                                                                             \
+    hipLaunchKernelGGL(ragged_to_padded_kernel<T>, grid, block, 0, s, (const T*)flat, first_dim, flat_stride, cu, \
+                       width, (T)pad_bits, n_out, (T*)out)
+    if (elem_bytes == 2) MRL_R2P(uint16_t);
+    else if (elem_bytes == 4) MRL_R2P(uint32_t);
+    else MRL_R2P(uint64_t);
+#undef MRL_R2P
+    return mrl::check_launch(fn);
+}
+
+extern "C" int mrl_padded_to_ragged(const void* padded, int elem_bytes, int64_t batch, int64_t width,
+                                    const int32_t* cu, int left_pad, int64_t total, void* flat, void* stream) {
+    const char* fn = "mrl_padded_to_ragged";
+    MRL_REQUIRE(elem_bytes == 2 || elem_bytes == 4 || elem_bytes == 8, MRL_ERR_UNSUPPORTED,
+                "%s: elem_bytes=%d (want 2, 4 or 8)", fn, elem_bytes);
+    MRL_REQUIRE(batch >= 0 && batch <= (1LL << 20) && width >= 0, MRL_ERR_INVALID_ARG, "%s: batch=%lld width=%lld", fn,
+                (long long)batch, (long long)width);
+    int rc = check_elems(fn, total);
+    if (rc != MRL_OK) return rc;
+    if (total == 0) return MRL_OK;
+    MRL_REQUIRE(padded && cu && flat && batch > 0, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+    hipStream_t s = mrl::as_stream(stream);
+    const dim3 grid(blocks_for(total)), block(kBlock);
+#define MRL_P2R(T)                                                                                              \
+    hipLaunchKernelGGL(padded_to_ragged_kernel<T>, grid, block, 0, s, (const T*)padded, (int)batch, width, cu, left_pad, \
+                       total, (T*)flat)
+    if (elem_bytes == 2) MRL_P2R(uint16_t);
+    else if (elem_bytes == 4) MRL_P2R(uint32_t);
+    else MRL_P2R(uint64_t);
+#undef MRL_P2R
     return mrl::check_launch(fn);
 }

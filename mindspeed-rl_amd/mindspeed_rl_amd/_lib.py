@@ -39,6 +39,9 @@ SIGNATURES = {
     "mrl_window_gather": [_vp, _int, _i64, _i64, _i64, _vp, _int, _i64, ctypes.c_uint64, _vp, _vp],
     "mrl_window_scatter": [_vp, _i64, _i64, _vp, _int, _i64, _vp, _vp],
     "mrl_generate_mask": [_vp, _int, _i64, _i64, _vp, _vp],
+    "mrl_ragged_layout": [_vp, _int, _i64, _i64, _vp, _int, _i64, _int, _vp, _vp, _vp, _vp],
+    "mrl_ragged_to_padded": [_vp, _int, _i64, _i64, _vp, _i64, _i64, ctypes.c_uint64, _vp, _vp],
+    "mrl_padded_to_ragged": [_vp, _int, _i64, _i64, _vp, _int, _i64, _vp, _vp],
     "mrl_group_advantage": [_vp, _int, _i64, _i64, _vp, _int, _i64, _vp, _vp, _vp],
     "mrl_group_keep_mask": [_vp, _int, _i64, _i64, _vp, _vp],
     "mrl_policy_loss_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _int, _vp, _int, _i64, _i64, _f32, _f32, _int, _f32, _f32,

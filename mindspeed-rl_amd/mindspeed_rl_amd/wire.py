@@ -1,0 +1,97 @@
+"""Ragged <-> padded experience columns: the on-wire layout either side of the loss path.
+
+Host-side mirror of ``unpack_pad_experience`` (``mindspeed_rl/trainer/utils/transfer_dock.py:
+1092-1198``) and ``truncate_rows`` (``mindspeed_rl/utils/pad_process.py:144-166``) with the
+reference's signatures.  The reference walks the rows in Python with one or two ``.item()`` calls
+per row; here each column costs one scan launch, one host read of two integers (to size the
+output) and one gather launch.
+"""
+import torch
+
+from . import _lib
+from .packing import _pad_bits
+
+_SCALAR_COLUMNS = ("prompt_length", "response_length", "age")
+
+
+def _index(t):
+    if t.dtype not in (torch.int32, torch.int64):
+        t = t.to(torch.int64)
+    return t.reshape(-1).contiguous()
+
+
+def unpack_pad_experience(batch_data, batch_data_length, pad_id, multiple):
+    """Restores padded ``[B, max_len]`` columns (``[B, D, max_len]`` for 2-D columns such as mrope
+    position ids) from flat packed columns and their per-sample lengths; ``max_len`` is rounded up
+    to ``multiple``; floating columns are padded with 0.0, integer columns with ``pad_id``;
+    ``prompt_length`` / ``response_length`` / ``age`` become ``[B, 1]`` views."""
+    if not batch_data:
+        raise ValueError("ERROR: empty batch_data")
+    if set(batch_data.keys()) != set(batch_data_length.keys()):
+        raise ValueError("ERROR: when unpack, keys from batch_data and batch_data_length dictionaries do not match")
+    out = {}
+    for key, length_list in batch_data_length.items():
+        data = batch_data[key]
+        if key in _SCALAR_COLUMNS:
+            out[key] = data.view(-1, 1)
+            continue
+        dev = _lib.require_device(data)
+        lengths = _index(length_list.to(dev))
+        batch = lengths.numel()
+        cu = torch.empty(batch + 1, dtype=torch.int32, device=dev)
+        info = torch.empty(2, dtype=torch.int64, device=dev)
+        stream = _lib.stream(dev)
+        _lib.call("mrl_ragged_layout", _lib.ptr(lengths), _lib.dtype_code(lengths), batch, int(multiple), None, 0, 0, 0,
+                  None, _lib.ptr(cu), _lib.ptr(info), stream)
+        width = int(info[1].item())              # the one host read per column: sizes the output
+        src = data.contiguous()
+        if src.element_size() not in (2, 4, 8):
+            raise TypeError("unsupported element size %d" % src.element_size())
+        pad = 0.0 if src.is_floating_point() else pad_id
+        if src.dim() > 1:
+            first_dim, stride = src.shape[0], src.shape[1]
+            result = torch.empty((batch, first_dim, width), dtype=src.dtype, device=dev)
+        else:
+            first_dim, stride = 1, src.shape[0]
+            result = torch.empty((batch, width), dtype=src.dtype, device=dev)
+        _lib.call("mrl_ragged_to_padded", _lib.ptr(src), src.element_size(), first_dim, stride, _lib.ptr(cu), batch,
+                  width, _pad_bits(src.dtype, pad), _lib.ptr(result), stream)
+        out[key] = result
+    return out
+
+
+def truncate_rows(tensor, index_tensor, left_pad=False):
+    """``tensor`` ``[mbs, seq_len]`` (4- or 8-byte elements), ``index_tensor`` ``[mbs, 1]``: list of
+    CPU rows ``tensor[i, :index_i]`` (``tensor[i, -index_i:]`` when ``left_pad``), an empty int32
+    row where ``index_i == 0`` and ``tensor[i, 0] == -1``.  One packed device-to-host copy instead
+    of one per row.  Negative indices are treated as 0."""
+    dev = _lib.require_device(tensor)
+    src = tensor.contiguous()
+    if src.element_size() not in (4, 8):
+        raise TypeError("truncate_rows supports 4- and 8-byte elements")
+    batch, width = src.shape
+    idx = _index(index_tensor.to(dev))
+    eff = torch.empty(batch, dtype=torch.int32, device=dev)
+    cu = torch.empty(batch + 1, dtype=torch.int32, device=dev)
+    info = torch.empty(2, dtype=torch.int64, device=dev)
+    stream = _lib.stream(dev)
+    # the -1 marker is an integer convention; float rows are cut by the index alone
+    rows_ptr = _lib.ptr(src) if not src.is_floating_point() else None
+    _lib.call("mrl_ragged_layout", _lib.ptr(idx), _lib.dtype_code(idx), batch, 1, rows_ptr, src.element_size(), width,
+              1 if left_pad else 0, _lib.ptr(eff), _lib.ptr(cu), _lib.ptr(info), stream)
+    total = int(info[0].item())
+    flat = torch.empty(total, dtype=src.dtype, device=dev)
+    _lib.call("mrl_padded_to_ragged", _lib.ptr(src), src.element_size(), batch, width, _lib.ptr(cu),
+              1 if left_pad else 0, total, _lib.ptr(flat), stream)
+    host = flat.cpu()
+    lens = eff.cpu().tolist()
+    first = src[:, 0].cpu().tolist() if not src.is_floating_point() else [0] * batch
+    idx_host = idx.cpu().tolist()
+    rows, lo = [], 0
+    for i, n in enumerate(lens):
+        if idx_host[i] == 0 and first[i] == -1:
+            rows.append(torch.tensor([], dtype=torch.int32))
+        else:
+            rows.append(host[lo:lo + n])
+        lo += n
+    return rows

@@ -8,6 +8,9 @@ Pure integer logic, restated as the per-sequence Python loops the reference uses
 * ``mindspeed_rl/utils/utils.py:57-67``            ``generate_mask``
 * ``mindspeed_rl/models/loss/base_loss_func.py:47-53`` window ``[P-1, P+R-1)``
 
+* ``mindspeed_rl/trainer/utils/transfer_dock.py:1092-1198``  ``unpack_pad_experience``
+* ``mindspeed_rl/utils/pad_process.py:144-166``               ``truncate_rows``
+
 Pinned by the reference-held vectors of ``tests/ut/utils/test_utils.py:22-28`` and
 ``tests/ut/utils/test_pad_process.py:48-62`` and by round-trip / brute-force properties.
 """
@@ -101,3 +104,47 @@ def truncate_middle_and_pad(responses, input_tensor, truncate_lengths, pad_value
 def response_window(prompt_length, response_length):
     """``models/loss/base_loss_func.py:47-53``: ``cat([P, P+R], dim=1) - 1``."""
     return torch.cat([prompt_length, prompt_length + response_length], dim=1) - 1
+
+
+def unpack_pad_experience(batch_data, batch_data_length, pad_id, multiple):
+    """``trainer/utils/transfer_dock.py:1092-1198``: flat packed columns + lengths -> padded columns."""
+    if not batch_data:
+        raise ValueError("ERROR: empty batch_data")
+    if set(batch_data.keys()) != set(batch_data_length.keys()):
+        raise ValueError("ERROR: when unpack, keys from batch_data and batch_data_length dictionaries do not match")
+    out = {}
+    for key, lengths in batch_data_length.items():
+        if key in ("prompt_length", "response_length", "age"):
+            out[key] = batch_data[key].view(-1, 1)
+            continue
+        data = batch_data[key]
+        width = torch.max(lengths).item()
+        if multiple > 1:
+            width = ((width + multiple - 1) // multiple) * multiple
+        fill = 0.0 if data.is_floating_point() else pad_id
+        cum = torch.cat([torch.tensor([0]), torch.cumsum(lengths, 0)])
+        if data.dim() > 1:
+            padded = torch.full((len(lengths), data.shape[0], width), fill, dtype=data.dtype)
+            for i in range(len(lengths)):
+                n = lengths[i]
+                for d in range(data.shape[0]):
+                    padded[i, d, :n] = data[d, cum[i]:cum[i] + n]
+        else:
+            padded = torch.full((len(lengths), width), fill, dtype=data.dtype)
+            for i in range(len(lengths)):
+                padded[i, :lengths[i]] = data[cum[i]:cum[i + 1]]
+        out[key] = padded
+    return out
+
+
+def truncate_rows(tensor, index_tensor, left_pad=False):
+    """``utils/pad_process.py:144-166``: list of CPU rows cut at ``index_tensor``."""
+    rows = []
+    for i in range(tensor.shape[0]):
+        if index_tensor[i].item() == 0 and tensor[i, 0].item() == -1:
+            row = torch.tensor([], dtype=torch.int32).cpu()
+        else:
+            n = index_tensor[i].item()
+            row = tensor[i, -n:].cpu() if left_pad else tensor[i, :n].cpu()
+        rows.append(row)
+    return rows

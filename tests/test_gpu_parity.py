@@ -327,6 +327,45 @@ def test_padded_window_bit_exact(dev, reference_vectors):
     assert torch.equal(gx.cpu(), gx_o)
 
 
+def test_wire_format_bit_exact(dev):
+    """unpack_pad_experience and truncate_rows against the reference's loops (oracle), bit for bit."""
+    gen = torch.Generator().manual_seed(61)
+    batch = 37
+    lens_a = torch.randint(0, 50, (batch,), generator=gen, dtype=torch.int32)
+    lens_b = torch.randint(1, 9, (batch,), generator=gen, dtype=torch.int32)
+    data = {"responses": torch.randint(0, 1000, (int(lens_a.sum()),), generator=gen),
+            "old_log_prob": torch.randn(int(lens_a.sum()), generator=gen),
+            "position_ids": torch.randint(0, 99, (3, int(lens_b.sum())), generator=gen),
+            "response_length": lens_a.clone()}
+    lens = {"responses": lens_a, "old_log_prob": lens_a, "position_ids": lens_b, "response_length": torch.ones(batch, dtype=torch.int32)}
+    for multiple in (1, 8):
+        want = o_pack.unpack_pad_experience(data, lens, -7, multiple)
+        got = mrl.unpack_pad_experience({k: v.to(dev) for k, v in data.items()}, lens, -7, multiple)
+        assert set(got) == set(want)
+        for k in want:
+            assert got[k].dtype == want[k].dtype and got[k].shape == want[k].shape, k
+            assert torch.equal(got[k].cpu(), want[k]), k
+    with pytest.raises(ValueError):
+        mrl.unpack_pad_experience({}, {}, 0, 1)
+    tensor = torch.randint(0, 500, (batch, 40), generator=gen)
+    tensor[3, 0] = -1
+    tensor[4, 0] = -1
+    idx = torch.randint(0, 41, (batch, 1), generator=gen)
+    idx[3] = 0
+    idx[5] = 0
+    for left in (False, True):
+        for cast in (torch.int64, torch.int32):
+            want = o_pack.truncate_rows(tensor.to(cast), idx, left)
+            got = mrl.truncate_rows(tensor.to(cast).to(dev), idx.to(dev), left)
+            assert len(got) == len(want)
+            for a, b in zip(got, want):
+                assert a.dtype == b.dtype and torch.equal(a, b)
+    f = torch.randn(batch, 40, generator=gen)
+    for left in (False, True):
+        for a, b in zip(mrl.truncate_rows(f.to(dev), idx.to(dev), left), o_pack.truncate_rows(f, idx, left)):
+            assert a.dtype == b.dtype and torch.equal(a, b)
+
+
 # --------------------------------------------------------------------------------- advantages
 def test_group_advantage_parity(dev, reference_vectors):
     v = reference_vectors["group_norm_advantage"]

@@ -393,3 +393,29 @@ def test_compute_loss_end_to_end_shapes():
                                             clip_higher_enable=True, clip_ratio_low=0.2, clip_ratio_high=0.28), **kw)
     assert d_stats["actor/kl_loss"] == 0.0 and d_stats["actor/entropy"] == 0.0
     assert oracle.__doc__ and "TEST INFRASTRUCTURE" in oracle.__doc__
+
+
+def test_wire_format_reference_vectors():
+    """truncate_rows vector of the reference (tests/ut/utils/test_pad_process.py:64-72) and the worked example
+    in the docstring of unpack_pad_experience (trainer/utils/transfer_dock.py:1096-1121)."""
+    tensor = torch.tensor([[1, 2, 3, 4], [5, 6, 7, 8], [9, 10, 11, 12]])
+    got = packing.truncate_rows(tensor, torch.tensor([[2], [3], [1]]))
+    assert [r.tolist() for r in got] == [[1, 2], [5, 6, 7], [9]]
+    assert [r.tolist() for r in packing.truncate_rows(tensor, torch.tensor([[2], [0], [1]]), left_pad=True)] == \
+        [[3, 4], [5, 6, 7, 8], [12]]
+    marked = torch.tensor([[-1, 0, 0], [4, 5, 6]])
+    got = packing.truncate_rows(marked, torch.tensor([[0], [2]]))
+    assert got[0].dtype == torch.int32 and got[0].numel() == 0 and got[1].tolist() == [4, 5]
+    data = {"prompts": torch.tensor([1, 1, 1, 2, 2, 2, 2, 3, 3, 3, 4, 4, 4, 4]),
+            "attention_mask": torch.tensor([1, 2, 2, 3, 3, 3, 4, 4, 4, 4])}
+    lens = {"prompts": torch.tensor([3, 4, 3, 4], dtype=torch.int32),
+            "attention_mask": torch.tensor([1, 2, 3, 4], dtype=torch.int32)}
+    out = packing.unpack_pad_experience(data, lens, -1, 8)
+    assert out["prompts"].tolist() == [[1, 1, 1, -1, -1, -1, -1, -1], [2, 2, 2, 2, -1, -1, -1, -1],
+                                       [3, 3, 3, -1, -1, -1, -1, -1], [4, 4, 4, 4, -1, -1, -1, -1]]
+    assert out["attention_mask"].tolist() == [[1, -1, -1, -1, -1, -1, -1, -1], [2, 2, -1, -1, -1, -1, -1, -1],
+                                              [3, 3, 3, -1, -1, -1, -1, -1], [4, 4, 4, 4, -1, -1, -1, -1]]
+    with pytest.raises(ValueError):
+        packing.unpack_pad_experience({}, {}, 0, 1)
+    with pytest.raises(ValueError):
+        packing.unpack_pad_experience(data, {"prompts": lens["prompts"]}, 0, 1)
