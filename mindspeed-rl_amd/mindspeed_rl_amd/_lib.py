@@ -75,7 +75,8 @@ class MrlError(RuntimeError):
 
 
 def library_path():
-    return _build.LIB_PATH
+    """The in-tree library; MRL_LIB_PATH points at another build of the same ABI (for experiments)."""
+    return os.environ.get("MRL_LIB_PATH") or _build.LIB_PATH
 
 
 def load():
