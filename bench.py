@@ -55,7 +55,6 @@ def parse_args():
                          "split: forward sweep, then the backward sweep from the saved logsumexp (2 reads + 1 write)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=2048, help="rows of the CPU baseline sample")
-    ap.add_argument("--copy-ceiling", action="store_true", help="also time the plain copy kernel")
     ap.add_argument("--seed", type=int, default=0)
     return ap.parse_args()
 
@@ -420,20 +419,32 @@ def main():
         "stats": {k: float(v) for k, v in stats.items()},
         "loss": float(loss.detach()),
     }
-    if args.copy_ceiling:
-        n = 8 << 30
-        src = torch.empty(n, dtype=torch.uint8, device=dev)
-        dst = torch.empty(n, dtype=torch.uint8, device=dev)
+    # practical ceilings on this box with the sweeps' access pattern (one workgroup per 152064-entry bf16 row)
+    del dz
+    probe_rows, probe_row_bytes = 32768, 304128
+    nbytes = probe_rows * probe_row_bytes
+    src = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    dst = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    ceilings = {}
+    for mode, name, passes in ((0, "read_GBps", 1), (1, "write_GBps", 1), (2, "copy_GBps", 2)):
         s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         for _ in range(2):
-            _lib.call("mrl_copy_bytes", src.data_ptr(), dst.data_ptr(), n, _lib.stream(dev))
+            _lib.call("mrl_bandwidth_probe", mode, src.data_ptr(), dst.data_ptr(), probe_rows, probe_row_bytes,
+                      _lib.stream(dev))
         s.record()
         for _ in range(5):
-            _lib.call("mrl_copy_bytes", src.data_ptr(), dst.data_ptr(), n, _lib.stream(dev))
+            _lib.call("mrl_bandwidth_probe", mode, src.data_ptr(), dst.data_ptr(), probe_rows, probe_row_bytes,
+                      _lib.stream(dev))
         e.record()
         torch.cuda.synchronize()
-        result["copy_ceiling_GBps"] = 2 * n * 5 / (s.elapsed_time(e) * 1e-3) / 1e9
-        del src, dst
+        ceilings[name] = passes * nbytes * 5 / (s.elapsed_time(e) * 1e-3) / 1e9
+    del src, dst
+    result["measured_ceiling"] = ceilings
+    # a read+write stream of R read bytes and W written bytes cannot beat R/read + W/write on this box
+    for k in kernels.values():
+        k["frac_of_measured_copy"] = k["GBps"] / ceilings["copy_GBps"]
+    result["roofline"]["frac_of_measured_copy_ceiling"] = kernels[dominant]["GBps"] / ceilings["copy_GBps"]
+    dz = None
     del dz
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(torch, w, args.cpu_rows, args.entropy_coeff, args.seed)

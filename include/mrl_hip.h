@@ -346,6 +346,15 @@ int mrl_lmhead_logprob_fwd(const void* hidden, const void* weight, int64_t n_tok
  * bandwidth ceiling next to the 8 TB/s vendor peak.  No counterpart in the reference. */
 int mrl_copy_bytes(const void* src, void* dst, int64_t n_bytes, void* stream);
 
+/* Bandwidth probes with the sweeps' access pattern (one 1024-thread workgroup per row of row_bytes
+ * bytes, a multiple of 16, at most 311 296): mode 0 reads n_rows rows from src (dst: 4 writable
+ * bytes, never written in practice), mode 1 writes n_rows rows to dst, mode 2 copies src to dst with
+ * the whole row in registers (all loads of a workgroup before its stores).  They measure the
+ * practical read / write / copy ceilings that the roofline fractions are also quoted against.  No
+ * counterpart in the reference. */
+int mrl_bandwidth_probe(int mode, const void* src, void* dst, int64_t n_rows, int64_t row_bytes,
+                        void* stream);
+
 #ifdef __cplusplus
 }
 #endif

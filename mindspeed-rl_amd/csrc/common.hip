@@ -33,6 +33,44 @@ __global__ __launch_bounds__(256) void copy_kernel(const u32x4* __restrict__ src
     }
 }
 
+
+// Bandwidth probes with the access pattern of the sweeps: one workgroup of 1024 threads per row of
+// `row_vec` 16-byte vectors.  They give the practical ceilings the kernels are measured against.
+constexpr int kProbeBlock = 1024;
+constexpr int kProbeMaxVec = 19;
+
+// read-only: every vector is loaded and folded into a value that is (never) written
+__global__ __launch_bounds__(kProbeBlock) void probe_read_kernel(const u32x4* __restrict__ src, int64_t row_vec,
+                                                                 unsigned* __restrict__ sink) {
+    const u32x4* row = src + (int64_t)blockIdx.x * row_vec;
+    unsigned acc = 0;
+    for (int64_t i = threadIdx.x; i < row_vec; i += kProbeBlock) {
+        const u32x4 v = __builtin_nontemporal_load(row + i);
+        acc ^= v.x ^ v.y ^ v.z ^ v.w;
+    }
+    if (acc == 0x9e3779b9u) sink[0] = acc;
+}
+
+__global__ __launch_bounds__(kProbeBlock) void probe_write_kernel(u32x4* __restrict__ dst, int64_t row_vec) {
+    u32x4* row = dst + (int64_t)blockIdx.x * row_vec;
+    const u32x4 v = {1u, 2u, 3u, 4u};
+    for (int64_t i = threadIdx.x; i < row_vec; i += kProbeBlock) __builtin_nontemporal_store(v, row + i);
+}
+
+// copy with the whole row in registers: all loads of a workgroup are issued before its stores;
+// range-checked buffer accesses keep the body free of branches
+__global__ __launch_bounds__(kProbeBlock) void probe_copy_kernel(const u32x4* __restrict__ src,
+                                                                 u32x4* __restrict__ dst, int row_vec) {
+    const mrl::rsrc_t s = mrl::make_rsrc(src + (int64_t)blockIdx.x * row_vec, (uint32_t)row_vec * 16u);
+    const mrl::rsrc_t d = mrl::make_rsrc(dst + (int64_t)blockIdx.x * row_vec, (uint32_t)row_vec * 16u);
+    u32x4 v[kProbeMaxVec];
+#pragma unroll
+    for (int q = 0; q < kProbeMaxVec; ++q) v[q] = mrl::buf_load_nt(s, (uint32_t)(q * kProbeBlock + threadIdx.x) * 16u);
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < kProbeMaxVec; ++q) mrl::buf_store_nt(v[q], d, (uint32_t)(q * kProbeBlock + threadIdx.x) * 16u);
+}
+
 }  // namespace
 
 extern "C" int mrl_version(void) { return MRL_VERSION; }
@@ -52,4 +90,30 @@ extern "C" int mrl_copy_bytes(const void* src, void* dst, int64_t n_bytes, void*
     hipLaunchKernelGGL(copy_kernel, dim3((unsigned)blocks), dim3(256), 0, mrl::as_stream(stream),
                        (const u32x4*)src, (u32x4*)dst, n_vec);
     return mrl::check_launch("mrl_copy_bytes");
+}
+
+extern "C" int mrl_bandwidth_probe(int mode, const void* src, void* dst, int64_t n_rows, int64_t row_bytes,
+                                   void* stream) {
+    const char* fn = "mrl_bandwidth_probe";
+    MRL_REQUIRE(mode >= 0 && mode <= 2, MRL_ERR_INVALID_ARG, "%s: mode=%d (0 read, 1 write, 2 copy)", fn, mode);
+    MRL_REQUIRE(n_rows >= 0 && n_rows <= 0x7fffffffLL && row_bytes > 0 && row_bytes % 16 == 0, MRL_ERR_INVALID_ARG,
+                "%s: n_rows=%lld row_bytes=%lld (row_bytes must be a positive multiple of 16)", fn, (long long)n_rows,
+                (long long)row_bytes);
+    MRL_REQUIRE(row_bytes / 16 <= (int64_t)kProbeMaxVec * kProbeBlock, MRL_ERR_UNSUPPORTED,
+                "%s: row_bytes=%lld exceeds %d bytes", fn, (long long)row_bytes, kProbeMaxVec * kProbeBlock * 16);
+    if (n_rows == 0) return MRL_OK;
+    MRL_REQUIRE((mode == 1 || src != nullptr) && dst != nullptr, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+    MRL_REQUIRE(mrl::aligned(src, 16) && mrl::aligned(dst, 16), MRL_ERR_MISALIGNED, "%s: pointers must be 16-byte aligned",
+                fn);
+    hipStream_t s = mrl::as_stream(stream);
+    const dim3 grid((unsigned)n_rows), block(kProbeBlock);
+    const int64_t row_vec = row_bytes / 16;
+    if (mode == 0) {
+        hipLaunchKernelGGL(probe_read_kernel, grid, block, 0, s, (const u32x4*)src, row_vec, (unsigned*)dst);
+    } else if (mode == 1) {
+        hipLaunchKernelGGL(probe_write_kernel, grid, block, 0, s, (u32x4*)dst, row_vec);
+    } else {
+        hipLaunchKernelGGL(probe_copy_kernel, grid, block, 0, s, (const u32x4*)src, (u32x4*)dst, (int)row_vec);
+    }
+    return mrl::check_launch(fn);
 }

@@ -18,6 +18,38 @@ __host__ __device__ inline u32x4 make_u32x4(unsigned a, unsigned b, unsigned c, 
     return v;
 }
 
+// Raw buffer access with hardware range checking: a load at a byte offset at or beyond `bytes`
+// returns zero and a store there is dropped, so the tail of a row needs no branch.  Branch-free
+// bodies matter on gfx9: with a branch around every access the compiler can no longer count the
+// accesses in flight and waits for ALL of them (vmcnt(0)) before each use - and stores count too.
+// `base` must be uniform over the wavefront.  Accesses carry the non-temporal hint.
+#if defined(__HIP_DEVICE_COMPILE__)
+using rsrc_t = __amdgpu_buffer_rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ u32x4 buf_load_nt(rsrc_t r, uint32_t byte_off) {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 2);
+}
+__device__ __forceinline__ void buf_store_nt(u32x4 v, rsrc_t r, uint32_t byte_off) {
+    __builtin_amdgcn_raw_buffer_store_b128(v, r, (int)byte_off, 0, 2);
+}
+// single entries, same cache policy as the vectors
+__device__ __forceinline__ void buf_store_b16(uint16_t v, rsrc_t r, uint32_t byte_off) {
+    __builtin_amdgcn_raw_buffer_store_b16((short)v, r, (int)byte_off, 0, 2);
+}
+__device__ __forceinline__ void buf_store_b32(uint32_t v, rsrc_t r, uint32_t byte_off) {
+    __builtin_amdgcn_raw_buffer_store_b32(v, r, (int)byte_off, 0, 2);
+}
+#else   // the host pass only has to parse the kernels
+struct rsrc_t {};
+__device__ inline rsrc_t make_rsrc(const void*, uint32_t) { return rsrc_t(); }
+__device__ inline u32x4 buf_load_nt(rsrc_t, uint32_t) { return make_u32x4(0, 0, 0, 0); }
+__device__ inline void buf_store_nt(u32x4, rsrc_t, uint32_t) {}
+__device__ inline void buf_store_b16(uint16_t, rsrc_t, uint32_t) {}
+__device__ inline void buf_store_b32(uint32_t, rsrc_t, uint32_t) {}
+#endif
+
 // Stores a printf-style message for mrl_last_error() and returns `code`.
 int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 void clear_error();

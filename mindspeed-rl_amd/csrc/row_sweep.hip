@@ -78,34 +78,177 @@ __device__ __forceinline__ float grad_elem(const RowGrad& g, float z) {
     return e * w;
 }
 
-// Writes dlogits for the vectors this thread holds.
-template <int DT, int NV, bool kEntropy>
-__device__ __forceinline__ void store_grads(const u32x4 (&v)[NV], int n_vec, const RowGrad& g, int y_vec, int y_lane,
-                                            u32x4* __restrict__ ovec) {
-    using E = Elem<DT>;
-    constexpr int kVec = E::kVec;
-    const int tid = threadIdx.x;
+// The kernels are instantiated for NV in {4, 8, 12, 16, 19} vectors per thread and the host picks
+// the smallest NV that holds the row, so the vectors below kFull are complete for every thread;
+// only the last few can reach past the end of the row.
+template <int NV>
+struct Tail {
+    static constexpr int kFull = NV == 19 ? 16 : NV - 4;
+};
+
+// Vector q of a row is addressed through a descriptor of its own (the row from byte q * 16 KiB on,
+// clamped to empty) with the same per-thread byte offset for every q: the descriptors live in
+// scalar registers and cost scalar instructions, where one vector offset per q would cost 19
+// vector registers that the row itself needs.
+struct RowRef {
+    const char* base;   // uniform over the workgroup
+    uint32_t bytes;     // 0: nothing is read (loads return zeros) or written
+};
+
+__device__ __forceinline__ RowRef row_ref(const void* base, uint32_t bytes) {
+    RowRef r = {reinterpret_cast<const char*>(base), bytes};
+    return r;
+}
+
+__device__ __forceinline__ mrl::rsrc_t vec_rsrc(const RowRef& row, int q) {
+    // signed arithmetic on purpose: an unsigned saturating subtraction is selected as a VECTOR
+    // instruction, which would make the descriptor non-uniform
+    const int skip = q * (kBlock * 16);
+    const int rest = (int)row.bytes - skip;
+    return mrl::make_rsrc(row.base + skip, (uint32_t)(rest > 0 ? rest : 0));
+}
+
+// Keeps the instruction scheduler from moving work of one vector across the work of the next: in
+// a fully unrolled, branch-free body it would otherwise unpack many vectors ahead of their use and
+// spill the row.
+__device__ __forceinline__ void vector_fence() { __builtin_amdgcn_sched_barrier(0); }
+
+__device__ __forceinline__ uint32_t lane_offset() { return (uint32_t)threadIdx.x * 16u; }
+
+// All loads of a row, back to back and without a branch: vectors past the end of the row come back
+// as zeros from the range check of the buffer access.
+template <int NV>
+__device__ __forceinline__ void load_row(u32x4 (&v)[NV], const RowRef& src) {
 #pragma unroll
     for (int q = 0; q < NV; ++q) {
-        const int idx = q * kBlock + tid;
-        if (idx < n_vec) {
-            float z[kVec], d[kVec];
-            E::unpack(v[q], z);
-#pragma unroll
-            for (int i = 0; i < kVec; ++i) d[i] = grad_elem<kEntropy>(g, z[i]);
-            if (idx == y_vec) {
-#pragma unroll
-                for (int i = 0; i < kVec; ++i)
-                    if (i == y_lane) d[i] += g.onehot;
-            }
-            __builtin_nontemporal_store(E::pack(d), ovec + idx);
-        }
+        v[q] = mrl::buf_load_nt(vec_rsrc(src, q), lane_offset());
+        vector_fence();     // keeps the requests in this order wherever a row is loaded
     }
 }
 
-__device__ __forceinline__ void zero_row(u32x4* __restrict__ ovec, int n_vec) {
+template <int NV>
+__device__ __forceinline__ void zero_row(const RowRef& dst) {
     const u32x4 zero = {0u, 0u, 0u, 0u};
-    for (int idx = threadIdx.x; idx < n_vec; idx += kBlock) __builtin_nontemporal_store(zero, ovec + idx);
+#pragma unroll
+    for (int q = 0; q < NV; ++q) mrl::buf_store_nt(zero, vec_rsrc(dst, q), lane_offset());
+}
+
+// Online-softmax statistics of the vectors one thread holds.  A vector past the end of the row
+// (zeros from the range-checked load) is processed like any other and its result discarded, which
+// costs three selects on the few vectors that can be affected and keeps the pass free of branches.
+template <int DT, int NV, bool kEntropy>
+__device__ __forceinline__ Stats thread_stats(const u32x4 (&v)[NV], int n_vec, float k) {
+    using E = Elem<DT>;
+    constexpr int kVec = E::kVec;
+    Stats st = {kMaxInit, 0.f, 0.f};
+#pragma unroll
+    for (int q = 0; q < NV; ++q) {
+        float z[kVec];
+        E::unpack(v[q], z);
+        Stats nx = st;
+        float vmax = nx.m;
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) vmax = fmaxf(vmax, z[i]);
+        grow_max<kEntropy>(nx, vmax, k);
+        const float mk = nx.m * k;
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) add_one<kEntropy>(nx, z[i], k, mk);
+        if (q >= Tail<NV>::kFull) {
+            const bool valid = q * kBlock + (int)threadIdx.x < n_vec;
+            st.m = valid ? nx.m : st.m;
+            st.s = valid ? nx.s : st.s;
+            st.u = valid ? nx.u : st.u;
+        } else {
+            st = nx;
+        }
+        // pins the running statistics here: without it the scheduler splits the whole unrolled pass
+        // into one chain per statistic and parks every exponential in scratch memory in between
+        asm volatile("" : "+v"(st.m), "+v"(st.s), "+v"(st.u));
+    }
+    return st;
+}
+
+template <int DT, bool kEntropy>
+__device__ __forceinline__ u32x4 grad_vec(const u32x4& v, const RowGrad& g) {
+    using E = Elem<DT>;
+    constexpr int kVec = E::kVec;
+    // The packed vector is passed through an empty asm statement so that the compiler cannot reuse
+    // the unpacked values of the statistics pass: kept alive across both passes they would be a
+    // second, four times larger copy of the row, and spill.
+    u32x4 x = v;
+    asm volatile("" : "+v"(x));
+    float z[kVec], d[kVec];
+    E::unpack(x, z);
+#pragma unroll
+    for (int i = 0; i < kVec; ++i) d[i] = grad_elem<kEntropy>(g, z[i]);
+    return E::pack(d);
+}
+
+// The label's entry gets the one-hot term on top of the softmax term.  The thread that has just
+// stored the vector holding it re-stores that single entry; for every other thread the byte offset
+// is out of range and the hardware drops the store, so there is no branch here either.  Two stores
+// of one thread to the same address stay in program order.
+template <int DT, bool kEntropy>
+__device__ __forceinline__ void store_label_grad(const RowRef& dst, const RowGrad& g, bool y_ok, int64_t y, float z_y) {
+    using E = Elem<DT>;
+    const bool owner = y_ok && (int)((y / E::kVec) % kBlock) == (int)threadIdx.x;
+    const uint32_t off = owner ? (uint32_t)y * (uint32_t)sizeof(typename E::T) : 0x80000000u;
+    E::buf_store(mrl::make_rsrc(dst.base, dst.bytes), off, grad_elem<kEntropy>(g, z_y) + g.onehot);
+}
+
+struct RowScalars {
+    float lp, ent;
+    Token t;
+    float g_lp, g_h;
+};
+
+template <bool kEntropy>
+__device__ __forceinline__ RowScalars row_scalars(const Stats& tot, float k, float inv_t, bool y_ok, float z_y,
+                                                  const float* __restrict__ ops, int has_old, const Params& p,
+                                                  float grad_scale, float m, float& lse) {
+    RowScalars s;
+    lse = (tot.m * k + fast_log2(tot.s)) * kLn2;
+    s.lp = (y_ok ? z_y * inv_t : tot.m * inv_t) - lse;
+    s.ent = kEntropy ? lse - (tot.u / tot.s) * inv_t : 0.f;
+    s.t = token_terms<true>(s.lp, ops[MRL_OP_OLD], has_old != 0, ops[MRL_OP_REF], ops[MRL_OP_ADV], p);
+    const float inv_tok = ops[MRL_OP_INVTOK];
+    s.g_lp = grad_scale * m * (ops[MRL_OP_WPG] * s.t.d_pg + p.kl_coef * inv_tok * s.t.d_kl);
+    s.g_h = kEntropy ? grad_scale * m * (-p.entropy_coeff * inv_tok) : 0.f;
+    return s;
+}
+
+template <bool kEntropy>
+__device__ __forceinline__ RowGrad row_grad(const RowScalars& s, float k, float inv_t, float lse) {
+    RowGrad g;
+    g.k = k;
+    g.lse2 = lse * kLog2e;
+    g.c0 = kEntropy ? inv_t * (-s.g_lp + s.g_h * (lse - s.ent)) : -s.g_lp * inv_t;
+    g.c1 = kEntropy ? -s.g_h * inv_t * inv_t : 0.f;
+    g.onehot = s.g_lp * inv_t;
+    return g;
+}
+
+__device__ __forceinline__ void write_row_outputs(int64_t r, const RowScalars& s, float m, float* __restrict__ logp,
+                                                  float* __restrict__ entropy, float* __restrict__ row_terms) {
+    if (logp) logp[r] = s.lp;
+    if (entropy) entropy[r] = s.ent;
+    float* out = row_terms + r * S_N;
+    out[S_PG] = s.t.pg * m;
+    out[S_CLIP] = s.t.clipped * m;
+    out[S_PPOKL] = s.t.neg_logr * m;
+    out[S_KL] = s.t.kl * m;
+    out[S_ENT] = s.ent * m;
+    out[S_MASK] = m;
+    out[6] = 0.f;
+    out[7] = 0.f;
+}
+
+__device__ __forceinline__ void write_masked_row_outputs(int64_t r, float* __restrict__ logp,
+                                                         float* __restrict__ entropy, float* __restrict__ row_terms) {
+    if (logp) logp[r] = 0.f;
+    if (entropy) entropy[r] = 0.f;
+#pragma unroll
+    for (int q = 0; q < S_N; ++q) row_terms[r * S_N + q] = 0.f;
 }
 
 template <int DT, int NV, bool kEntropy>
@@ -122,94 +265,54 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_kernel(
     const int64_t r = blockIdx.x;
     const int tid = threadIdx.x;
     const int n_vec = vocab / kVec;
+    const uint32_t row_bytes = (uint32_t)vocab * (uint32_t)sizeof(T);
     const T* row = logits + r * row_stride;
-    u32x4* ovec = reinterpret_cast<u32x4*>(dlogits + r * d_stride);
-    const u32x4* ivec = reinterpret_cast<const u32x4*>(row);
+    const RowRef src = row_ref(row, row_bytes);
+    const RowRef dst = row_ref(dlogits + r * d_stride, row_bytes);
 
     const float* ops = row_ops + r * MRL_ROW_OPS;
     const float m = ops[MRL_OP_MASK];
     if (m == 0.f) {                       // not a response token: no gradient, nothing to read
-        zero_row(ovec, n_vec);
-        if (tid == 0) {
-            if (logp) logp[r] = 0.f;
-            if (entropy) entropy[r] = 0.f;
-#pragma unroll
-            for (int q = 0; q < S_N; ++q) row_terms[r * S_N + q] = 0.f;
-        }
+        zero_row<NV>(dst);
+        if (tid == 0) write_masked_row_outputs(r, logp, entropy, row_terms);
         return;
     }
 
     // the whole row: every load is in flight before the first use
     u32x4 v[NV];
-#pragma unroll
-    for (int q = 0; q < NV; ++q) {
-        const int idx = q * kBlock + tid;
-        if (idx < n_vec) v[q] = __builtin_nontemporal_load(ivec + idx);
-    }
+    load_row<NV>(v, src);
     const int64_t y = load_label(labels, labels_dtype, r);
     const bool y_ok = (y >= 0) && (y < (int64_t)vocab);
-    const float z_y = y_ok ? E::load(row + y) : 0.f;
-    const float old_lp = ops[MRL_OP_OLD], ref_lp = ops[MRL_OP_REF], adv = ops[MRL_OP_ADV];
-    const float w_pg = ops[MRL_OP_WPG], inv_tok = ops[MRL_OP_INVTOK];
+    const float z_y = E::load(row + (y_ok ? y : 0));
 
     const float k = inv_t * kLog2e;
-    Stats st = {kMaxInit, 0.f, 0.f};
-#pragma unroll
-    for (int q = 0; q < NV; ++q) {
-        const int idx = q * kBlock + tid;
-        if (idx < n_vec) {
-            float z[kVec];
-            E::unpack(v[q], z);
-            float vmax = st.m;
-#pragma unroll
-            for (int i = 0; i < kVec; ++i) vmax = fmaxf(vmax, z[i]);
-            grow_max<kEntropy>(st, vmax, k);
-            const float mk = st.m * k;
-#pragma unroll
-            for (int i = 0; i < kVec; ++i) add_one<kEntropy>(st, z[i], k, mk);
-        }
-    }
+    const Stats st = thread_stats<DT, NV, kEntropy>(v, n_vec, k);
     const Stats tot = block_reduce_1024<kEntropy>(st, k, lds);
 
     // row scalars, computed redundantly by every thread (uniform values)
-    const float lse = (tot.m * k + fast_log2(tot.s)) * kLn2;
-    const float lp = (y_ok ? z_y * inv_t : tot.m * inv_t) - lse;
-    const float ent = kEntropy ? lse - (tot.u / tot.s) * inv_t : 0.f;
-    const Token t = token_terms<true>(lp, old_lp, has_old != 0, ref_lp, adv, p);
-    const float g_lp = grad_scale * m * (w_pg * t.d_pg + p.kl_coef * inv_tok * t.d_kl);
-    const float g_h = kEntropy ? grad_scale * m * (-p.entropy_coeff * inv_tok) : 0.f;
+    float lse;
+    const RowScalars s = row_scalars<kEntropy>(tot, k, inv_t, y_ok, z_y, ops, has_old, p, grad_scale, m, lse);
+    if (tid == 0) write_row_outputs(r, s, m, logp, entropy, row_terms);
 
-    if (g_lp == 0.f && g_h == 0.f) {
-        zero_row(ovec, n_vec);
+    if (s.g_lp == 0.f && s.g_h == 0.f) {
+        zero_row<NV>(dst);
     } else {
-        RowGrad g;
-        g.k = k;
-        g.lse2 = lse * kLog2e;
-        g.c0 = kEntropy ? inv_t * (-g_lp + g_h * (lse - ent)) : -g_lp * inv_t;
-        g.c1 = kEntropy ? -g_h * inv_t * inv_t : 0.f;
-        g.onehot = g_lp * inv_t;
-        store_grads<DT, NV, kEntropy>(v, n_vec, g, y_ok ? (int)(y / kVec) : -1, y_ok ? (int)(y % kVec) : 0, ovec);
-    }
-    if (tid == 0) {
-        if (logp) logp[r] = lp;
-        if (entropy) entropy[r] = ent;
-        float* out = row_terms + r * S_N;
-        out[S_PG] = t.pg * m;
-        out[S_CLIP] = t.clipped * m;
-        out[S_PPOKL] = t.neg_logr * m;
-        out[S_KL] = t.kl * m;
-        out[S_ENT] = ent * m;
-        out[S_MASK] = m;
-        out[6] = 0.f;
-        out[7] = 0.f;
+        const RowGrad g = row_grad<kEntropy>(s, k, inv_t, lse);
+#pragma unroll
+        for (int q = 0; q < NV; ++q) {
+            mrl::buf_store_nt(grad_vec<DT, kEntropy>(v[q], g), vec_rsrc(dst, q), lane_offset());
+            vector_fence();
+        }
+        store_label_grad<DT, kEntropy>(dst, g, y_ok, y, z_y);
     }
 }
 
-// Persistent variant of the fused sweep: one workgroup per CU walks rows r, r + grid, ... and, while
-// it turns the registers of row r into dlogits, refills each register with the same vector of its
-// NEXT row as soon as the store has been issued.  The loads of row r+grid are therefore in flight
-// during the gradient pass of row r, and the statistics pass of the next row starts on data that
-// has already arrived - the register file never has to hold two rows.
+// Persistent variant of the fused sweep: one workgroup per CU walks rows r, r + grid, ... and, once
+// it has turned the registers of row r into dlogits, refills them with its NEXT row.  The loads of
+// row r+grid are in flight while the row's scalars are written and the loop turns over, and the
+// statistics pass of the next row starts on its first vectors while the last are still arriving -
+// the register file never has to hold two rows.  With kInterleave each register is refilled right
+// after its own store instead of after the last store.
 template <int DT, int NV, bool kEntropy, bool kInterleave>
 __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
     const typename Elem<DT>::T* logits, int64_t row_stride, int vocab, int64_t n_rows,
@@ -223,126 +326,81 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
 
     const int tid = threadIdx.x;
     const int n_vec = vocab / kVec;
+    const uint32_t row_bytes = (uint32_t)vocab * (uint32_t)sizeof(T);
     const float k = inv_t * kLog2e;
     const int64_t step = gridDim.x;
 
+    // A row that is not a response token is never read: its descriptor gets zero bytes, so the
+    // (unconditional) loads return zeros without touching memory.  The label of a row and the logit
+    // at the label are requested BEFORE the row itself: loads return in order, so a request behind
+    // the row could only be used once the whole row has arrived.
     u32x4 v[NV];
     int64_t r = blockIdx.x;
-    bool loaded = false;                    // v holds row r
-    if (r < n_rows && row_ops[r * MRL_ROW_OPS + MRL_OP_MASK] != 0.f) {
-        const u32x4* ivec = reinterpret_cast<const u32x4*>(logits + r * row_stride);
-#pragma unroll
-        for (int q = 0; q < NV; ++q) {
-            const int idx = q * kBlock + tid;
-            if (idx < n_vec) v[q] = __builtin_nontemporal_load(ivec + idx);
-        }
-        loaded = true;
+    int64_t y = 0;
+    uint32_t zy_bits = 0;                   // the logit at the label as loaded; converted where it is used
+    if (r < n_rows) {
+        const bool live = row_ops[r * MRL_ROW_OPS + MRL_OP_MASK] != 0.f;
+        const T* row = logits + r * row_stride;
+        y = load_label(labels, labels_dtype, r);
+        zy_bits = E::load_bits(row + ((y >= 0 && y < (int64_t)vocab) ? y : 0));
+        vector_fence();
+        load_row<NV>(v, row_ref(row, live ? row_bytes : 0u));
     }
     for (; r < n_rows; r += step) {
-        const T* row = logits + r * row_stride;
-        u32x4* ovec = reinterpret_cast<u32x4*>(dlogits + r * d_stride);
+        const RowRef dst = row_ref(dlogits + r * d_stride, row_bytes);
         const float* ops = row_ops + r * MRL_ROW_OPS;
         const float m = ops[MRL_OP_MASK];
+        const bool y_ok = (y >= 0) && (y < (int64_t)vocab);
         const int64_t r2 = r + step;
-        const bool next_live = (r2 < n_rows) && (row_ops[r2 * MRL_ROW_OPS + MRL_OP_MASK] != 0.f);
-        const u32x4* nvec = reinterpret_cast<const u32x4*>(logits + (next_live ? r2 : r) * row_stride);
+        const bool has_next = r2 < n_rows;
+        const int64_t rn = has_next ? r2 : r;
+        const bool next_live = has_next && (row_ops[rn * MRL_ROW_OPS + MRL_OP_MASK] != 0.f);
+        const T* nrow = logits + rn * row_stride;
+        const RowRef nxt = row_ref(nrow, next_live ? row_bytes : 0u);
+        const int64_t y_next = load_label(labels, labels_dtype, rn);
+        const T* zy_next_ptr = nrow + ((y_next >= 0 && y_next < (int64_t)vocab) ? y_next : 0);
+        uint32_t zy_next = 0;
 
-        bool wrote = false;                 // dlogits of row r written (and the next row prefetched) in the gradient pass
+        bool wrote = false;                 // dlogits of row r written and the next row requested
         if (m != 0.f) {
-            const int64_t y = load_label(labels, labels_dtype, r);
-            const bool y_ok = (y >= 0) && (y < (int64_t)vocab);
-            const float z_y = y_ok ? E::load(row + y) : 0.f;
-            Stats st = {kMaxInit, 0.f, 0.f};
-#pragma unroll
-            for (int q = 0; q < NV; ++q) {
-                const int idx = q * kBlock + tid;
-                if (idx < n_vec) {
-                    float z[kVec];
-                    E::unpack(v[q], z);
-                    float vmax = st.m;
-#pragma unroll
-                    for (int i = 0; i < kVec; ++i) vmax = fmaxf(vmax, z[i]);
-                    grow_max<kEntropy>(st, vmax, k);
-                    const float mk = st.m * k;
-#pragma unroll
-                    for (int i = 0; i < kVec; ++i) add_one<kEntropy>(st, z[i], k, mk);
-                }
-            }
+            const float z_y = E::from_bits(zy_bits);
+            const Stats st = thread_stats<DT, NV, kEntropy>(v, n_vec, k);
             const Stats tot = block_reduce_1024<kEntropy>(st, k, lds);
-            const float lse = (tot.m * k + fast_log2(tot.s)) * kLn2;
-            const float lp = (y_ok ? z_y * inv_t : tot.m * inv_t) - lse;
-            const float ent = kEntropy ? lse - (tot.u / tot.s) * inv_t : 0.f;
-            const Token t = token_terms<true>(lp, ops[MRL_OP_OLD], has_old != 0, ops[MRL_OP_REF], ops[MRL_OP_ADV], p);
-            const float inv_tok = ops[MRL_OP_INVTOK];
-            const float g_lp = grad_scale * m * (ops[MRL_OP_WPG] * t.d_pg + p.kl_coef * inv_tok * t.d_kl);
-            const float g_h = kEntropy ? grad_scale * m * (-p.entropy_coeff * inv_tok) : 0.f;
-            if (g_lp != 0.f || g_h != 0.f) {
-                RowGrad g;
-                g.k = k;
-                g.lse2 = lse * kLog2e;
-                g.c0 = kEntropy ? inv_t * (-g_lp + g_h * (lse - ent)) : -g_lp * inv_t;
-                g.c1 = kEntropy ? -g_h * inv_t * inv_t : 0.f;
-                g.onehot = g_lp * inv_t;
-                const int y_vec = y_ok ? (int)(y / kVec) : -1;
-                const int y_lane = y_ok ? (int)(y % kVec) : 0;
+            float lse;
+            const RowScalars s = row_scalars<kEntropy>(tot, k, inv_t, y_ok, z_y, ops, has_old, p, grad_scale, m, lse);
+            if (tid == 0) write_row_outputs(r, s, m, logp, entropy, row_terms);
+            if (s.g_lp != 0.f || s.g_h != 0.f) {
+                const RowGrad g = row_grad<kEntropy>(s, k, inv_t, lse);
+                if (kInterleave) {
+                    zy_next = E::load_bits(zy_next_ptr);
+                    vector_fence();
+                }
 #pragma unroll
                 for (int q = 0; q < NV; ++q) {
-                    const int idx = q * kBlock + tid;
-                    if (idx < n_vec) {
-                        float z[kVec], d[kVec];
-                        E::unpack(v[q], z);
-#pragma unroll
-                        for (int i = 0; i < kVec; ++i) d[i] = grad_elem<kEntropy>(g, z[i]);
-                        if (idx == y_vec) {
-#pragma unroll
-                            for (int i = 0; i < kVec; ++i)
-                                if (i == y_lane) d[i] += g.onehot;
-                        }
-                        __builtin_nontemporal_store(E::pack(d), ovec + idx);
-                        if (kInterleave && next_live) v[q] = __builtin_nontemporal_load(nvec + idx);   // refill
-                    }
+                    mrl::buf_store_nt(grad_vec<DT, kEntropy>(v[q], g), vec_rsrc(dst, q), lane_offset());
+                    if (kInterleave) v[q] = mrl::buf_load_nt(vec_rsrc(nxt, q), lane_offset());
+                    vector_fence();
                 }
-                if (!kInterleave && next_live) {
-#pragma unroll
-                    for (int q = 0; q < NV; ++q) {
-                        const int idx = q * kBlock + tid;
-                        if (idx < n_vec) v[q] = __builtin_nontemporal_load(nvec + idx);
-                    }
+                store_label_grad<DT, kEntropy>(dst, g, y_ok, y, z_y);
+                if (!kInterleave) {
+                    zy_next = E::load_bits(zy_next_ptr);
+                    vector_fence();
+                    load_row<NV>(v, nxt);
                 }
                 wrote = true;
             }
-            if (tid == 0) {
-                if (logp) logp[r] = lp;
-                if (entropy) entropy[r] = ent;
-                float* out = row_terms + r * S_N;
-                out[S_PG] = t.pg * m;
-                out[S_CLIP] = t.clipped * m;
-                out[S_PPOKL] = t.neg_logr * m;
-                out[S_KL] = t.kl * m;
-                out[S_ENT] = ent * m;
-                out[S_MASK] = m;
-                out[6] = 0.f;
-                out[7] = 0.f;
-            }
         } else if (tid == 0) {
-            if (logp) logp[r] = 0.f;
-            if (entropy) entropy[r] = 0.f;
-#pragma unroll
-            for (int q = 0; q < S_N; ++q) row_terms[r * S_N + q] = 0.f;
+            write_masked_row_outputs(r, logp, entropy, row_terms);
         }
-        if (!wrote) {                       // no gradient for this row: zeros, then fetch the next row plainly
-            zero_row(ovec, n_vec);
-            if (next_live) {
-#pragma unroll
-                for (int q = 0; q < NV; ++q) {
-                    const int idx = q * kBlock + tid;
-                    if (idx < n_vec) v[q] = __builtin_nontemporal_load(nvec + idx);
-                }
-            }
+        if (!wrote) {                       // no gradient for this row: zeros, then fetch the next row
+            zero_row<NV>(dst);
+            zy_next = E::load_bits(zy_next_ptr);
+            vector_fence();
+            load_row<NV>(v, nxt);
         }
-        loaded = next_live;
+        y = y_next;
+        zy_bits = zy_next;
     }
-    (void)loaded;
 }
 
 // Conditional in-place rescale: multiplies every row by upstream/assumed unless that ratio is 1
@@ -396,6 +454,15 @@ bool persistent_enabled() {
     return on;
 }
 
+// MRL_SWEEP_INTERLEAVE=1 refills each register right after its own store (a tuning switch).
+bool interleave_enabled() {
+    static const bool on = [] {
+        const char* e = getenv("MRL_SWEEP_INTERLEAVE");
+        return e && e[0] == '1';
+    }();
+    return on;
+}
+
 template <int DT, int NV>
 int launch_fused(const mrl::FusedArgs& a) {
     using T = typename Elem<DT>::T;
@@ -404,12 +471,15 @@ int launch_fused(const mrl::FusedArgs& a) {
     const int cus = persistent_enabled() ? cu_count() : 0;
     if (cus > 0 && a.n_rows > 2 * (int64_t)cus) {
         const dim3 pgrid((unsigned)cus);
-#define MRL_FUSEDP_LAUNCH(ENT)                                                                                     \
-    hipLaunchKernelGGL((fused_sweep_persistent_kernel<DT, NV, ENT, false>), pgrid, block, 0, a.stream, (const T*)a.logits, \
+#define MRL_FUSEDP_LAUNCH(ENT, IL)                                                                                \
+    hipLaunchKernelGGL((fused_sweep_persistent_kernel<DT, NV, ENT, IL>), pgrid, block, 0, a.stream, (const T*)a.logits, \
                        a.row_stride, (int)a.vocab, a.n_rows, a.labels, a.labels_dtype, a.inv_t, a.row_ops,         \
                        a.has_old, p, a.grad_scale, (T*)a.dlogits, a.d_stride, a.logp, a.entropy, a.row_terms)
-        if (a.with_entropy) MRL_FUSEDP_LAUNCH(true);
-        else MRL_FUSEDP_LAUNCH(false);
+        const bool il = interleave_enabled();
+        if (a.with_entropy && il) MRL_FUSEDP_LAUNCH(true, true);
+        else if (a.with_entropy) MRL_FUSEDP_LAUNCH(true, false);
+        else if (il) MRL_FUSEDP_LAUNCH(false, true);
+        else MRL_FUSEDP_LAUNCH(false, false);
 #undef MRL_FUSEDP_LAUNCH
         return mrl::check_launch("mrl_fused_logprob_loss");
     }

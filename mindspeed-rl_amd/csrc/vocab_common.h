@@ -33,7 +33,14 @@ struct Elem<MRL_F32> {
                           __float_as_uint(z[3]));
     }
     static __device__ __forceinline__ float load(const T* p) { return *p; }
+    // the entry as loaded and its conversion, separately: a kernel that requests an entry long
+    // before it needs it converts at the use, so that nothing waits at the request
+    static __device__ __forceinline__ uint32_t load_bits(const T* p) { return __float_as_uint(*p); }
+    static __device__ __forceinline__ float from_bits(uint32_t b) { return __uint_as_float(b); }
     static __device__ __forceinline__ void store(T* p, float v) { *p = v; }
+    static __device__ __forceinline__ void buf_store(mrl::rsrc_t r, uint32_t byte_off, float v) {
+        mrl::buf_store_b32(__float_as_uint(v), r, byte_off);
+    }
 };
 
 template <>
@@ -57,9 +64,15 @@ struct Elem<MRL_BF16> {
         return mrl::make_u32x4(pack2(z[0], z[1]), pack2(z[2], z[3]), pack2(z[4], z[5]), pack2(z[6], z[7]));
     }
     static __device__ __forceinline__ float load(const T* p) { return __uint_as_float((uint32_t)(*p) << 16); }
+    static __device__ __forceinline__ uint32_t load_bits(const T* p) { return *p; }
+    static __device__ __forceinline__ float from_bits(uint32_t b) { return __uint_as_float(b << 16); }
     static __device__ __forceinline__ void store(T* p, float v) {
         __bf16 h = (__bf16)v;
         *p = __builtin_bit_cast(uint16_t, h);
+    }
+    static __device__ __forceinline__ void buf_store(mrl::rsrc_t r, uint32_t byte_off, float v) {
+        __bf16 h = (__bf16)v;
+        mrl::buf_store_b16(__builtin_bit_cast(uint16_t, h), r, byte_off);
     }
 };
 
@@ -87,9 +100,17 @@ struct Elem<MRL_F16> {
     static __device__ __forceinline__ float load(const T* p) {
         return (float)__builtin_bit_cast(_Float16, *p);
     }
+    static __device__ __forceinline__ uint32_t load_bits(const T* p) { return *p; }
+    static __device__ __forceinline__ float from_bits(uint32_t b) {
+        return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
+    }
     static __device__ __forceinline__ void store(T* p, float v) {
         _Float16 h = (_Float16)v;
         *p = __builtin_bit_cast(uint16_t, h);
+    }
+    static __device__ __forceinline__ void buf_store(mrl::rsrc_t r, uint32_t byte_off, float v) {
+        _Float16 h = (_Float16)v;
+        mrl::buf_store_b16(__builtin_bit_cast(uint16_t, h), r, byte_off);
     }
 };
 

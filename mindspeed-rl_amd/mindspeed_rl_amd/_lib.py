@@ -59,6 +59,7 @@ SIGNATURES = {
     "mrl_lmhead_workspace_bytes": [_i64, _i64],
     "mrl_lmhead_logprob_fwd": [_vp, _vp, _i64, _i64, _i64, _vp, _int, _f32, _vp, _vp, _vp, _vp, _i64, _vp],
     "mrl_copy_bytes": [_vp, _vp, _i64, _vp],
+    "mrl_bandwidth_probe": [_int, _vp, _vp, _i64, _i64, _vp],
 }
 _RESTYPES = {"mrl_last_error": ctypes.c_char_p, "mrl_fused_max_vocab": ctypes.c_int64,
              "mrl_lmhead_workspace_bytes": ctypes.c_int64}
