@@ -26,6 +26,18 @@ struct FusedArgs {
     hipStream_t stream;
 };
 
+struct BwdArgs {
+    const void* logits; int dtype; int64_t n_rows, vocab, row_stride;
+    const void* labels; int labels_dtype; float inv_t;
+    const float* lse; const float* entropy; const float* g_logp; const float* g_entropy;
+    void* dlogits; int64_t d_stride;
+    hipStream_t stream;
+};
+
+// Backward of log-prob / entropy for given per-row upstream gradients, dlogits in the dtype of the
+// logits, one workgroup per row with the row in registers.  Call only if row_sweep_supported().
+int launch_bwd_rows(const BwdArgs& a);
+
 // True if rows of this dtype / vocab / alignment fit the row-in-registers kernels.
 bool row_sweep_supported(int dtype, int64_t vocab, const void* in, int64_t in_stride, const void* out,
                          int64_t out_stride, int64_t n_rows);

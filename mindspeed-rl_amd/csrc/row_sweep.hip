@@ -403,6 +403,124 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
     }
 }
 
+// Backward for given upstream gradients (the split path): the row is loaded into registers in one
+// burst, turned into dlogits and stored in one burst - the access pattern of the copy probe, which
+// a streaming loop of loads and stores does not reach.
+template <int DT, int NV, bool kEntropy>
+__global__ __launch_bounds__(kBlock) void bwd_rows_kernel(
+    const typename Elem<DT>::T* logits, int64_t row_stride, int vocab, const void* __restrict__ labels,
+    int labels_dtype, float inv_t, const float* __restrict__ lse_in, const float* __restrict__ ent_in,
+    const float* __restrict__ g_logp, const float* __restrict__ g_entropy, typename Elem<DT>::T* dlogits,
+    int64_t d_stride) {
+    using E = Elem<DT>;
+    using T = typename E::T;
+    const int64_t r = blockIdx.x;
+    const uint32_t row_bytes = (uint32_t)vocab * (uint32_t)sizeof(T);
+    const T* row = logits + r * row_stride;
+    const RowRef dst = row_ref(dlogits + r * d_stride, row_bytes);
+
+    const float g_lp = g_logp ? g_logp[r] : 0.f;
+    const float g_h = (kEntropy && g_entropy) ? g_entropy[r] : 0.f;
+    if (g_lp == 0.f && g_h == 0.f) {      // nothing flows into this row: zeros, the logits are not read
+        zero_row<NV>(dst);
+        return;
+    }
+    const int64_t y = load_label(labels, labels_dtype, r);
+    const bool y_ok = (y >= 0) && (y < (int64_t)vocab);
+    const uint32_t zy_bits = E::load_bits(row + (y_ok ? y : 0));
+    vector_fence();
+    u32x4 v[NV];
+    load_row<NV>(v, row_ref(row, row_bytes));
+
+    const float lse = lse_in[r];
+    RowGrad g;
+    g.k = inv_t * kLog2e;
+    g.lse2 = lse * kLog2e;
+    g.c0 = kEntropy ? inv_t * (-g_lp + g_h * (lse - ent_in[r])) : -g_lp * inv_t;
+    g.c1 = kEntropy ? -g_h * inv_t * inv_t : 0.f;
+    g.onehot = g_lp * inv_t;
+#pragma unroll
+    for (int q = 0; q < NV; ++q) {
+        mrl::buf_store_nt(grad_vec<DT, kEntropy>(v[q], g), vec_rsrc(dst, q), lane_offset());
+        vector_fence();
+    }
+    store_label_grad<DT, kEntropy>(dst, g, y_ok, y, E::from_bits(zy_bits));
+}
+
+// Persistent form of bwd_rows_kernel: one workgroup per CU walks rows r, r + grid, ... and requests
+// its next row right after the stores of the current one, so that the gradient arithmetic of a row
+// runs while the following row is on its way.
+template <int DT, int NV, bool kEntropy>
+__global__ __launch_bounds__(kBlock) void bwd_rows_persistent_kernel(
+    const typename Elem<DT>::T* logits, int64_t row_stride, int vocab, int64_t n_rows,
+    const void* __restrict__ labels, int labels_dtype, float inv_t, const float* __restrict__ lse_in,
+    const float* __restrict__ ent_in, const float* __restrict__ g_logp, const float* __restrict__ g_entropy,
+    typename Elem<DT>::T* dlogits, int64_t d_stride) {
+    using E = Elem<DT>;
+    using T = typename E::T;
+    const uint32_t row_bytes = (uint32_t)vocab * (uint32_t)sizeof(T);
+    const int64_t step = gridDim.x;
+    auto grad_lp = [&](int64_t r) { return g_logp ? g_logp[r] : 0.f; };
+    auto grad_h = [&](int64_t r) { return (kEntropy && g_entropy) ? g_entropy[r] : 0.f; };
+
+    u32x4 v[NV];
+    int64_t r = blockIdx.x;
+    int64_t y = 0;
+    uint32_t zy_bits = 0;
+    if (r < n_rows) {
+        const bool live = grad_lp(r) != 0.f || grad_h(r) != 0.f;
+        const T* row = logits + r * row_stride;
+        y = load_label(labels, labels_dtype, r);
+        zy_bits = E::load_bits(row + ((y >= 0 && y < (int64_t)vocab) ? y : 0));
+        vector_fence();
+        load_row<NV>(v, row_ref(row, live ? row_bytes : 0u));
+    }
+    for (; r < n_rows; r += step) {
+        const RowRef dst = row_ref(dlogits + r * d_stride, row_bytes);
+        const float g_lp = grad_lp(r), g_h = grad_h(r);
+        const bool y_ok = (y >= 0) && (y < (int64_t)vocab);
+        const int64_t r2 = r + step;
+        const bool has_next = r2 < n_rows;
+        const int64_t rn = has_next ? r2 : r;
+        const bool next_live = has_next && (grad_lp(rn) != 0.f || grad_h(rn) != 0.f);
+        const T* nrow = logits + rn * row_stride;
+        const int64_t y_next = load_label(labels, labels_dtype, rn);
+        const T* zy_next_ptr = nrow + ((y_next >= 0 && y_next < (int64_t)vocab) ? y_next : 0);
+        const RowRef nxt = row_ref(nrow, next_live ? row_bytes : 0u);
+        uint32_t zy_next = 0;
+        bool wrote = false;
+        if (g_lp != 0.f || g_h != 0.f) {
+            const float lse = lse_in[r];
+            RowGrad g;
+            g.k = inv_t * kLog2e;
+            g.lse2 = lse * kLog2e;
+            g.c0 = kEntropy ? inv_t * (-g_lp + g_h * (lse - ent_in[r])) : -g_lp * inv_t;
+            g.c1 = kEntropy ? -g_h * inv_t * inv_t : 0.f;
+            g.onehot = g_lp * inv_t;
+#pragma unroll
+            for (int q = 0; q < NV; ++q) {
+                mrl::buf_store_nt(grad_vec<DT, kEntropy>(v[q], g), vec_rsrc(dst, q), lane_offset());
+                vector_fence();
+            }
+            store_label_grad<DT, kEntropy>(dst, g, y_ok, y, E::from_bits(zy_bits));
+            // the refill is written out on both paths: after a join the compiler would wait for
+            // every store of the row before the first load of the next
+            zy_next = E::load_bits(zy_next_ptr);
+            vector_fence();
+            load_row<NV>(v, nxt);
+            wrote = true;
+        }
+        if (!wrote) {
+            zero_row<NV>(dst);
+            zy_next = E::load_bits(zy_next_ptr);
+            vector_fence();
+            load_row<NV>(v, nxt);
+        }
+        zy_bits = zy_next;
+        y = y_next;
+    }
+}
+
 // Conditional in-place rescale: multiplies every row by upstream/assumed unless that ratio is 1
 // (then every workgroup exits at once; the grid is kept small so that this costs microseconds).
 template <int DT>
@@ -505,9 +623,48 @@ int launch_fused(const mrl::FusedArgs& a) {
 
 template <int DT>
 int fused_by_nv(int nv, const mrl::FusedArgs& a) { MRL_NV_SWITCH(launch_fused, DT, nv, a) }
+
+template <int DT, int NV>
+int launch_bwd_rows_nv(const mrl::BwdArgs& a) {
+    using T = typename Elem<DT>::T;
+    const dim3 block(kBlock);
+    const int cus = persistent_enabled() ? cu_count() : 0;
+    if (cus > 0 && a.n_rows > 2 * (int64_t)cus) {
+        const dim3 pgrid((unsigned)cus);
+#define MRL_BWDP_LAUNCH(ENT)                                                                                      \
+    hipLaunchKernelGGL((bwd_rows_persistent_kernel<DT, NV, ENT>), pgrid, block, 0, a.stream, (const T*)a.logits,  \
+                       a.row_stride, (int)a.vocab, a.n_rows, a.labels, a.labels_dtype, a.inv_t, a.lse, a.entropy, \
+                       a.g_logp, a.g_entropy, (T*)a.dlogits, a.d_stride)
+        if (a.g_entropy != nullptr) MRL_BWDP_LAUNCH(true);
+        else MRL_BWDP_LAUNCH(false);
+#undef MRL_BWDP_LAUNCH
+        return mrl::check_launch("mrl_vocab_logprob_bwd");
+    }
+    const dim3 grid((unsigned)a.n_rows);
+#define MRL_BWDR_LAUNCH(ENT)                                                                                   \
+    hipLaunchKernelGGL((bwd_rows_kernel<DT, NV, ENT>), grid, block, 0, a.stream, (const T*)a.logits, a.row_stride, \
+                       (int)a.vocab, a.labels, a.labels_dtype, a.inv_t, a.lse, a.entropy, a.g_logp, a.g_entropy,   \
+                       (T*)a.dlogits, a.d_stride)
+    if (a.g_entropy != nullptr) MRL_BWDR_LAUNCH(true);
+    else MRL_BWDR_LAUNCH(false);
+#undef MRL_BWDR_LAUNCH
+    return mrl::check_launch("mrl_vocab_logprob_bwd");
+}
+
+template <int DT>
+int bwd_rows_by_nv(int nv, const mrl::BwdArgs& a) { MRL_NV_SWITCH(launch_bwd_rows_nv, DT, nv, a) }
 }  // namespace
 
 namespace mrl {
+
+int launch_bwd_rows(const BwdArgs& a) {
+    const int nv = pick_nv(a.vocab / (16 / float_dtype_bytes(a.dtype)));
+    switch (a.dtype) {
+        case MRL_F32: return bwd_rows_by_nv<MRL_F32>(nv, a);
+        case MRL_BF16: return bwd_rows_by_nv<MRL_BF16>(nv, a);
+        default: return bwd_rows_by_nv<MRL_F16>(nv, a);
+    }
+}
 
 bool row_sweep_supported(int dtype, int64_t vocab, const void* in, int64_t in_stride, const void* out,
                          int64_t out_stride, int64_t n_rows) {

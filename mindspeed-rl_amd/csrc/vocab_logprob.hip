@@ -8,7 +8,10 @@
 // most once per group of kUnroll vectors and only when the running maximum grows, so the steady
 // state costs one convert, one FMA and one v_exp_f32 per element.  Wavefront reduction uses
 // cross-lane shuffles, the four wavefronts combine through LDS.
+#include <stdlib.h>
+
 #include "mrl_internal.h"
+#include "row_sweep.h"
 #include "vocab_common.h"
 
 namespace {
@@ -314,6 +317,15 @@ int launch_bwd(const void* logits, int64_t n_rows, int vocab, int64_t row_stride
     return mrl::check_launch("mrl_vocab_logprob_bwd");
 }
 
+// MRL_BWD_ROWS=0 keeps the streaming backward kernel for every shape (a tuning / debugging switch).
+bool sweep_rows_enabled() {
+    static const bool on = [] {
+        const char* e = getenv("MRL_BWD_ROWS");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
 int check_common(const char* fn, const void* logits, int logits_dtype, int64_t n_rows, int64_t vocab,
                  int64_t row_stride, const void* labels, int labels_dtype, float inv_t) {
     MRL_REQUIRE(n_rows >= 0 && vocab > 0, MRL_ERR_INVALID_ARG, "%s: n_rows=%lld vocab=%lld", fn,
@@ -416,6 +428,13 @@ extern "C" int mrl_vocab_logprob_bwd(const void* logits, int logits_dtype, int64
     }
     hipStream_t s = mrl::as_stream(stream);
     const int v = (int)vocab;
+    // rows that fill a 1024-thread workgroup and fit its register file take the row-in-registers kernel
+    if (dlogits_dtype == logits_dtype && sweep_rows_enabled() && vocab * ib >= 16 * 1024 &&
+        mrl::row_sweep_supported(logits_dtype, vocab, logits, row_stride, dlogits, dlogits_row_stride, n_rows)) {
+        const mrl::BwdArgs a = {logits, logits_dtype, n_rows, vocab, row_stride, labels, labels_dtype, inv_temperature,
+                                lse, entropy, g_logp, g_entropy, dlogits, dlogits_row_stride, s};
+        return mrl::launch_bwd_rows(a);
+    }
 #define MRL_BWD(DI, DO)                                                                                      \
     (labels_dtype == MRL_I32                                                                                 \
          ? launch_bwd<DI, DO, int32_t>(logits, n_rows, v, row_stride, labels, inv_temperature, lse, entropy, \
