@@ -776,6 +776,81 @@ def test_fused_sweep_vocab_sizes(dev, dtype, vocab):
     assert (dz.float().cpu() - dz_o).abs().max().item() <= 2 ** -8 * dz_o.abs().max().item() + 1e-9
 
 
+@pytest.mark.parametrize("dtype,vocab", [(torch.bfloat16, 8200), (torch.float32, 4100), (torch.float16, 40960)])
+def test_persistent_row_sweeps(dev, dtype, vocab):
+    """More rows than twice the CU count: the persistent row-in-registers kernels (one workgroup per
+    CU walking rows) of the split backward and of the fused sweep, with rows that are skipped (no
+    gradient / no response token) next to each other, at the ends and a whole grid stride apart,
+    labels outside the vocabulary, a row tail that does not fill the last vector of every thread."""
+    gen = torch.Generator().manual_seed(vocab)
+    rows = 700
+    z = _logits(gen, rows, vocab, dtype)
+    y = torch.randint(0, vocab, (rows,), generator=gen)
+    y[5], y[300], y[699] = -100, vocab + 5, vocab
+    g_lp = torch.randn(rows, generator=gen) * 0.1
+    g_h = torch.randn(rows, generator=gen) * 0.01
+    dead = [0, 1, 2, 255, 256, 257, 258, 511, 512, 513, 698, 699]
+    g_lp[dead] = 0.0
+    g_h[dead] = 0.0
+    g_h[40:60] = 0.0                                     # log-prob gradient only
+    g_lp[70:90] = 0.0                                    # entropy gradient only
+    zo = z.float().requires_grad_()
+    lp_o = o_vocab.compute_log_probs(zo, y)
+    h_o = o_vocab.vocab_parallel_entropy(zo)
+    (dz_o,) = torch.autograd.grad((lp_o * g_lp).sum() + (h_o * g_h).sum(), zo)
+    zd = z.to(dev).requires_grad_()
+    lp, h, lse = mrl.vocab_logprob_entropy(zd, y.to(dev))
+    assert (lp.cpu() - lp_o.detach()).abs().max().item() < 1e-4
+    (dz,) = torch.autograd.grad([lp, h], zd, [g_lp.to(dev), g_h.to(dev)])
+    tol = 1e-5 if dtype == torch.float32 else TOL_DLOGITS
+    assert (dz.float().cpu() - dz_o).abs().max().item() < tol
+    assert not dz[dead].any().item()
+    assert torch.equal(zd.detach().cpu(), z)
+    # log-prob gradient alone (the kernel variant without the entropy term), in place over the logits
+    (dz_lp_o,) = torch.autograd.grad((o_vocab.compute_log_probs(zo, y) * g_lp).sum(), zo)
+    zin = z.to(dev).clone()
+    gd, yd = g_lp.to(dev), y.to(dev)
+    _lib.call("mrl_vocab_logprob_bwd", zin.data_ptr(), _lib.dtype_code(zin), rows, vocab, vocab, yd.data_ptr(), _lib.I64,
+              1.0, lse.data_ptr(), None, gd.data_ptr(), None, zin.data_ptr(), _lib.dtype_code(zin), vocab,
+              _lib.stream(dev))
+    torch.cuda.synchronize()
+    assert (zin.float().cpu() - dz_lp_o).abs().max().item() < tol
+
+
+def test_fused_sweep_persistent_with_skipped_rows(dev):
+    """The fused sweep on more than 2 x CU-count rows: prompt rows, alignment padding and sequences
+    without a response are rows it must not read but must zero."""
+    gen = torch.Generator().manual_seed(21)
+    logits, b, kw, _, _ = _make_batch(gen, 6, 4, 20, 40, 8200, torch.bfloat16, 3.0, 4, prompt_hi=4)
+    assert logits.shape[1] > 600
+    b["response_length"][8:12] = 0
+    b["old_log_prob"][8:12] = 0
+    b["ref_log_prob"][8:12] = 0
+    meta = dict(clip_ratio=0.2, kl_coef=0.02, kl_penalty="low_var_kl", entropy_coeff=0.002)
+    zo = logits.float().requires_grad_()
+    want, want_stats = o_loss.grpo_compute_loss(zo, b, meta, **kw)
+    (dz_o,) = torch.autograd.grad(want, zo)
+    f = mrl.LossFuncFactory.get_instance("ray_grpo", "actor")
+    f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.02), "kl_penalty": "low_var_kl",
+                          "entropy_coeff": 0.002})
+    for coeff in (0.002, 0.0):
+        if coeff == 0.0:
+            meta["entropy_coeff"] = 0.0
+            f.add_loss_meta_info({"entropy_coeff": 0.0})
+            zo = logits.float().requires_grad_()
+            want, want_stats = o_loss.grpo_compute_loss(zo, b, meta, **kw)
+            (dz_o,) = torch.autograd.grad(want, zo)
+        zd = logits.to(dev).requires_grad_()
+        got, got_stats = f.compute_loss(zd, _to_dev(b, dev), fused=True, **_to_dev(kw, dev))
+        (dz,) = torch.autograd.grad(got, zd)
+        assert abs(got.item() - want.item()) <= TOL_LOSS_REL * abs(want.item()) + 1e-7
+        for k in want_stats:
+            assert abs(got_stats[k] - want_stats[k]) <= TOL_LOSS_REL * abs(want_stats[k]) + 1e-6, k
+        assert (dz.float().cpu() - dz_o).abs().max().item() <= 2 ** -8 * dz_o.abs().max().item() + 1e-9
+        assert torch.equal(dz.float().cpu() != 0, dz_o != 0) or \
+            ((dz.float().cpu() != 0) <= (dz_o != 0)).all().item()      # nothing outside the response rows
+
+
 @pytest.mark.parametrize("tokens,vocab,hdim", [(300, 1000, 128), (129, 256, 64), (64, 4096 + 24, 256),
                                                (517, 2 * 2048 + 256, 3584)])
 def test_lmhead_logprob_forward(dev, tokens, vocab, hdim):

@@ -81,6 +81,26 @@ def test_argument_validation_launches_nothing():
     assert lib.mrl_policy_loss_fwd(p, None, None, p, None, p, _lib.F32, None, 0, 2, 4, 0.8, 1.2, 9, 0.0, 0.0, 0, 1.0, p,
                                    p, None) == -1                                          # kl enum
     assert lib.mrl_copy_bytes(p, p + 1024, 24, None) == -1
+    # fused sweep: a vocabulary the registers cannot hold, one that is not a whole number of vectors
+    assert lib.mrl_fused_max_vocab(_lib.BF16) == 155648 and lib.mrl_fused_max_vocab(_lib.I64) == 0
+    for vocab in (155656, 1003):
+        rc = lib.mrl_fused_logprob_loss(p, _lib.BF16, 2, vocab, vocab, p, _lib.I64, 1.0, p, 1, 0.8, 1.2, 4, 0.0, 0.0,
+                                        1.0, p, vocab, None, None, p, None)
+        assert rc == -2, vocab
+    assert lib.mrl_fused_logprob_loss(p, _lib.BF16, 2, 64, 64, p, _lib.I64, 1.0, None, 1, 0.8, 1.2, 4, 0.0, 0.0, 1.0,
+                                      p, 64, None, None, p, None) == -1                   # no row operands
+    assert lib.mrl_scale_rows(p, _lib.I32, 2, 64, 64, p, 1.0, None) == -2
+    # fused lm_head: hidden size must be a multiple of the K tile, workspace must be large enough
+    assert lib.mrl_lmhead_workspace_bytes(100, 1000) > 0
+    assert lib.mrl_lmhead_logprob_fwd(p, p, 4, 1000, 100, p, _lib.I64, 1.0, p, None, None, p, 1 << 20, None) != 0
+    assert lib.mrl_lmhead_logprob_fwd(p, p, 4, 1000, 128, p, _lib.I64, 1.0, p, None, None, p, 16, None) != 0
+    assert b"workspace" in lib.mrl_last_error()
+    # bandwidth probe
+    assert lib.mrl_bandwidth_probe(3, p, p, 1, 1024, None) == -1
+    assert lib.mrl_bandwidth_probe(2, p, p, 1, 1000, None) == -1
+    assert lib.mrl_bandwidth_probe(2, p, p, 1, 19 * 1024 * 16 + 16, None) == -2
+    assert lib.mrl_bandwidth_probe(2, None, p, 1, 1024, None) == -1
+    assert lib.mrl_bandwidth_probe(2, None, None, 0, 1024, None) == 0
     with pytest.raises(_lib.MrlError) as err:
         _lib.call("mrl_copy_bytes", p, p + 1024, 24, None)
     assert err.value.code == -1 and "multiple of 16" in str(err.value)
