@@ -1,7 +1,7 @@
 """Ragged <-> padded experience columns: the on-wire layout either side of the loss path.
 
-Host-side mirror of ``unpack_pad_experience`` (``mindspeed_rl/trainer/utils/transfer_dock.py:
-1092-1198``) and ``truncate_rows`` (``mindspeed_rl/utils/pad_process.py:144-166``) with the
+Host-side mirror of ``pack_experience_columns`` / ``unpack_pad_experience``
+(``mindspeed_rl/trainer/utils/transfer_dock.py:1014-1198``) and ``truncate_rows`` (``mindspeed_rl/utils/pad_process.py:144-166``) with the
 reference's signatures.  The reference walks the rows in Python with one or two ``.item()`` calls
 per row; here each column costs one scan launch, one host read of two integers (to size the
 output) and one gather launch.
@@ -18,6 +18,75 @@ def _index(t):
     if t.dtype not in (torch.int32, torch.int64):
         t = t.to(torch.int64)
     return t.reshape(-1).contiguous()
+
+
+def pack_padded_columns(padded, lengths, left_pad=False):
+    """Device form of the packing step: ``padded`` maps column -> ``[B, W]`` tensor (4- or 8-byte
+    elements), ``lengths`` column -> ``[B]`` or ``[B, 1]`` integer lengths.  Returns
+    ``(batch_data, batch_data_length)`` in the layout of :func:`pack_experience_columns`: one flat
+    tensor per column holding ``padded[i, :len_i]`` back to back (``padded[i, W - len_i:]`` with
+    ``left_pad``) and the int32 lengths.  One scan launch, one host read (the total, to size the
+    output) and one gather launch per column."""
+    if not padded:
+        raise ValueError("ERROR: when pack, get an empty experience_dict")
+    if set(padded.keys()) != set(lengths.keys()):
+        raise ValueError("ERROR: when pack, keys of the columns and of their lengths do not match")
+    batch_data, batch_data_length = {}, {}
+    for key, src in padded.items():
+        dev = _lib.require_device(src)
+        src = src.contiguous()
+        if src.dim() != 2 or src.element_size() not in (4, 8):
+            raise TypeError("pack_padded_columns takes [B, W] columns with 4- or 8-byte elements")
+        batch, width = src.shape
+        idx = _index(lengths[key].to(dev))
+        if idx.numel() != batch:
+            raise ValueError("ERROR: when pack, experience '%s' number=%d does not match experience_count=%d"
+                             % (key, idx.numel(), batch))
+        eff = torch.empty(batch, dtype=torch.int32, device=dev)
+        cu = torch.empty(batch + 1, dtype=torch.int32, device=dev)
+        info = torch.empty(2, dtype=torch.int64, device=dev)
+        stream = _lib.stream(dev)
+        _lib.call("mrl_ragged_layout", _lib.ptr(idx), _lib.dtype_code(idx), batch, 1, None, src.element_size(), width,
+                  0, _lib.ptr(eff), _lib.ptr(cu), _lib.ptr(info), stream)
+        total = int(info[0].item())
+        flat = torch.empty(total, dtype=src.dtype, device=dev)
+        _lib.call("mrl_padded_to_ragged", _lib.ptr(src), src.element_size(), batch, width, _lib.ptr(cu),
+                  1 if left_pad else 0, total, _lib.ptr(flat), stream)
+        batch_data[key] = flat
+        batch_data_length[key] = eff
+    return batch_data, batch_data_length
+
+
+def pack_experience_columns(experience_consumer_stage, experience_dict, experience_count, enable_partial_rollout=False):
+    """Mirror of ``pack_experience_columns`` (``trainer/utils/transfer_dock.py:1014-1089``) for lists of
+    per-sample DEVICE tensors: one flat tensor per column (``[D, sum]`` for 2-D samples) plus int32
+    lengths.  The samples are separate allocations, so the concatenation is the library's batched
+    copy (``torch.cat``); the lengths come from the shapes, without a device read.  The reference
+    goes through ``.tolist()`` for every sample."""
+    if not experience_dict:
+        raise ValueError("ERROR: when pack, get an empty experience_dict")
+    if enable_partial_rollout and experience_consumer_stage == "actor_rollout":
+        experience_count = len(experience_dict["prompts"])
+    else:
+        for key, value in experience_dict.items():
+            if len(value) != experience_count:
+                raise ValueError("ERROR: when pack, experience '%s' number=%d does not match experience_count=%d"
+                                 % (key, len(value), experience_count))
+    batch_data, batch_data_length = {}, {}
+    for key, value in experience_dict.items():
+        value = list(value[:experience_count])
+        dev = _lib.require_device(value[0])
+        if value[0].dim() > 1:
+            first_dim = value[0].shape[0]
+            if any(v.shape[0] != first_dim for v in value):
+                raise ValueError("ERROR: when pack 2D tensor, first dimension must be the same for all experiences")
+            batch_data[key] = torch.cat(value, dim=1)
+            sizes = [v.shape[1] for v in value]
+        else:
+            batch_data[key] = torch.cat(value, dim=0)
+            sizes = [v.shape[0] for v in value]
+        batch_data_length[key] = torch.tensor(sizes, dtype=torch.int32).to(dev)
+    return batch_data, batch_data_length
 
 
 def unpack_pad_experience(batch_data, batch_data_length, pad_id, multiple):

@@ -106,6 +106,39 @@ def response_window(prompt_length, response_length):
     return torch.cat([prompt_length, prompt_length + response_length], dim=1) - 1
 
 
+def pack_experience_columns(experience_consumer_stage, experience_dict, experience_count, enable_partial_rollout=False):
+    """``trainer/utils/transfer_dock.py:1014-1089``: lists of per-sample tensors -> one flat tensor per
+    column (``[D, sum]`` for 2-D samples ``[D, n_i]``) plus int32 lengths."""
+    if not experience_dict:
+        raise ValueError("ERROR: when pack, get an empty experience_dict")
+    if enable_partial_rollout and experience_consumer_stage == "actor_rollout":
+        experience_count = len(experience_dict["prompts"])
+    else:
+        for key, value in experience_dict.items():
+            if len(value) != experience_count:
+                raise ValueError("ERROR: when pack, experience '%s' number=%d does not match experience_count=%d"
+                                 % (key, len(value), experience_count))
+    batch_data, batch_data_length = {}, {}
+    for key, value in experience_dict.items():
+        if value[0].dim() > 1:
+            first_dim = value[0].shape[0]
+            for i in range(experience_count):
+                if value[i].shape[0] != first_dim:
+                    raise ValueError("ERROR: when pack 2D tensor, first dimension must be the same for all experiences")
+            rows = [[x for i in range(experience_count) for x in value[i][d].tolist()] for d in range(first_dim)]
+            batch_data[key] = torch.tensor(rows, dtype=value[0].dtype)
+            batch_data_length[key] = torch.tensor([value[i].shape[1] for i in range(experience_count)],
+                                                  dtype=torch.int32)
+        else:
+            flat, lengths = [], []
+            for i in range(experience_count):
+                flat.extend(value[i].tolist())
+                lengths.append(len(value[i]))
+            batch_data[key] = torch.tensor(flat, dtype=value[0].dtype)
+            batch_data_length[key] = torch.tensor(lengths, dtype=torch.int32)
+    return batch_data, batch_data_length
+
+
 def unpack_pad_experience(batch_data, batch_data_length, pad_id, multiple):
     """``trainer/utils/transfer_dock.py:1092-1198``: flat packed columns + lengths -> padded columns."""
     if not batch_data:

@@ -364,6 +364,29 @@ def test_wire_format_bit_exact(dev):
     for left in (False, True):
         for a, b in zip(mrl.truncate_rows(f.to(dev), idx.to(dev), left), o_pack.truncate_rows(f, idx, left)):
             assert a.dtype == b.dtype and torch.equal(a, b)
+    # packing: lists of samples (the reference's input) and padded columns + lengths (the device form)
+    cu_a = torch.cat([torch.zeros(1, dtype=torch.int64), lens_a.long().cumsum(0)])
+    cu_b = torch.cat([torch.zeros(1, dtype=torch.int64), lens_b.long().cumsum(0)])
+    samples = {"responses": [data["responses"][cu_a[i]:cu_a[i + 1]] for i in range(batch)],
+               "old_log_prob": [data["old_log_prob"][cu_a[i]:cu_a[i + 1]] for i in range(batch)],
+               "position_ids": [data["position_ids"][:, cu_b[i]:cu_b[i + 1]] for i in range(batch)]}
+    want, want_len = o_pack.pack_experience_columns("actor_train", samples, batch)
+    got, got_len = mrl.pack_experience_columns("actor_train", {k: [t.to(dev) for t in v] for k, v in samples.items()},
+                                               batch)
+    for k in want:
+        assert got[k].dtype == want[k].dtype and torch.equal(got[k].cpu(), want[k]), k
+        assert got_len[k].dtype == torch.int32 and torch.equal(got_len[k].cpu(), want_len[k]), k
+    padded = o_pack.unpack_pad_experience({k: data[k] for k in ("responses", "old_log_prob")},
+                                          {k: lens[k] for k in ("responses", "old_log_prob")}, -7, 8)
+    got, got_len = mrl.pack_padded_columns({k: v.to(dev) for k, v in padded.items()},
+                                           {"responses": lens_a.to(dev), "old_log_prob": lens_a.view(-1, 1)})
+    for k in padded:
+        assert torch.equal(got[k].cpu(), data[k]) and torch.equal(got_len[k].cpu(), lens_a), k
+    right = torch.flip(padded["responses"], dims=[1])          # the same samples, reversed and right-aligned
+    got, _ = mrl.pack_padded_columns({"r": right.to(dev)}, {"r": lens_a}, left_pad=True)
+    assert torch.equal(got["r"].cpu(), torch.cat([torch.flip(s_, dims=[0]) for s_ in samples["responses"]]))
+    with pytest.raises(ValueError):
+        mrl.pack_experience_columns("actor_train", {"responses": samples["responses"]}, batch - 1)
 
 
 # --------------------------------------------------------------------------------- advantages

@@ -419,3 +419,22 @@ def test_wire_format_reference_vectors():
         packing.unpack_pad_experience({}, {}, 0, 1)
     with pytest.raises(ValueError):
         packing.unpack_pad_experience(data, {"prompts": lens["prompts"]}, 0, 1)
+    # the worked example in the docstring of pack_experience_columns (transfer_dock.py:1015-1037): the
+    # same columns as lists of samples pack to exactly the flat tensors and lengths above
+    samples = {"prompts": [torch.tensor([1, 1, 1]), torch.tensor([2, 2, 2, 2]), torch.tensor([3, 3, 3]),
+                           torch.tensor([4, 4, 4, 4])],
+               "attention_mask": [torch.tensor([1]), torch.tensor([2, 2]), torch.tensor([3, 3, 3]),
+                                  torch.tensor([4, 4, 4, 4])]}
+    flat, flat_len = packing.pack_experience_columns("actor_train", samples, 4)
+    for k in data:
+        assert torch.equal(flat[k], data[k]) and torch.equal(flat_len[k], lens[k]) and flat_len[k].dtype == torch.int32
+    pos = {"position_ids": [torch.arange(6).view(3, 2), torch.arange(9).view(3, 3) + 10]}
+    flat, flat_len = packing.pack_experience_columns("actor_train", pos, 2)
+    assert flat["position_ids"].tolist() == [[0, 1, 10, 11, 12], [2, 3, 13, 14, 15], [4, 5, 16, 17, 18]]
+    assert flat_len["position_ids"].tolist() == [2, 3]
+    back = packing.unpack_pad_experience(flat, flat_len, 0, 1)["position_ids"]
+    assert back.shape == (2, 3, 3) and back[0, :, :2].tolist() == pos["position_ids"][0].tolist()
+    with pytest.raises(ValueError):
+        packing.pack_experience_columns("actor_train", samples, 3)
+    with pytest.raises(ValueError):
+        packing.pack_experience_columns("actor_train", {}, 0)
