@@ -341,6 +341,53 @@ int mrl_lmhead_logprob_fwd(const void* hidden, const void* weight, int64_t n_tok
                            void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * PPO's value side (the "next" row after the actor path): rewards with the KL penalty, GAE,
+ * whitening and the critic's clipped value loss.  All tensors [batch, width] fp32, contiguous.
+ *
+ * mrl_kl_token_rewards: the arithmetic inside apply_kl_penalty
+ * (mindspeed_rl/trainer/utils/compute_utils.py:80-97): mask = (j < response_length[i]);
+ * kld = compute_kl_penalty(old_log_prob, ref_log_prob, kl_penalty) * mask; rewards[i, j] =
+ * (j == response_length[i] - 1 ? scores[i] : 0) - beta * kld (a zero length puts the score on the
+ * last column, like python's index -1); row_kl[i] = sum_j kld / (sum_j mask + 1e-8).  The caller
+ * averages row_kl for kl_ctrl.update(). */
+int mrl_kl_token_rewards(const float* old_log_prob, const float* ref_log_prob,
+                         const void* response_length, int length_dtype, const float* scores,
+                         int64_t batch, int64_t width, int kl_penalty, float beta, float* rewards,
+                         float* row_kl, void* stream);
+
+/* mrl_gae_scan: the reverse scan of compute_gae_advantage_return (compute_utils.py:134-145), before
+ * its whitening: delta_t = rewards[t] + gamma * values[t+1] - values[t] (values[width] = 0),
+ * lastgaelam = delta_t + (gamma * lam) * lastgaelam, advantages[t] = lastgaelam, returns =
+ * advantages + values.  fp32 with the reference's operation order and roundings: bit-identical to
+ * the torch loop.  Outputs must not alias the inputs. */
+int mrl_gae_scan(const float* rewards, const float* values, int64_t batch, int64_t width, float gamma,
+                 float lam, float* advantages, float* returns, void* stream);
+
+/* mrl_masked_whiten: masked_whiten / masked_var / masked_mean (mindspeed_rl/utils/
+ * torch_functional.py:46-106) over n entries: mean = sum(x*mask)/(sum(mask)+1e-8), var the same of
+ * (x-mean)^2 times sum(mask)/(sum(mask)-1) unless sum(mask) == 1, out = (x-mean)*rsqrt(var+1e-8)
+ * (+ mean unless shift_mean).  mask: F32, I64, I32 or U8.  info (3 doubles on the device) receives
+ * sum(mask), mean, var; the caller raises the reference's ValueError when sum(mask) == 0.
+ * out may alias x. */
+int mrl_masked_whiten(const float* x, const void* mask, int mask_dtype, int64_t n, int shift_mean,
+                      float* out, double* info, void* stream);
+
+/* mrl_value_loss_fwd / _bwd: CriticLossFunc._compute_value_loss
+ * (mindspeed_rl/models/loss/critic_loss_func.py:82-111) and its backward with respect to vpreds:
+ * vf_loss = 0.5 * masked_mean(max((vp-ret)^2, (clamp(vp, v-c, v+c)-ret)^2)), vf_clipfrac =
+ * masked_mean(second > first).  The mask is `mask` or, if NULL, (j < response_length[i]).
+ * out (4 floats): loss_scale * vf_loss, vf_loss, vf_clipfrac, sum(mask).  The backward follows
+ * torch: the larger operand of max gets the gradient (halved on ties), clamp passes it inside the
+ * closed interval; g_vpreds = upstream[0] * d(out[0])/d(vpreds). */
+int mrl_value_loss_fwd(const float* vpreds, const float* returns, const float* values, const void* mask,
+                       int mask_dtype, const void* response_length, int length_dtype, int64_t batch,
+                       int64_t width, float cliprange_value, float loss_scale, float* out, void* stream);
+int mrl_value_loss_bwd(const float* vpreds, const float* returns, const float* values, const void* mask,
+                       int mask_dtype, const void* response_length, int length_dtype, int64_t batch,
+                       int64_t width, float cliprange_value, float loss_scale, const float* out,
+                       const float* upstream, float* g_vpreds, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Plain device-to-device copy kernel of n_bytes (multiple of 16, 16-byte aligned pointers);
  * used to calibrate the rocprofv3 FETCH_SIZE / WRITE_SIZE counters and as the measured
  * bandwidth ceiling next to the 8 TB/s vendor peak.  No counterpart in the reference. */

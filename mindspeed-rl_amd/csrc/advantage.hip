@@ -57,16 +57,16 @@ __global__ __launch_bounds__(kBlock) void group_advantage_kernel(const void* __r
 // numpy's arithmetic, one correctly rounded operation at a time (no FMA contraction)
 template <typename F> struct Rn;
 template <> struct Rn<double> {
-    static __device__ __forceinline__ double add(double a, double b) { return __dadd_rn(a, b); }
-    static __device__ __forceinline__ double sub(double a, double b) { return __dsub_rn(a, b); }
-    static __device__ __forceinline__ double mul(double a, double b) { return __dmul_rn(a, b); }
+    static __device__ __forceinline__ double add(double a, double b) { return mrl::add_rn(a, b); }
+    static __device__ __forceinline__ double sub(double a, double b) { return mrl::sub_rn(a, b); }
+    static __device__ __forceinline__ double mul(double a, double b) { return mrl::mul_rn(a, b); }
     static __device__ __forceinline__ double div(double a, double b) { return __ddiv_rn(a, b); }
     static __device__ __forceinline__ double root(double a) { return __dsqrt_rn(a); }
 };
 template <> struct Rn<float> {
-    static __device__ __forceinline__ float add(float a, float b) { return __fadd_rn(a, b); }
-    static __device__ __forceinline__ float sub(float a, float b) { return __fsub_rn(a, b); }
-    static __device__ __forceinline__ float mul(float a, float b) { return __fmul_rn(a, b); }
+    static __device__ __forceinline__ float add(float a, float b) { return mrl::add_rn(a, b); }
+    static __device__ __forceinline__ float sub(float a, float b) { return mrl::sub_rn(a, b); }
+    static __device__ __forceinline__ float mul(float a, float b) { return mrl::mul_rn(a, b); }
     static __device__ __forceinline__ float div(float a, float b) { return __fdiv_rn(a, b); }
     static __device__ __forceinline__ float root(float a) { return __fsqrt_rn(a); }
 };

@@ -50,6 +50,26 @@ __device__ inline void buf_store_b16(uint16_t, rsrc_t, uint32_t) {}
 __device__ inline void buf_store_b32(uint32_t, rsrc_t, uint32_t) {}
 #endif
 
+// Single IEEE operations that stay single: HIP compiles with floating-point contraction on, and its
+// __fadd_rn / __fmul_rn are plain operators, so `a + b * c` (also across inlined calls) becomes one
+// fused multiply-add with a single rounding.  Where a kernel has to reproduce the separately rounded
+// arithmetic of numpy or of a torch CPU loop bit for bit, it goes through these.
+template <typename F>
+__host__ __device__ __forceinline__ F add_rn(F a, F b) {
+#pragma clang fp contract(off)
+    return a + b;
+}
+template <typename F>
+__host__ __device__ __forceinline__ F sub_rn(F a, F b) {
+#pragma clang fp contract(off)
+    return a - b;
+}
+template <typename F>
+__host__ __device__ __forceinline__ F mul_rn(F a, F b) {
+#pragma clang fp contract(off)
+    return a * b;
+}
+
 // Stores a printf-style message for mrl_last_error() and returns `code`.
 int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 void clear_error();

@@ -14,6 +14,8 @@ from .loss import (BaseLossFunc, DAPOActorLossFunc, GRPOActorLossFunc, LossFuncF
                    policy_loss)
 from .packing import (generate_mask, pack_index, postprocess_packed_seqs, preprocess_packed_seqs, response_window,
                       truncate_middle_and_pad, truncate_prompt_and_pad)
+from .value_path import (AdaptiveKLController, CriticLossFunc, compute_gae_advantage_return, kl_token_level_rewards,
+                         masked_var, masked_whiten, value_loss)
 from .wire import pack_experience_columns, pack_padded_columns, truncate_rows, unpack_pad_experience
 from .vocab_ops import (compute_kl_penalty, compute_log_probs, get_parallel_state, get_vocab_parallel,
                         set_parallel_state, set_vocab_parallel, vocab_logprob_entropy, vocab_parallel_cross_entropy,

@@ -118,7 +118,7 @@ def _unpad_raw(packed, seqlens, cu, seq_len, prompt):
 def postprocess_packed_seqs(output, seqlens_in_batch, cu_seqlens_padded, seq_len, prompt_length=None):
     """Reference: ``utils/remove_padding.py:90-136``: packed ``[1,T,...]`` -> ``[B,seq_len,...]``
     with optional prompt truncation (``start += P-1``, ``len -= P``).  Differentiable for fp32
-    ``[1,T]`` inputs.  A window longer than ``seq_len`` is cut to ``seq_len`` (the reference
+    ``[1,T]`` and ``[1,T,1]`` inputs.  A window longer than ``seq_len`` is cut to ``seq_len`` (the reference
     raises there)."""
     if output.shape[0] != 1:
         raise ValueError("Expected output tensor to have shape[0] == 1 (packed batch dimension)")
@@ -126,9 +126,11 @@ def postprocess_packed_seqs(output, seqlens_in_batch, cu_seqlens_padded, seq_len
     cu = cu_seqlens_padded.to(torch.int32).contiguous()
     prompt = None if prompt_length is None else _as_index(prompt_length)
     if output.requires_grad and torch.is_grad_enabled():
-        if output.dim() != 2 or output.dtype != torch.float32:
-            raise TypeError("gradients are supported for fp32 [1, T] inputs only")
-        return _UnpadGather.apply(output, seqlens, cu, seq_len, prompt)
+        scalar_rows = output.dim() == 2 or (output.dim() == 3 and output.shape[2] == 1)
+        if not scalar_rows or output.dtype != torch.float32:
+            raise TypeError("gradients are supported for fp32 [1, T] or [1, T, 1] inputs only")
+        out = _UnpadGather.apply(output.reshape(1, output.shape[1]), seqlens, cu, seq_len, prompt)
+        return out.unsqueeze(-1) if output.dim() == 3 else out
     return _unpad_raw(output, seqlens, cu, seq_len, prompt)
 
 
@@ -203,10 +205,18 @@ def truncate_prompt_and_pad(responses, input_tensor, truncate_lengths, pad_value
 
 def truncate_middle_and_pad(responses, input_tensor, truncate_lengths, pad_value=0.0):
     """Reference: ``utils/pad_process.py:74-106``: ``[mbs, seq_len, vocab]`` ->
-    ``[mbs, responses.shape[-1], vocab]``; forward only."""
+    ``[mbs, responses.shape[-1], vocab]``.  Differentiable for fp32 inputs with a last dimension of 1
+    (the value head's output); wider inputs are forward only."""
     if input_tensor.dim() != 3:
         raise ValueError("input_tensor must have shape (mbs, seq_len, vocab_size)")
-    return _window_raw(input_tensor, _window_tensor(truncate_lengths), responses.shape[-1], pad_value)
+    window = _window_tensor(truncate_lengths)
+    out_len = responses.shape[-1]
+    if input_tensor.requires_grad and torch.is_grad_enabled():
+        if input_tensor.shape[2] != 1 or input_tensor.dtype != torch.float32:
+            raise TypeError("gradients are supported for fp32 inputs with a last dimension of 1 only")
+        flat = input_tensor.reshape(input_tensor.shape[0], input_tensor.shape[1])
+        return _WindowGather.apply(flat, window, out_len, pad_value).unsqueeze(-1)
+    return _window_raw(input_tensor, window, out_len, pad_value)
 
 
 def response_window(prompt_length, response_length):

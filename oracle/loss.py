@@ -10,6 +10,8 @@ Restates with stock torch ops (so that autograd supplies the backward the refere
   ``dapo_actor_loss_func.py:47-102``                                ``compute_loss`` tail (scale + stats)
 * ``mindspeed_rl/models/loss/ppo_actor_loss_func.py:39-133``       PPO actor (the GRPO surrogate without KL)
 * ``mindspeed_rl/models/loss/logprob_computer.py:94-145``          ``StandardLogProbComputer.compute``
+* ``mindspeed_rl/utils/torch_functional.py:62-106``                ``masked_var`` / ``masked_whiten``
+* ``mindspeed_rl/models/loss/critic_loss_func.py:37-111``          critic value loss (``compute_loss`` + clipped MSE)
 
 Pinned by ``tests/ut/utils/test_compute_utils.py:92-108`` (KL vectors),
 ``tests/ut/utils/test_torch_functional.py:24-29`` (masked mean) and hand-derived cases.
@@ -29,6 +31,32 @@ def masked_sum(values, mask, axis=None):
 def masked_mean(values, mask, axis=None, epsilon=1e-8):
     """``torch_functional.py:46-59``."""
     return masked_sum(values, mask, axis) / (mask.sum(axis=axis) + epsilon)
+
+
+def masked_var(values, mask, unbiased=True):
+    """``torch_functional.py:62-87``."""
+    mean = masked_mean(values, mask)
+    centered_values = values - mean
+    variance = masked_mean(centered_values ** 2, mask)
+    if unbiased:
+        mask_sum = mask.sum()
+        if mask_sum == 0:
+            raise ValueError("At least one element in the mask has to be 1.")
+        elif mask_sum == 1:
+            bessel_correction = mask_sum
+        else:
+            bessel_correction = mask_sum / (mask_sum - 1)
+        variance = variance * bessel_correction
+    return variance
+
+
+def masked_whiten(values, mask, shift_mean=True):
+    """``torch_functional.py:90-106``."""
+    mean, var = masked_mean(values, mask), masked_var(values, mask)
+    whitened = (values - mean) * torch.rsqrt(var + 1e-8)
+    if not shift_mean:
+        whitened += mean
+    return whitened
 
 
 def compute_kl_penalty(logprob, ref_logprob, kl_penalty="low_var_kl"):
@@ -198,3 +226,38 @@ def ppo_compute_loss(output, batch, meta, forward_only=False, **kwargs):
     policy_loss, stats = _finish(pg_loss, clipfrac, ppo_kl, torch.zeros(()), ent, batch, forward_only, kwargs)
     del stats["actor/kl_loss"]
     return policy_loss, stats
+
+
+def value_loss(vpreds, returns, values, response_mask, cliprange_value):
+    """``critic_loss_func.py:82-111``."""
+    vpreds = vpreds.squeeze()
+    vpredclipped = torch.clamp(vpreds, values - cliprange_value, values + cliprange_value)
+    vf_losses1 = (vpreds - returns) ** 2
+    vf_losses2 = (vpredclipped - returns) ** 2
+    vf_loss = 0.5 * masked_mean(torch.max(vf_losses1, vf_losses2), response_mask)
+    vf_clipfrac = masked_mean(torch.gt(vf_losses2, vf_losses1).float(), response_mask)
+    return vf_loss, vf_clipfrac
+
+
+def critic_compute_loss(output, batch, cliprange_value=0.5, forward_only=False, **kwargs):
+    """``critic_loss_func.py:37-80``: ``output`` is the value head's ``[B, S, 1]`` (or packed
+    ``[1, T, 1]``); the response window is cut with ``truncate_middle_and_pad``."""
+    if kwargs.get("use_remove_padding", False):
+        output = packing.postprocess_packed_seqs(output, kwargs.get("seqlens_in_batch"),
+                                                 kwargs.get("cu_seqlens_padded"), kwargs.get("seq_len"))
+    if "responses" not in batch:
+        raise ValueError("The responses is None")
+    truncate_lengths = torch.cat([batch["prompt_length"], batch["prompt_length"] + batch["response_length"]],
+                                 dim=1) - 1
+    vpreds = packing.truncate_middle_and_pad(batch["responses"], output, truncate_lengths)
+    if forward_only:
+        return vpreds
+    response_mask = packing.generate_mask(batch["responses"], batch["response_length"])
+    vf_loss, vf_clipfrac = value_loss(vpreds, batch.get("returns"), batch.get("values"), response_mask,
+                                      cliprange_value)
+    if kwargs.get("use_dynamic_bsz", False) and not forward_only:
+        loss = vf_loss * (batch["responses"].size(0) / kwargs.get("actual_micro_batch_size"))
+    else:
+        loss = vf_loss
+    stats = {"critic/vf_loss": abs(vf_loss.detach().item()), "critic/vf_clipfrac": vf_clipfrac.detach().item()}
+    return loss, stats

@@ -389,6 +389,147 @@ def test_wire_format_bit_exact(dev):
         mrl.pack_experience_columns("actor_train", {"responses": samples["responses"]}, batch - 1)
 
 
+# --------------------------------------------------------------------------------- PPO value side
+def test_value_side_reference_vectors_on_device(dev, reference_vectors):
+    w = reference_vectors["masked_whiten"]
+    got = mrl.masked_whiten(torch.tensor(w["values"]).to(dev), torch.tensor(w["mask"]).to(dev))
+    assert torch.allclose(got.cpu(), torch.tensor(w["expected"]), atol=w["atol"])
+    v = reference_vectors["masked_var"]
+    got = mrl.masked_var(torch.tensor(v["values"]).to(dev), torch.tensor(v["mask"]).to(dev), unbiased=True)
+    assert torch.isclose(got.cpu(), torch.tensor(v["expected"]), atol=v["atol"])
+    with pytest.raises(ValueError, match="At least one element"):
+        mrl.masked_whiten(torch.ones(4, device=dev), torch.zeros(4, device=dev))
+    g = reference_vectors["gae"]
+    adv, ret = mrl.compute_gae_advantage_return(torch.tensor(g["token_level_rewards"]).to(dev),
+                                                torch.tensor(g["values"]).to(dev), torch.tensor(g["eos_mask"]).to(dev),
+                                                torch.tensor(g["gamma"]), torch.tensor(g["lam"]))
+    assert torch.equal(adv.cpu(), torch.tensor(g["expected_advantages"]))
+    assert torch.equal(ret.cpu(), torch.tensor(g["expected_returns"]))
+    a = reference_vectors["adaptive_kl"]
+    for case in a["cases"]:
+        ctrl = mrl.AdaptiveKLController(a["init_kl_coef"], a["target_kl"], a["horizon"])
+        ctrl.update(case["current_kl"], case["n_steps"])
+        assert ctrl.value == case["expected"]
+    crit = mrl.LossFuncFactory.get_instance(*reference_vectors["critic"]["registry_key"])
+    assert isinstance(crit, mrl.CriticLossFunc)
+    assert crit.cliprange_value == reference_vectors["critic"]["default_cliprange_value"]
+    crit.add_loss_meta_info({"cliprange_value": 0.3})
+    assert crit.cliprange_value == 0.3
+    crit.add_loss_meta_info(None)
+    c = reference_vectors["critic"]["no_clipping"]
+    vf, frac = crit._compute_value_loss(torch.tensor(c["vpreds"]).to(dev), torch.tensor(c["returns"]).to(dev),
+                                        torch.tensor(c["values"]).to(dev),
+                                        torch.tensor(c["response_mask"], dtype=torch.float32).to(dev),
+                                        c["cliprange_value"])
+    assert frac.item() == 0 and vf.item() == 0.0
+    with pytest.raises(ValueError, match="The responses is None"):
+        crit._get_policy_loss_input({"values": torch.zeros(1, 1)})
+
+
+@pytest.mark.parametrize("batch,width", [(37, 300), (3, 5000), (1, 1), (130, 2048)])
+def test_gae_and_whitening_parity(dev, batch, width):
+    """The scan is bit-identical to the reference's torch loop (same fp32 operation order), also across
+    the 2048-entry staging chunks; the whitened advantages agree to fp32 summation-order accuracy."""
+    gen = torch.Generator().manual_seed(batch * 100 + width)
+    r = torch.randn(batch, width, generator=gen)
+    v = torch.randn(batch, width, generator=gen)
+    lens = torch.randint(1, width + 1, (batch, 1), generator=gen)
+    mask = o_pack.generate_mask(r, lens)
+    mask[0, 0] = 1
+    if batch * width > 1:
+        mask.view(-1)[1] = 1                # at least two entries: the unbiased variance is defined
+    for gamma, lam in ((1.0, 0.95), (0.97, 0.9)):
+        want_adv, want_ret = o_adv.compute_gae_advantage_return(r, v, mask, torch.tensor(gamma), torch.tensor(lam))
+        adv, ret = mrl.compute_gae_advantage_return(r.to(dev), v.to(dev), mask.to(dev), gamma, lam)
+        assert torch.equal(ret.cpu(), want_ret)
+        scale = max(1.0, want_adv.abs().max().item())
+        assert (adv.cpu() - want_adv).abs().max().item() < 1e-5 * scale
+    # masked_var stand-alone, both estimators, float and bool masks
+    for unbiased in (True, False):
+        want = o_loss.masked_var(r, mask.float(), unbiased)
+        for m in (mask.float(), mask.bool(), mask):
+            got = mrl.masked_var(r.to(dev), m.to(dev), unbiased)
+            assert got.item() == pytest.approx(want.item(), rel=1e-5, abs=1e-7)
+    got = mrl.masked_whiten(r.to(dev), mask.to(dev), shift_mean=False)
+    assert (got.cpu() - o_loss.masked_whiten(r, mask.float(), shift_mean=False)).abs().max().item() < 1e-5 * max(
+        1.0, r.abs().max().item() * 2)
+
+
+@pytest.mark.parametrize("penalty", ["kl", "abs", "mse", "low_var_kl"])
+def test_kl_token_rewards_parity(dev, penalty):
+    gen = torch.Generator().manual_seed(17)
+    batch, width = 29, 77
+    old = -torch.rand(batch, width, generator=gen) * 5
+    ref = old + torch.randn(batch, width, generator=gen) * 0.3
+    lens = torch.randint(1, width + 1, (batch, 1), generator=gen)
+    lens[3] = width
+    lens[4] = 1
+    scores = torch.randn(batch, generator=gen)
+    want, want_kl = o_adv.kl_token_level_rewards(old, ref, lens, scores, 0.05, penalty)
+    for cast in (torch.int64, torch.int32):
+        got, got_kl = mrl.kl_token_level_rewards(old.to(dev), ref.to(dev), lens.to(cast).to(dev), scores.to(dev), 0.05,
+                                                 penalty)
+        assert (got.cpu() - want).abs().max().item() < 1e-6
+        assert got_kl == pytest.approx(want_kl, rel=1e-5, abs=1e-8)
+    with pytest.raises(NotImplementedError):
+        mrl.kl_token_level_rewards(old.to(dev), ref.to(dev), lens.to(dev), scores.to(dev), 0.05, "full")
+
+
+def test_value_loss_and_critic_parity(dev):
+    gen = torch.Generator().manual_seed(23)
+    batch, width = 19, 53
+    values = torch.randn(batch, width, generator=gen)
+    vp = values + torch.randn(batch, width, generator=gen) * 0.4
+    vp[0, :5] = values[0, :5]                        # ties of the two squared errors
+    vp[1, :5] = values[1, :5] + 0.2                  # exactly on the edge of the clip interval
+    returns = values + torch.randn(batch, width, generator=gen)
+    lens = torch.randint(0, width + 1, (batch, 1), generator=gen)
+    mask = o_pack.generate_mask(vp, lens).float()
+    for m_o, kwargs in ((mask, dict(response_mask=mask.to(dev))), (mask, dict(response_length=lens.to(dev))),
+                        (mask * 0.5, dict(response_mask=(mask * 0.5).to(dev)))):
+        vo = vp.clone().requires_grad_()
+        want, want_frac = o_loss.value_loss(vo, returns, values, m_o, 0.2)
+        (g_o,) = torch.autograd.grad(want * 3.0, vo)
+        vd = vp.to(dev).requires_grad_()
+        got, out = mrl.value_loss(vd, returns.to(dev), values.to(dev), cliprange_value=0.2, loss_scale=3.0, **kwargs)
+        assert got.item() == pytest.approx(3.0 * want.item(), rel=TOL_LOSS_REL)
+        assert out[1].item() == pytest.approx(want.item(), rel=TOL_LOSS_REL)
+        assert out[2].item() == pytest.approx(want_frac.item(), rel=1e-5, abs=1e-8)
+        (g,) = torch.autograd.grad(got, vd)
+        assert (g.cpu() - g_o).abs().max().item() < 1e-6
+    # the loss object end to end: value head output [B, S, 1] padded, and [1, T, 1] packed
+    n_seq, align = 6, 4
+    plen = torch.randint(1, 5, (n_seq, 1), generator=gen, dtype=torch.int32)
+    rlen = torch.randint(1, 12, (n_seq, 1), generator=gen, dtype=torch.int32)
+    seq = int((plen + rlen).max())
+    resp_w = int(rlen.max())
+    ids = torch.ones(n_seq, seq, dtype=torch.int64)
+    mask1d = o_pack.generate_mask(ids, plen + rlen)
+    _, _, _, seqlens, cu = o_pack.preprocess_packed_seqs(ids, ids, mask1d, align)
+    total = int(cu[-1])
+    b = {"responses": torch.zeros(n_seq, resp_w, dtype=torch.int64), "prompt_length": plen, "response_length": rlen,
+         "values": torch.randn(n_seq, resp_w, generator=gen), "returns": torch.randn(n_seq, resp_w, generator=gen)}
+    crit = mrl.CriticLossFunc()
+    crit.add_loss_meta_info({"cliprange_value": 0.3})
+    cases = ((torch.randn(n_seq, seq, 1, generator=gen), {}),
+             (torch.randn(1, total, 1, generator=gen), dict(use_remove_padding=True, seqlens_in_batch=seqlens,
+                                                            cu_seqlens_padded=cu, seq_len=seq)))
+    for out_cpu, kw in cases:
+        for dyn in ({}, dict(use_dynamic_bsz=True, actual_micro_batch_size=4)):
+            zo = out_cpu.clone().requires_grad_()
+            want, want_stats = o_loss.critic_compute_loss(zo, b, 0.3, **kw, **dyn)
+            (g_o,) = torch.autograd.grad(want, zo)
+            zd = out_cpu.to(dev).requires_grad_()
+            got, stats = crit.compute_loss(zd, _to_dev(b, dev), **_to_dev(kw, dev), **dyn)
+            assert got.item() == pytest.approx(want.item(), rel=TOL_LOSS_REL)
+            for k in want_stats:
+                assert stats[k] == pytest.approx(want_stats[k], rel=TOL_LOSS_REL, abs=1e-8), k
+            (g,) = torch.autograd.grad(got, zd)
+            assert g.shape == out_cpu.shape and (g.cpu() - g_o).abs().max().item() < 1e-6
+        vpreds = crit.compute_loss(out_cpu.to(dev), _to_dev(b, dev), forward_only=True, **_to_dev(kw, dev))
+        assert torch.equal(vpreds.cpu(), o_loss.critic_compute_loss(out_cpu, b, 0.3, forward_only=True, **kw))
+
+
 # --------------------------------------------------------------------------------- advantages
 def test_group_advantage_parity(dev, reference_vectors):
     v = reference_vectors["group_norm_advantage"]

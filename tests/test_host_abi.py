@@ -95,6 +95,16 @@ def test_argument_validation_launches_nothing():
     assert lib.mrl_lmhead_logprob_fwd(p, p, 4, 1000, 100, p, _lib.I64, 1.0, p, None, None, p, 1 << 20, None) != 0
     assert lib.mrl_lmhead_logprob_fwd(p, p, 4, 1000, 128, p, _lib.I64, 1.0, p, None, None, p, 16, None) != 0
     assert b"workspace" in lib.mrl_last_error()
+    # PPO value side
+    assert lib.mrl_gae_scan(p, p + 512, 2, 8, 1.0, 0.95, p, p + 1024, None) == -1 and b"alias" in lib.mrl_last_error()
+    assert lib.mrl_gae_scan(p, p + 512, 2, 0, 1.0, 0.95, p + 1024, p + 2048, None) == -1
+    assert lib.mrl_gae_scan(None, None, 0, 8, 1.0, 0.95, None, None, None) == 0
+    assert lib.mrl_kl_token_rewards(p, p, p, _lib.I64, p, 2, 8, 0, 0.1, p, p, None) == -1   # no such penalty
+    assert lib.mrl_kl_token_rewards(p, p, p, _lib.F32, p, 2, 8, 1, 0.1, p, p, None) == -2   # lengths dtype
+    assert lib.mrl_masked_whiten(p, p, _lib.F64, 8, 1, p, p, None) == -2
+    assert lib.mrl_masked_whiten(p, p, _lib.F32, 8, 1, p, None, None) == -1
+    assert lib.mrl_value_loss_fwd(p, p, p, None, 0, None, 0, 2, 4, 0.5, 1.0, p, None) == -1  # no mask, no lengths
+    assert lib.mrl_value_loss_bwd(p, p, p, p, _lib.F32, None, 0, 2, 4, 0.5, 1.0, p, None, p, None) == -1
     # bandwidth probe
     assert lib.mrl_bandwidth_probe(3, p, p, 1, 1024, None) == -1
     assert lib.mrl_bandwidth_probe(2, p, p, 1, 1000, None) == -1
@@ -119,6 +129,7 @@ def test_registry_contract(reference_vectors):
     key = reference_vectors["dapo_defaults"]["registry_key"]
     assert isinstance(mrl.LossFuncFactory.get_instance(*key), mrl.DAPOActorLossFunc)
     assert isinstance(mrl.LossFuncFactory.get_instance("ray_ppo", "actor"), mrl.PPOActorLossFunc)
+    assert isinstance(mrl.LossFuncFactory.get_instance("ray_ppo", "critic"), mrl.CriticLossFunc)
     assert isinstance(mrl.LossFuncFactory.get_instance("ray_grpo", "reference"), mrl.ReferenceLossFunc)
     assert isinstance(mrl.LossFuncFactory.get_instance("ray_ppo", "reference"), mrl.ReferenceLossFunc)
     assert mrl.LossFuncFactory.get_instance("nope", "actor") is None

@@ -438,3 +438,97 @@ def test_wire_format_reference_vectors():
         packing.pack_experience_columns("actor_train", samples, 3)
     with pytest.raises(ValueError):
         packing.pack_experience_columns("actor_train", {}, 0)
+
+
+# --------------------------------------------------------------------------------- PPO value side
+def test_value_side_reference_vectors(reference_vectors):
+    """masked_var / masked_whiten (tests/ut/utils/test_torch_functional.py:36-55), GAE and the adaptive
+    KL controller (tests/ut/utils/test_compute_utils.py:7-58), critic defaults and the no-clipping case
+    (tests/ut/models/loss/test_critic_loss_func.py:28-141)."""
+    v = reference_vectors["masked_var"]
+    got = loss.masked_var(torch.tensor(v["values"]), torch.tensor(v["mask"]), unbiased=True)
+    assert torch.isclose(got, torch.tensor(v["expected"]), atol=v["atol"])
+    w = reference_vectors["masked_whiten"]
+    got = loss.masked_whiten(torch.tensor(w["values"]), torch.tensor(w["mask"]))
+    assert torch.allclose(got, torch.tensor(w["expected"]), atol=w["atol"])
+    g = reference_vectors["gae"]
+    adv, ret = advantage.compute_gae_advantage_return(torch.tensor(g["token_level_rewards"]), torch.tensor(g["values"]),
+                                                      torch.tensor(g["eos_mask"]), torch.tensor(g["gamma"]),
+                                                      torch.tensor(g["lam"]))
+    assert torch.equal(adv, torch.tensor(g["expected_advantages"]))
+    assert torch.equal(ret, torch.tensor(g["expected_returns"]))
+    a = reference_vectors["adaptive_kl"]
+    for case in a["cases"]:
+        ctrl = advantage.AdaptiveKLController(a["init_kl_coef"], a["target_kl"], a["horizon"])
+        ctrl.update(case["current_kl"], case["n_steps"])
+        assert ctrl.value == case["expected"]
+    c = reference_vectors["critic"]["no_clipping"]
+    vf, frac = loss.value_loss(torch.tensor(c["vpreds"]), torch.tensor(c["returns"]), torch.tensor(c["values"]),
+                               torch.tensor(c["response_mask"], dtype=torch.float32), c["cliprange_value"])
+    assert frac.item() == c["expected_clipfrac"] and vf.item() == 0.0
+    c = reference_vectors["critic"]["generic"]
+    vf, frac = loss.value_loss(torch.tensor(c["vpreds"]), torch.tensor(c["returns"]), torch.tensor(c["values"]),
+                               torch.tensor(c["response_mask"], dtype=torch.float32), c["cliprange_value"])
+    # every masked error is 0.1: 0.5 * mean(0.01); vpreds == values, so nothing is clipped
+    assert vf.item() == pytest.approx(0.005, rel=1e-5) and frac.item() == 0.0
+
+
+def test_value_side_closed_forms():
+    """What the mathematics fixes: GAE as the discounted sum of TD errors (fp64 brute force), lam = 1
+    gives discounted returns, whitening gives zero masked mean and unit unbiased masked variance, the
+    value loss in its three regimes (inside the clip range, clipped and worse, clipped and better) with
+    the gradient of each, and the KL reward layout."""
+    gen = torch.Generator().manual_seed(3)
+    B, L = 5, 17
+    r = torch.randn(B, L, generator=gen)
+    v = torch.randn(B, L, generator=gen)
+    mask = packing.generate_mask(r, torch.tensor([[17], [1], [9], [16], [2]])).float()
+    gamma, lam = torch.tensor(0.97), torch.tensor(0.9)
+    adv, ret = advantage.compute_gae_advantage_return(r, v, mask, gamma, lam)
+    r64, v64 = r.double(), v.double()
+    vn = torch.cat([v64[:, 1:], torch.zeros(B, 1, dtype=torch.float64)], 1)
+    delta = r64 + 0.97 * vn - v64
+    raw = torch.zeros(B, L, dtype=torch.float64)
+    for t in range(L):
+        for k in range(t, L):
+            raw[:, t] += (float(gamma) * float(lam)) ** (k - t) * delta[:, k]
+    assert (ret.double() - (raw + v64)).abs().max().item() < 1e-5
+    want = loss.masked_whiten(raw.float(), mask)
+    assert (adv - want).abs().max().item() < 1e-5
+    n = mask.sum()
+    assert abs((adv * mask).sum().item() / n.item()) < 1e-6
+    assert ((adv * mask) ** 2).sum().item() / (n.item() - 1) == pytest.approx(1.0, rel=1e-4)
+    # lam = 1: returns are the discounted reward-to-go (values cancel)
+    _, ret1 = advantage.compute_gae_advantage_return(r, v, mask, torch.tensor(0.5), torch.tensor(1.0))
+    togo = torch.zeros(B, L, dtype=torch.float64)
+    for t in range(L):
+        for k in range(t, L):
+            togo[:, t] += 0.5 ** (k - t) * r64[:, k]
+    assert (ret1.double() - togo).abs().max().item() < 1e-5
+    # masked_var: biased / unbiased, one-element mask, empty mask raises
+    x = torch.tensor([1.0, 5.0, 100.0])
+    m = torch.tensor([1.0, 1.0, 0.0])
+    assert loss.masked_var(x, m, unbiased=False).item() == pytest.approx(4.0)
+    assert loss.masked_var(x, m).item() == pytest.approx(8.0)
+    assert loss.masked_var(x, torch.tensor([0.0, 1.0, 0.0])).item() == pytest.approx(0.0)
+    with pytest.raises(ValueError):
+        loss.masked_var(x, torch.zeros(3))
+    # value loss regimes, clip 0.5, value 0: vp 0.2 / ret 1 (inside), vp 2 / ret 3 (clipped to 0.5, worse:
+    # takes the clipped error, no gradient), vp 2 / ret 0 (clipped, better: takes the raw error)
+    vp = torch.tensor([[0.2, 2.0, 2.0, 9.0]], requires_grad=True)
+    rt = torch.tensor([[1.0, 3.0, 0.0, 0.0]])
+    vf, frac = loss.value_loss(vp, rt, torch.zeros(1, 4), torch.tensor([[1.0, 1.0, 1.0, 0.0]]), 0.5)
+    assert vf.item() == pytest.approx(0.5 * (0.64 + 6.25 + 4.0) / 3, rel=1e-6)
+    assert frac.item() == pytest.approx(1 / 3, rel=1e-6)
+    (g,) = torch.autograd.grad(vf, vp)
+    assert torch.allclose(g, torch.tensor([[0.5 * 2 * (0.2 - 1.0) / 3, 0.0, 0.5 * 2 * 2.0 / 3, 0.0]]), atol=1e-6)
+    # KL rewards: score at the last response token, -beta * kl elsewhere, nothing past the response
+    old = torch.tensor([[-1.0, -2.0, -3.0], [-1.0, -1.0, -1.0]])
+    ref = torch.tensor([[-1.5, -2.0, -2.0], [-2.0, -2.0, -2.0]])
+    rew, cur = advantage.kl_token_level_rewards(old, ref, torch.tensor([[2], [3]]), torch.tensor([10.0, -4.0]), 0.1, "kl")
+    assert torch.allclose(rew, torch.tensor([[-0.05, 10.0, 0.0], [-0.1, -0.1, -4.1]]), atol=1e-6)
+    assert cur == pytest.approx(0.5 * (0.25 + 1.0), rel=1e-6)
+    out = loss.critic_compute_loss(torch.arange(12.0).view(2, 6, 1), {
+        "responses": torch.zeros(2, 3), "prompt_length": torch.tensor([[2], [1]]),
+        "response_length": torch.tensor([[3], [2]])}, forward_only=True)
+    assert out.squeeze(-1).tolist() == [[1.0, 2.0, 3.0], [6.0, 7.0, 0.0]]
