@@ -1,0 +1,159 @@
+"""Oracle (test infrastructure): token-budget micro-batch partitioning.
+
+Restates ``mindspeed_rl/utils/seqlen_balancing.py`` of the reference:
+
+* ``:12-124``   ``karmarkar_karp`` (largest differencing method on k-tuples of sets, with the
+  reference's tie-breaking: sets ordered by (sum, size, items), states by (spread descending, largest
+  set descending))
+* ``:127-156``  ``heapq_partition`` (longest first onto the lightest group; equal-size variant)
+* ``:159-188``  ``get_seqlen_balanced_partitions``
+* ``:310-336``  ``heapq_partition_with_max`` (a group that would overflow is closed and replaced)
+* ``:339-380``  ``rearrange_micro_batches`` at data-parallel size 1, text-only (the multimodal bin
+  packing branch and the MAX all-reduce of the bin count are not on this path)
+* ``:383-388``  ``get_reverse_idx``
+
+PARITY UNPINNED against reference-held vectors: the reference has no test or fixture for this
+module.  Pinned by textbook results of the differencing method, by brute force over all
+assignments on small inputs, and by the invariants every partitioner must keep.
+"""
+import copy
+import heapq
+
+
+class _Set:
+    def __init__(self):
+        self.sum = 0
+        self.items = []
+
+    def add(self, idx, val):
+        self.items.append((idx, val))
+        self.sum += val
+
+    def merge(self, other):
+        for idx, val in other.items:
+            self.add(idx, val)
+
+    def __lt__(self, other):
+        if self.sum != other.sum:
+            return self.sum < other.sum
+        if len(self.items) != len(other.items):
+            return len(self.items) < len(other.items)
+        return self.items < other.items
+
+
+class _State:
+    def __init__(self, items, k):
+        self.k = k
+        self.sets = [_Set() for _ in range(k)]
+        for i, (idx, seqlen) in enumerate(items):
+            self.sets[i].add(idx, seqlen)
+        self.sets = sorted(self.sets, reverse=True)
+
+    def merge(self, other):
+        for i in range(self.k):
+            self.sets[i].merge(other.sets[self.k - 1 - i])
+        self.sets = sorted(self.sets, reverse=True)
+
+    @property
+    def spread(self):
+        return self.sets[0].sum - self.sets[-1].sum
+
+    def __lt__(self, other):
+        if self.spread != other.spread:
+            return self.spread > other.spread
+        return self.sets[0] > other.sets[0]
+
+
+def karmarkar_karp(seqlen_list, k_partitions, equal_size):
+    ordered = sorted([(seqlen, i) for i, seqlen in enumerate(seqlen_list)])
+    heap = []
+    if equal_size:
+        if len(seqlen_list) % k_partitions != 0:
+            raise ValueError("%d %% %d != 0" % (len(seqlen_list), k_partitions))
+        for offset in range(0, len(ordered), k_partitions):
+            items = [(ordered[offset + i][1], ordered[offset + i][0]) for i in range(k_partitions)]
+            heapq.heappush(heap, _State(items, k_partitions))
+    else:
+        for seqlen, idx in ordered:
+            heapq.heappush(heap, _State([(idx, seqlen)], k_partitions))
+    while len(heap) > 1:
+        first = heapq.heappop(heap)
+        second = heapq.heappop(heap)
+        first.merge(second)
+        heapq.heappush(heap, first)
+    partitions = [[idx for idx, _ in s.items] for s in heap[0].sets]
+    if equal_size:
+        for partition in partitions:
+            if len(partition) * k_partitions != len(seqlen_list):
+                raise ValueError("%d * %d != %d" % (len(partition), k_partitions, len(seqlen_list)))
+    return partitions
+
+
+def heapq_partition(seqlen_list, k_partitions, equal_size):
+    per_group = len(seqlen_list) // k_partitions
+    ordered = sorted([(seqlen, i) for i, seqlen in enumerate(seqlen_list)], reverse=True)
+    groups = [[0, 0, i, []] for i in range(k_partitions)]
+    heapq.heapify(groups)
+    partitions = []
+    for seqlen, i in ordered:
+        group = heapq.heappop(groups)
+        group[3].append(i)
+        group[0] += seqlen
+        group[1] += 1
+        if equal_size:
+            if group[1] < per_group:
+                heapq.heappush(groups, group)
+            else:
+                partitions.append(group[3])
+        else:
+            heapq.heappush(groups, group)
+    partitions.extend([group[3] for group in groups])
+    if equal_size:
+        for i, partition in enumerate(partitions):
+            if len(partition) * k_partitions != len(seqlen_list):
+                raise ValueError("Partition %d has %d items, expected %d" % (i, len(partition), per_group))
+    return partitions
+
+
+def get_seqlen_balanced_partitions(seqlen_list, k_partitions, equal_size):
+    if k_partitions > len(seqlen_list):
+        raise ValueError("number of items:[%d] < k_partitions:[%d]" % (len(seqlen_list), k_partitions))
+    partitions = heapq_partition(seqlen_list, k_partitions, equal_size)
+    return [sorted(p) for p in partitions]
+
+
+def heapq_partition_with_max(seqlen_list, k_partitions, max_token_len):
+    ordered = sorted([(seqlen, i) for i, seqlen in enumerate(seqlen_list)], reverse=True)
+    groups = [[0, 0, i, []] for i in range(k_partitions)]
+    group_num = len(groups)
+    heapq.heapify(groups)
+    partitions = []
+    for seqlen, i in ordered:
+        group = heapq.heappop(groups)
+        if group[0] + seqlen > max_token_len:
+            partitions.append(group[3])
+            heapq.heappush(groups, [seqlen, 1, group_num, [i]])
+            group_num += 1
+        else:
+            group[0] += seqlen
+            group[1] += 1
+            group[3].append(i)
+            heapq.heappush(groups, group)
+    partitions.extend([group[3] for group in groups])
+    return partitions
+
+
+def rearrange_micro_batches(seqlen_list, max_token_len, dynamic_max_batch_size=None, dp_group=None):
+    total = sum(seqlen_list)
+    k_partitions = (total + max_token_len - 1) // max_token_len
+    k_partitions = len(heapq_partition_with_max(seqlen_list, k_partitions, max_token_len))
+    if dynamic_max_batch_size is not None:
+        k_partitions = max(k_partitions, (len(seqlen_list) + dynamic_max_batch_size - 1) // dynamic_max_batch_size)
+    return karmarkar_karp(seqlen_list, k_partitions, equal_size=False)
+
+
+def get_reverse_idx(idx_map):
+    reverse = copy.deepcopy(idx_map)
+    for i, idx in enumerate(idx_map):
+        reverse[idx] = i
+    return reverse
