@@ -15,6 +15,8 @@
 // Vocabulary groups (gridDim = token tiles x groups, group = blockIdx % groups so that the
 // workgroups of one XCD read the same W rows) leave per-group partial statistics that a small
 // second kernel merges, together with the label logit (one fp32 dot product per token).
+#include <stdlib.h>
+
 #include "mrl_internal.h"
 #include "vocab_common.h"
 
@@ -186,6 +188,203 @@ __global__ __launch_bounds__(kThreads, (kTB <= 2 ? 2 : 1)) void lmhead_fwd_kerne
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// Second generation of the tile loop: a 512-thread workgroup (2 x 4 wavefronts, one workgroup per
+// CU) owns 256 vocabulary rows x 256 tokens, so each wavefront keeps the 128 x 64 sub-tile of the
+// kernel above but every staged byte feeds twice the MFMA work.  Operands go from global memory
+// straight into LDS (global_load_lds_dwordx4: no staging registers, no ds_write), into one of two
+// stage buffers, so the loads of k-step s+1 run during the MFMAs of k-step s and a k-step costs
+// ONE barrier.  A direct load puts lane i of a wavefront at LDS byte base + 16 i, which rules out
+// padded rows; instead the 16-byte chunks are XOR-swizzled inside each 256-byte pair of rows:
+//   physical slot (0..15) = logical slot ^ (pair index & 15),  logical slot = (row & 1) * 8 + chunk
+// The 16 lanes that a ds_read_b128 serves together read 16 consecutive rows at one chunk, i.e. 8
+// pairs x 2 rows -> 16 different slots -> all 64 banks, no conflict.  The loop runs over the
+// flattened (vocabulary tile, k-step) sequence, so the first loads of the next tile are in flight
+// during the softmax statistics of the current one.
+constexpr int kThreads2 = 512;
+constexpr int BT2 = 256;                         // tokens per workgroup
+constexpr int kOperandBytes = 256 * BK * 2;      // one operand of one stage: 256 rows x 128 bytes
+constexpr int kStageBytes = 2 * kOperandBytes;   // A (weights) then B (hidden)
+constexpr int kLdsBytes2 = 2 * kStageBytes;      // two stages
+
+// Global element offset (row * hdim + column, without the k-step) of the chunk that lane `lane`
+// of wavefront `wave` brings in with its load j (0..3) of an operand whose tile has `rows_valid`
+// rows left (rows beyond are clamped to the last valid one and masked later).
+__device__ __forceinline__ int stage_src_offset(int wave, int lane, int j, int hdim, int rows_valid) {
+    const int phys_row = (wave * 4 + j) * 8 + (lane >> 3);
+    const int pair = phys_row >> 1;
+    const int slot = ((phys_row & 1) << 3) | (lane & 7);
+    const int logical = slot ^ (pair & 15);
+    int row = 2 * pair + (logical >> 3);
+    if (row >= rows_valid) row = rows_valid - 1;
+    return row * hdim + (logical & 7) * 8;
+}
+
+__global__ __launch_bounds__(kThreads2, 1) void lmhead_fwd_kernel_v2(
+    const uint16_t* __restrict__ hidden, const uint16_t* __restrict__ weight, int64_t n_tokens, int vocab, int hdim,
+    int n_groups, int tiles_per_group, float k_scale, float* __restrict__ partial) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    __shared__ Stats comb[4][2][32];             // [token wavefront][token block][lane % 32]
+    constexpr int kTB = 2;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wv = wave >> 2, wt = wave & 3;
+    const int group = blockIdx.x % n_groups;
+    const int64_t t0 = (int64_t)(blockIdx.x / n_groups) * BT2;
+    const int n_vtiles = (vocab + BV - 1) / BV;
+    const int tile_begin = group * tiles_per_group;
+    const int tile_end = min(tile_begin + tiles_per_group, n_vtiles);
+    const int n_ksteps = hdim / BK;
+
+    // sources of this lane's four chunks per operand and stage
+    const uint16_t* b_base = hidden + t0 * hdim;
+    const int tokens_valid = (int)min((int64_t)BT2, n_tokens - t0);
+    int b_off[4], a_off[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) b_off[j] = stage_src_offset(wave, lane, j, hdim, tokens_valid);
+
+    auto issue = [&](int tile, int kstep, int buf) {
+        const uint16_t* a_src = weight + (int64_t)tile * BV * hdim + kstep * BK;
+        const uint16_t* b_src = b_base + kstep * BK;
+        unsigned char* dst = smem + buf * kStageBytes + (wave * 4) * 1024;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            __builtin_amdgcn_global_load_lds(
+                (const void __attribute__((address_space(1)))*)(a_src + a_off[j]),
+                (void __attribute__((address_space(3)))*)(dst + j * 1024), 16, 0, 0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            __builtin_amdgcn_global_load_lds(
+                (const void __attribute__((address_space(1)))*)(b_src + b_off[j]),
+                (void __attribute__((address_space(3)))*)(dst + kOperandBytes + j * 1024), 16, 0, 0);
+    };
+    auto set_a_rows = [&](int tile) {
+        const int rows_valid = min(BV, vocab - tile * BV);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) a_off[j] = stage_src_offset(wave, lane, j, hdim, rows_valid);
+    };
+
+    // fragment addresses: row (lane & 31) of a 32-row block, chunk 2 ks + (lane >> 5)
+    const int frag_pair = (lane & 31) >> 1;
+    const int frag_slot = (((lane & 1) << 3) | (lane >> 5)) ^ frag_pair;          // ^ (2 ks) per k sub-step
+    const int a_frag = (wv * 64) * 256 + frag_pair * 256;                          // + vb * 16 * 256
+    const int b_frag = kOperandBytes + (wt * 32) * 256 + frag_pair * 256;          // + tb * 16 * 256
+
+    Stats st[kTB];
+#pragma unroll
+    for (int tb = 0; tb < kTB; ++tb) st[tb] = {kMaxInit, 0.f, 0.f};
+
+    int next_tile = tile_begin, next_k = 0, buf = 0;
+    if (next_tile < tile_end) {
+        set_a_rows(next_tile);
+        issue(next_tile, 0, 0);
+        if (++next_k == n_ksteps) {
+            next_k = 0;
+            ++next_tile;
+        }
+    }
+    for (int tile = tile_begin; tile < tile_end; ++tile) {
+        const int v0 = tile * BV;
+        floatx16 acc[4][kTB];
+#pragma unroll
+        for (int vb = 0; vb < 4; ++vb)
+#pragma unroll
+            for (int tb = 0; tb < kTB; ++tb)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc[vb][tb][i] = 0.f;
+
+        for (int kstep = 0; kstep < n_ksteps; ++kstep) {
+            // this stage has landed (every wavefront waits for its own loads, then for the others),
+            // and nobody still reads the other buffer
+            __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0)
+            __syncthreads();
+            if (next_tile < tile_end) {
+                if (next_k == 0) set_a_rows(next_tile);
+                issue(next_tile, next_k, buf ^ 1);
+                if (++next_k == n_ksteps) {
+                    next_k = 0;
+                    ++next_tile;
+                }
+            }
+            const unsigned char* stage = smem + buf * kStageBytes;
+#pragma unroll
+            for (int ks = 0; ks < BK / 16; ++ks) {
+                const int slot_bytes = (frag_slot ^ (2 * ks)) * 16;
+                bf16x8 af[4], bfr[kTB];
+#pragma unroll
+                for (int vb = 0; vb < 4; ++vb)
+                    af[vb] = *reinterpret_cast<const bf16x8*>(stage + a_frag + vb * 16 * 256 + slot_bytes);
+#pragma unroll
+                for (int tb = 0; tb < kTB; ++tb)
+                    bfr[tb] = *reinterpret_cast<const bf16x8*>(stage + b_frag + tb * 16 * 256 + slot_bytes);
+#pragma unroll
+                for (int vb = 0; vb < 4; ++vb)
+#pragma unroll
+                    for (int tb = 0; tb < kTB; ++tb)
+                        acc[vb][tb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[vb], bfr[tb], acc[vb][tb], 0, 0, 0);
+            }
+            buf ^= 1;
+        }
+
+        // online softmax statistics of this tile: a lane holds 64 vocabulary rows of each token column
+        const bool ragged = (v0 + BV > vocab);
+#pragma unroll
+        for (int tb = 0; tb < kTB; ++tb) {
+            if (ragged) {
+#pragma unroll
+                for (int vb = 0; vb < 4; ++vb)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const int v = v0 + wv * 128 + vb * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
+                        if (v >= vocab) acc[vb][tb][i] = kMaxInit;
+                    }
+            }
+            float vmax = st[tb].m;
+#pragma unroll
+            for (int vb = 0; vb < 4; ++vb)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) vmax = fmaxf(vmax, acc[vb][tb][i]);
+            grow_max<true>(st[tb], vmax, k_scale);
+            const float mk = st[tb].m * k_scale;
+#pragma unroll
+            for (int vb = 0; vb < 4; ++vb)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) add_one<true>(st[tb], acc[vb][tb][i], k_scale, mk);
+        }
+    }
+
+    // combine the two lane halves (same token, other vocabulary rows), then the two vocabulary wavefronts
+#pragma unroll
+    for (int tb = 0; tb < kTB; ++tb) {
+        Stats o;
+        o.m = __shfl_xor(st[tb].m, 32, 64);
+        o.s = __shfl_xor(st[tb].s, 32, 64);
+        o.u = __shfl_xor(st[tb].u, 32, 64);
+        st[tb] = merge<true>(st[tb], o, k_scale);
+    }
+    __syncthreads();
+    if (wv == 1 && lane < 32) {
+#pragma unroll
+        for (int tb = 0; tb < kTB; ++tb) comb[wt][tb][lane] = st[tb];
+    }
+    __syncthreads();
+    if (wv == 0 && lane < 32) {
+#pragma unroll
+        for (int tb = 0; tb < kTB; ++tb) {
+            const Stats r = merge<true>(st[tb], comb[wt][tb][lane], k_scale);
+            const int64_t t = t0 + wt * 64 + tb * 32 + lane;
+            if (t < n_tokens) {
+                float* p = partial + ((int64_t)group * n_tokens + t) * 4;
+                p[0] = r.m;
+                p[1] = r.s;
+                p[2] = r.u;
+                p[3] = 0.f;
+            }
+        }
+    }
+}
+
 // One wavefront per token: merges the per-group partial statistics and computes the label logit
 // as an fp32 dot product of the token's hidden row with the label's weight row.
 template <typename LabelT>
@@ -229,6 +428,15 @@ __global__ __launch_bounds__(256) void lmhead_finish_kernel(
     }
 }
 
+// MRL_LMHEAD_V2=0 selects the first-generation tile loop (a tuning / debugging switch).
+bool lmhead_v2_enabled() {
+    static const bool on = [] {
+        const char* e = getenv("MRL_LMHEAD_V2");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
 }  // namespace
 
 extern "C" int64_t mrl_lmhead_workspace_bytes(int64_t n_tokens, int64_t vocab) {
@@ -261,17 +469,29 @@ extern "C" int mrl_lmhead_logprob_fwd(const void* hidden, const void* weight, in
     const int n_groups = MRL_LMHEAD_GROUPS;
     const int n_vtiles = (int)((vocab + BV - 1) / BV);
     const int tiles_per_group = (n_vtiles + n_groups - 1) / n_groups;
-    // 128-token tiles (4x2 MFMA blocks per wavefront, two workgroups per CU); a 256-token tile with the
-    // accumulators in AGPRs measured slower (758 vs 916 TFLOP/s at 32k tokens) and is not instantiated
-    constexpr int kTokenBlocks = 2;
-    const int64_t n_ttiles = (n_tokens + 64 * kTokenBlocks - 1) / (64 * kTokenBlocks);
-    MRL_REQUIRE(n_ttiles * n_groups <= 0x7fffffffLL, MRL_ERR_UNSUPPORTED, "%s: grid too large", fn);
     hipStream_t s = mrl::as_stream(stream);
     float* partial = (float*)workspace;
     // a group without tiles (tiny vocabularies) still writes its neutral partials
-    hipLaunchKernelGGL(lmhead_fwd_kernel<kTokenBlocks>, dim3((unsigned)(n_ttiles * n_groups)), dim3(kThreads), 0, s,
-                       (const uint16_t*)hidden, (const uint16_t*)weight, n_tokens, (int)vocab, (int)hidden_dim,
-                       n_groups, tiles_per_group, inv_temperature * kLog2e, partial);
+    if (lmhead_v2_enabled()) {
+        // 256-token tiles, operands straight into two LDS stages (128 KiB of dynamic LDS)
+        static const hipError_t attr = hipFuncSetAttribute((const void*)lmhead_fwd_kernel_v2,
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes2);
+        MRL_REQUIRE(attr == hipSuccess, MRL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", fn, kLdsBytes2,
+                    hipGetErrorString(attr));
+        const int64_t n_ttiles = (n_tokens + BT2 - 1) / BT2;
+        MRL_REQUIRE(n_ttiles * n_groups <= 0x7fffffffLL, MRL_ERR_UNSUPPORTED, "%s: grid too large", fn);
+        hipLaunchKernelGGL(lmhead_fwd_kernel_v2, dim3((unsigned)(n_ttiles * n_groups)), dim3(kThreads2), kLdsBytes2, s,
+                           (const uint16_t*)hidden, (const uint16_t*)weight, n_tokens, (int)vocab, (int)hidden_dim,
+                           n_groups, tiles_per_group, inv_temperature * kLog2e, partial);
+    } else {
+        // 128-token tiles (4x2 MFMA blocks per wavefront, two workgroups per CU), operands staged through registers
+        constexpr int kTokenBlocks = 2;
+        const int64_t n_ttiles = (n_tokens + 64 * kTokenBlocks - 1) / (64 * kTokenBlocks);
+        MRL_REQUIRE(n_ttiles * n_groups <= 0x7fffffffLL, MRL_ERR_UNSUPPORTED, "%s: grid too large", fn);
+        hipLaunchKernelGGL(lmhead_fwd_kernel<kTokenBlocks>, dim3((unsigned)(n_ttiles * n_groups)), dim3(kThreads), 0, s,
+                           (const uint16_t*)hidden, (const uint16_t*)weight, n_tokens, (int)vocab, (int)hidden_dim,
+                           n_groups, tiles_per_group, inv_temperature * kLog2e, partial);
+    }
     int rc = mrl::check_launch(fn);
     if (rc != MRL_OK) return rc;
     const dim3 fgrid((unsigned)((n_tokens + 3) / 4)), fblock(256);
