@@ -244,20 +244,24 @@ __global__ __launch_bounds__(kThreads2, 1) void lmhead_fwd_kernel_v2(
 #pragma unroll
     for (int j = 0; j < 4; ++j) b_off[j] = stage_src_offset(wave, lane, j, hdim, tokens_valid);
 
+    // Buffer (MUBUF) form of the LDS load on purpose: the global_load_lds form is a FLAT instruction
+    // that touches two address spaces, and while one is pending the compiler turns every LDS wait
+    // into lgkmcnt(0), which would undo the fragment pipeline below.
+    const mrl::rsrc_t w_rsrc = mrl::make_rsrc(weight, 0xffffffffu);
+    const mrl::rsrc_t h_rsrc = mrl::make_rsrc(b_base, 0xffffffffu);
     auto issue = [&](int tile, int kstep, int buf) {
-        const uint16_t* a_src = weight + (int64_t)tile * BV * hdim + kstep * BK;
-        const uint16_t* b_src = b_base + kstep * BK;
+        const uint32_t a_tile = (uint32_t)(((int64_t)tile * BV * hdim + kstep * BK) * 2);
+        const uint32_t b_tile = (uint32_t)(kstep * BK * 2);
         unsigned char* dst = smem + buf * kStageBytes + (wave * 4) * 1024;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            __builtin_amdgcn_global_load_lds(
-                (const void __attribute__((address_space(1)))*)(a_src + a_off[j]),
-                (void __attribute__((address_space(3)))*)(dst + j * 1024), 16, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (void __attribute__((address_space(3)))*)(dst + j * 1024), 16,
+                                                 a_off[j] * 2, a_tile, 0, 0);
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            __builtin_amdgcn_global_load_lds(
-                (const void __attribute__((address_space(1)))*)(b_src + b_off[j]),
-                (void __attribute__((address_space(3)))*)(dst + kOperandBytes + j * 1024), 16, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(h_rsrc,
+                                                 (void __attribute__((address_space(3)))*)(dst + kOperandBytes + j * 1024),
+                                                 16, b_off[j] * 2, b_tile, 0, 0);
     };
     auto set_a_rows = [&](int tile) {
         const int rows_valid = min(BV, vocab - tile * BV);
@@ -275,82 +279,114 @@ __global__ __launch_bounds__(kThreads2, 1) void lmhead_fwd_kernel_v2(
 #pragma unroll
     for (int tb = 0; tb < kTB; ++tb) st[tb] = {kMaxInit, 0.f, 0.f};
 
-    int next_tile = tile_begin, next_k = 0, buf = 0;
-    if (next_tile < tile_end) {
-        set_a_rows(next_tile);
-        issue(next_tile, 0, 0);
+    // The (tile, k-step) stages are numbered 0 .. n_stages-1; stage s lives in buffer s & 1.
+    const int n_stages = (tile_end > tile_begin ? tile_end - tile_begin : 0) * n_ksteps;
+    int next_tile = tile_begin, next_k = 0;      // the stage that is requested next
+    auto issue_next = [&](int buf) {
+        if (next_k == 0) set_a_rows(next_tile);
+        issue(next_tile, next_k, buf);
         if (++next_k == n_ksteps) {
             next_k = 0;
             ++next_tile;
         }
-    }
-    for (int tile = tile_begin; tile < tile_end; ++tile) {
-        const int v0 = tile * BV;
-        floatx16 acc[4][kTB];
+    };
+    struct Frags {
+        bf16x8 a[4], b[kTB];
+    };
+    auto read_frags = [&](Frags& f, const unsigned char* stage, int ks) {
+        const int slot_bytes = (frag_slot ^ (2 * ks)) * 16;
+#pragma unroll
+        for (int vb = 0; vb < 4; ++vb)
+            f.a[vb] = *reinterpret_cast<const bf16x8*>(stage + a_frag + vb * 16 * 256 + slot_bytes);
+#pragma unroll
+        for (int tb = 0; tb < kTB; ++tb)
+            f.b[tb] = *reinterpret_cast<const bf16x8*>(stage + b_frag + tb * 16 * 256 + slot_bytes);
+    };
+    floatx16 acc[4][kTB];
+    auto zero_acc = [&]() {
 #pragma unroll
         for (int vb = 0; vb < 4; ++vb)
 #pragma unroll
             for (int tb = 0; tb < kTB; ++tb)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) acc[vb][tb][i] = 0.f;
+    };
+    auto mma = [&](const Frags& f) {
+#pragma unroll
+        for (int vb = 0; vb < 4; ++vb)
+#pragma unroll
+            for (int tb = 0; tb < kTB; ++tb)
+                acc[vb][tb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[vb], f.b[tb], acc[vb][tb], 0, 0, 0);
+    };
 
-        for (int kstep = 0; kstep < n_ksteps; ++kstep) {
-            // this stage has landed (every wavefront waits for its own loads, then for the others),
-            // and nobody still reads the other buffer
-            __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0)
-            __syncthreads();
-            if (next_tile < tile_end) {
-                if (next_k == 0) set_a_rows(next_tile);
-                issue(next_tile, next_k, buf ^ 1);
-                if (++next_k == n_ksteps) {
-                    next_k = 0;
-                    ++next_tile;
-                }
-            }
+    if (n_stages > 0) {
+        Frags f0, f1;
+        issue_next(0);
+        __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0): stage 0 has landed
+        __syncthreads();
+        if (n_stages > 1) issue_next(1);
+        read_frags(f0, smem, 0);
+        zero_acc();
+        int tile = tile_begin, kstep = 0;
+        for (int stage_idx = 0; stage_idx < n_stages; ++stage_idx) {
+            const int buf = stage_idx & 1;
             const unsigned char* stage = smem + buf * kStageBytes;
+            // software pipeline: the fragments of sub-step ks+1 are requested before the MFMAs of ks
+            read_frags(f1, stage, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(f0);
+            __builtin_amdgcn_sched_barrier(0);
+            read_frags(f0, stage, 2);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(f1);
+            __builtin_amdgcn_sched_barrier(0);
+            read_frags(f1, stage, 3);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(f0);
+            __builtin_amdgcn_sched_barrier(0);
+            // The last fragments of this stage are in registers and the next stage has landed: after
+            // the barrier this buffer may be overwritten, and the first fragments of the next stage are
+            // requested before the last MFMAs of this one are issued.  The barrier and the read are
+            // unconditional (after the last stage the read fetches unused bytes of the other buffer): a
+            // branch around them would make the wait before the MFMAs cover the new request as well.
+            __builtin_amdgcn_s_waitcnt(0x0070);            // vmcnt(0) lgkmcnt(0)
+            __syncthreads();
+            if (stage_idx + 2 < n_stages) issue_next(buf);
+            read_frags(f0, smem + (buf ^ 1) * kStageBytes, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(f1);
+            __builtin_amdgcn_sched_barrier(0);
+            if (++kstep == n_ksteps) {
+                // online softmax statistics of this tile: a lane holds 64 vocabulary rows of each token column
+                const int v0 = tile * BV;
+                const bool ragged = (v0 + BV > vocab);
 #pragma unroll
-            for (int ks = 0; ks < BK / 16; ++ks) {
-                const int slot_bytes = (frag_slot ^ (2 * ks)) * 16;
-                bf16x8 af[4], bfr[kTB];
+                for (int tb = 0; tb < kTB; ++tb) {
+                    if (ragged) {
 #pragma unroll
-                for (int vb = 0; vb < 4; ++vb)
-                    af[vb] = *reinterpret_cast<const bf16x8*>(stage + a_frag + vb * 16 * 256 + slot_bytes);
+                        for (int vb = 0; vb < 4; ++vb)
 #pragma unroll
-                for (int tb = 0; tb < kTB; ++tb)
-                    bfr[tb] = *reinterpret_cast<const bf16x8*>(stage + b_frag + tb * 16 * 256 + slot_bytes);
-#pragma unroll
-                for (int vb = 0; vb < 4; ++vb)
-#pragma unroll
-                    for (int tb = 0; tb < kTB; ++tb)
-                        acc[vb][tb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[vb], bfr[tb], acc[vb][tb], 0, 0, 0);
-            }
-            buf ^= 1;
-        }
-
-        // online softmax statistics of this tile: a lane holds 64 vocabulary rows of each token column
-        const bool ragged = (v0 + BV > vocab);
-#pragma unroll
-        for (int tb = 0; tb < kTB; ++tb) {
-            if (ragged) {
-#pragma unroll
-                for (int vb = 0; vb < 4; ++vb)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const int v = v0 + wv * 128 + vb * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
-                        if (v >= vocab) acc[vb][tb][i] = kMaxInit;
+                            for (int i = 0; i < 16; ++i) {
+                                const int v = v0 + wv * 128 + vb * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
+                                if (v >= vocab) acc[vb][tb][i] = kMaxInit;
+                            }
                     }
+                    float vmax = st[tb].m;
+#pragma unroll
+                    for (int vb = 0; vb < 4; ++vb)
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) vmax = fmaxf(vmax, acc[vb][tb][i]);
+                    grow_max<true>(st[tb], vmax, k_scale);
+                    const float mk = st[tb].m * k_scale;
+#pragma unroll
+                    for (int vb = 0; vb < 4; ++vb)
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) add_one<true>(st[tb], acc[vb][tb][i], k_scale, mk);
+                }
+                zero_acc();
+                kstep = 0;
+                ++tile;
             }
-            float vmax = st[tb].m;
-#pragma unroll
-            for (int vb = 0; vb < 4; ++vb)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) vmax = fmaxf(vmax, acc[vb][tb][i]);
-            grow_max<true>(st[tb], vmax, k_scale);
-            const float mk = st[tb].m * k_scale;
-#pragma unroll
-            for (int vb = 0; vb < 4; ++vb)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) add_one<true>(st[tb], acc[vb][tb][i], k_scale, mk);
         }
     }
 
@@ -472,7 +508,8 @@ extern "C" int mrl_lmhead_logprob_fwd(const void* hidden, const void* weight, in
     hipStream_t s = mrl::as_stream(stream);
     float* partial = (float*)workspace;
     // a group without tiles (tiny vocabularies) still writes its neutral partials
-    if (lmhead_v2_enabled()) {
+    // the second-generation loop addresses the weights with 32-bit byte offsets
+    if (lmhead_v2_enabled() && vocab * hidden_dim * 2 < (1LL << 32)) {
         // 256-token tiles, operands straight into two LDS stages (128 KiB of dynamic LDS)
         static const hipError_t attr = hipFuncSetAttribute((const void*)lmhead_fwd_kernel_v2,
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes2);
