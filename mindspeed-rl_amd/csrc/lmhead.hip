@@ -230,8 +230,16 @@ __global__ __launch_bounds__(kThreads2, 1) void lmhead_fwd_kernel_v2(
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wv = wave >> 2, wt = wave & 3;
-    const int group = blockIdx.x % n_groups;
-    const int64_t t0 = (int64_t)(blockIdx.x / n_groups) * BT2;
+    // Workgroups are dealt round-robin to the 8 XCDs and one round of 256 fills the chip.  The 32
+    // workgroups that share an XCD (and its L2) in a round are 4 token tiles x 8 vocabulary groups:
+    // the 8 that stream the same hidden block and the 4 that stream the same weight tiles run side
+    // by side, so most of both streams hits in L2 (with one vocabulary group per XCD every
+    // workgroup re-read its own hidden block from beyond the L2 for each vocabulary tile).
+    const int xcd = blockIdx.x & 7, slot = (blockIdx.x >> 3) & 31, round = blockIdx.x >> 8;
+    const int group = slot & 7;
+    const int64_t ttile = (int64_t)(round * 8 + xcd) * 4 + (slot >> 3);
+    const int64_t t0 = ttile * BT2;
+    if (t0 >= n_tokens) return;                 // padding of the last round
     const int n_vtiles = (vocab + BV - 1) / BV;
     const int tile_begin = group * tiles_per_group;
     const int tile_end = min(tile_begin + tiles_per_group, n_vtiles);
@@ -516,8 +524,10 @@ extern "C" int mrl_lmhead_logprob_fwd(const void* hidden, const void* weight, in
         MRL_REQUIRE(attr == hipSuccess, MRL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", fn, kLdsBytes2,
                     hipGetErrorString(attr));
         const int64_t n_ttiles = (n_tokens + BT2 - 1) / BT2;
-        MRL_REQUIRE(n_ttiles * n_groups <= 0x7fffffffLL, MRL_ERR_UNSUPPORTED, "%s: grid too large", fn);
-        hipLaunchKernelGGL(lmhead_fwd_kernel_v2, dim3((unsigned)(n_ttiles * n_groups)), dim3(kThreads2), kLdsBytes2, s,
+        const int64_t n_rounds = (n_ttiles + 31) / 32;       // 32 token tiles x 8 groups per round of 256 workgroups
+        MRL_REQUIRE(n_rounds * 256 <= 0x7fffffffLL, MRL_ERR_UNSUPPORTED, "%s: grid too large", fn);
+        static_assert(MRL_LMHEAD_GROUPS == 8, "the workgroup mapping assumes 8 vocabulary groups");
+        hipLaunchKernelGGL(lmhead_fwd_kernel_v2, dim3((unsigned)(n_rounds * 256)), dim3(kThreads2), kLdsBytes2, s,
                            (const uint16_t*)hidden, (const uint16_t*)weight, n_tokens, (int)vocab, (int)hidden_dim,
                            n_groups, tiles_per_group, inv_temperature * kLog2e, partial);
     } else {
