@@ -220,7 +220,7 @@ def run_lmhead(args):
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "configs[3] forward: hidden [%d,3584] x W [152064,3584]^T, online logsumexp, logits never "
                                "stored" % tokens, "accumulate": "f32"},
-        "roofline": {"kernel": "lmhead_fwd_kernel + lmhead_finish_kernel (mrl_lmhead_logprob_fwd)", "bound": "mfma",
+        "roofline": {"kernel": "lmhead_fwd_kernel_v2 + lmhead_finish_kernel (mrl_lmhead_logprob_fwd)", "bound": "mfma",
                      "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "flops_per_launch": flops, "avg_ms": ms},
         "max_abs_err_vs_fp32_gemm_256_rows": err,
