@@ -127,7 +127,7 @@ def build_device_batch(torch, mrl, w, plen, rlen, rewards, dev, seed):
     return logits, b, kw, total
 
 
-def cpu_baseline(torch, w, rows_target, entropy_coeff, seed):
+def cpu_baseline(torch, w, rows_target, entropy_coeff, seed, mrl=None, dev=None, path="fused"):
     """Times the oracle (torch-CPU restatement of the reference op chain) fwd+bwd on a bounded
     sample of the same workload: one group of G responses with lengths scaled so that the packed
     batch has about `rows_target` rows at the full vocabulary."""
@@ -174,11 +174,29 @@ def cpu_baseline(torch, w, rows_target, entropy_coeff, seed):
     one()
     times = sorted(one() for _ in range(3))
     med = times[len(times) // 2]
-    return {
+    out = {
         "value": tokens / med, "unit": "tokens/s", "cores": threads, "kind": "port",
         "sample": "%d responses, %d packed rows x V=%d (fp32 up-cast), oracle fwd+bwd, median of 3 after 1 warm-up, "
                   "%.2f s per pass" % (group, total, vocab, med),
     }
+    if dev is not None:
+        # the same sample through the HIP path, checked against the oracle at the full vocabulary
+        z = z32.detach().requires_grad_()
+        want, _ = o_loss.grpo_compute_loss(z, b, meta, **kw)
+        (dz_o,) = torch.autograd.grad(want, z)
+        f = mrl.LossFuncFactory.get_instance("ray_grpo", "actor")
+        f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.001), "kl_penalty": "low_var_kl",
+                              "entropy_coeff": entropy_coeff})
+        to_dev = lambda d: {k: (v.to(dev) if isinstance(v, torch.Tensor) else v) for k, v in d.items()}
+        zd = logits.to(dev).requires_grad_()
+        got, _ = f.compute_loss(zd, to_dev(b), fused=(path == "fused"), **to_dev(kw))
+        (dz,) = torch.autograd.grad(got, zd)
+        out["sample_parity"] = {
+            "loss_rel_err": abs(got.item() - want.item()) / max(abs(want.item()), 1e-30),
+            "dlogits_max_abs_err": (dz.float().cpu() - dz_o).abs().max().item(),
+            "dlogits_max_abs": dz_o.abs().max().item(),
+        }
+    return out
 
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0
@@ -459,7 +477,7 @@ def main():
     dz = None
     del dz
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(torch, w, args.cpu_rows, args.entropy_coeff, args.seed)
+        result["cpu_baseline"] = cpu_baseline(torch, w, args.cpu_rows, args.entropy_coeff, args.seed, mrl, dev, args.path)
     print(json.dumps(result), flush=True)
 
 

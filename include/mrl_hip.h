@@ -4,7 +4,8 @@
  *
  * The reference has no native code and no FFI for this path: every function below replaces a
  * chain of torch ops in the reference's Python (cited per entry point, paths relative to the
- * reference tree).  Host code binds these symbols with ctypes.
+ * reference tree).  Host code binds these symbols with ctypes (mindspeed_rl_amd/_lib.py holds
+ * the argument types of every entry point).
  *
  * Conventions, all entry points:
  *   - plain C: raw DEVICE pointers, explicit int64 sizes, dtype enums, the HIP stream as void*
