@@ -321,7 +321,8 @@ def run_lmhead_train(args):
 # HBM bytes per launch of the dominant kernel from the committed rocprofv3 --pmc summary
 # (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for the copy probe); only
 # the default workload has been profiled that way, every other run reports null.
-PROFILED_TRAFFIC_BYTES = {("c1", "fused", "mrl_fused_logprob_loss"): 104.06e9}
+PROFILED_TRAFFIC_BYTES = {("c1", "fused", "mrl_fused_logprob_loss"): 104.06e9,
+                          ("c1", "split", "mrl_vocab_logprob_bwd"): 104.31e9}
 
 
 def _profiled_traffic(args, w, dominant):
@@ -401,7 +402,7 @@ def main():
         "mrl_vocab_logprob_bwd": live_rows * 2 * row_bytes + dead_rows * row_bytes,
         "mrl_fused_logprob_loss": live_rows * 2 * row_bytes + dead_rows * row_bytes,
     }
-    kernel_symbol = {"mrl_vocab_logprob_fwd": "vocab_fwd_kernel", "mrl_vocab_logprob_bwd": "vocab_bwd_kernel",
+    kernel_symbol = {"mrl_vocab_logprob_fwd": "vocab_fwd_kernel", "mrl_vocab_logprob_bwd": "bwd_rows_persistent_kernel",
                      "mrl_fused_logprob_loss": "fused_sweep_persistent_kernel"}
     kernels = {}
     for name, nbytes in kernel_bytes.items():
