@@ -178,6 +178,13 @@ int mrl_ragged_layout(const void* lengths, int lengths_dtype, int64_t batch, int
                       const void* rows, int elem_bytes, int64_t width, int left_pad, int32_t* eff_len,
                       int32_t* cu, int64_t* info, void* stream);
 
+/* mrl_first_match: the search inside remove_padding_and_split_to_list
+ * (mindspeed_rl/utils/pad_process.py:44-62): first[i] = index of the first entry of integer row i
+ * (elem_bytes 4 or 8) that equals `value`, plus `extra` (0 or 1), clamped to width; width if the
+ * row has no such entry.  int32 [batch]. */
+int mrl_first_match(const void* rows, int elem_bytes, int64_t batch, int64_t width, int64_t value, int extra,
+                    int32_t* first, void* stream);
+
 /* out[i, d, j] = flat[d * flat_stride + cu[i] + j] for j < cu[i+1] - cu[i], else pad_bits; out is
  * [batch, first_dim, width] (first_dim = 1 for ordinary columns, 3 for mrope position ids). */
 int mrl_ragged_to_padded(const void* flat, int elem_bytes, int64_t first_dim, int64_t flat_stride,
@@ -198,6 +205,12 @@ int mrl_padded_to_ragged(const void* padded, int elem_bytes, int64_t batch, int6
 int mrl_group_advantage(const void* rewards, int rewards_dtype, int64_t batch, int64_t group,
                         const void* mask, int mask_dtype, int64_t width, float* advantages,
                         float* returns, void* stream);
+
+/* mrl_group_standardize: get_last_reward (mindspeed_rl/trainer/utils/compute_utils.py:277-291):
+ * out[i] = (r_i - mean_g) / (unbiased_std_g + eps) over the group of `group` consecutive rewards
+ * that holds i; fp64 internally, fp32 result.  n must be a multiple of group. */
+int mrl_group_standardize(const void* rewards, int rewards_dtype, int64_t n, int64_t group, double eps,
+                          float* out, void* stream);
 
 /* DAPO dynamic-sampling predicate (mindspeed_rl/workers/dynamic_sampling.py:81-86): keep[r] = 1
  * for every row of a group iff numpy.std(group) > 0 or the group has one member, else 0.  The

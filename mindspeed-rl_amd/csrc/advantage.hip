@@ -54,6 +54,25 @@ __global__ __launch_bounds__(kBlock) void group_advantage_kernel(const void* __r
     }
 }
 
+// One thread per reward: (r - mean) / (unbiased std + eps) inside its group, fp64 internally.
+__global__ __launch_bounds__(kBlock) void group_standardize_kernel(const void* __restrict__ rewards, int rdtype,
+                                                                   int64_t n, int64_t group, double eps,
+                                                                   float* __restrict__ out) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const int64_t g0 = (i / group) * group;
+    double sum = 0.0;
+    for (int64_t q = 0; q < group; ++q) sum += reward_at(rewards, rdtype, g0 + q);
+    const double mean = sum / (double)group;
+    double ss = 0.0;
+    for (int64_t q = 0; q < group; ++q) {
+        const double d = reward_at(rewards, rdtype, g0 + q) - mean;
+        ss += d * d;
+    }
+    const double sd = sqrt(ss / (double)(group - 1));
+    out[i] = (float)((reward_at(rewards, rdtype, i) - mean) / (sd + eps));
+}
+
 // numpy's arithmetic, one correctly rounded operation at a time (no FMA contraction)
 template <typename F> struct Rn;
 template <> struct Rn<double> {
@@ -164,5 +183,21 @@ extern "C" int mrl_group_keep_mask(const void* metric, int metric_dtype, int64_t
         hipLaunchKernelGGL(group_keep_kernel<float>, dim3(blocks), dim3(kBlock), 0, s, (const float*)metric, n, group,
                            n_groups, keep);
     }
+    return mrl::check_launch(fn);
+}
+
+extern "C" int mrl_group_standardize(const void* rewards, int rewards_dtype, int64_t n, int64_t group, double eps,
+                                     float* out, void* stream) {
+    const char* fn = "mrl_group_standardize";
+    MRL_REQUIRE(rewards_dtype == MRL_F32 || rewards_dtype == MRL_F64, MRL_ERR_UNSUPPORTED,
+                "%s: rewards dtype %d (want F32 or F64)", fn, rewards_dtype);
+    MRL_REQUIRE(n >= 0 && group >= 1, MRL_ERR_INVALID_ARG, "%s: n=%lld group=%lld", fn, (long long)n, (long long)group);
+    MRL_REQUIRE(n % group == 0, MRL_ERR_INVALID_ARG, "%s: n=%lld is not a multiple of group=%lld", fn, (long long)n,
+                (long long)group);
+    if (n == 0) return MRL_OK;
+    MRL_REQUIRE(rewards && out, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+    const unsigned blocks = (unsigned)((n + kBlock - 1) / kBlock);
+    hipLaunchKernelGGL(group_standardize_kernel, dim3(blocks), dim3(kBlock), 0, mrl::as_stream(stream), rewards,
+                       rewards_dtype, n, group, eps, out);
     return mrl::check_launch(fn);
 }

@@ -341,6 +341,32 @@ int check_elems(const char* fn, int64_t n) {
     return MRL_OK;
 }
 
+// first[i] = smallest j with rows[i, j] == value, or width if there is none; `extra` is added to a
+// found index (clamped to width).  One wavefront per row.
+template <typename T>
+__global__ __launch_bounds__(256) void first_match_kernel(const T* __restrict__ rows, int64_t batch, int64_t width,
+                                                          T value, int extra, int32_t* __restrict__ first) {
+    const int64_t i = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (i >= batch) return;
+    const int lane = threadIdx.x & 63;
+    const T* row = rows + i * width;
+    int64_t best = width;
+    for (int64_t j0 = 0; j0 < width && best == width; j0 += 64) {       // `best` is uniform after the reduction
+        const int64_t j = j0 + lane;
+        int64_t mine = (j < width && row[j] == value) ? j : width;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            const int64_t o = __shfl_xor(mine, off, 64);
+            mine = o < mine ? o : mine;
+        }
+        best = mine;
+    }
+    if (lane == 0) {
+        int64_t n = best < width ? best + extra : width;
+        first[i] = (int32_t)(n < width ? n : width);
+    }
+}
+
 }  // namespace
 
 extern "C" int mrl_pack_index_build(const void* attention_mask, int mask_dtype, int64_t batch, int64_t width,
@@ -587,5 +613,25 @@ extern "C" int mrl_padded_to_ragged(const void* padded, int elem_bytes, int64_t 
     else if (elem_bytes == 4) MRL_P2R(uint32_t);
     else MRL_P2R(uint64_t);
 #undef MRL_P2R
+    return mrl::check_launch(fn);
+}
+
+extern "C" int mrl_first_match(const void* rows, int elem_bytes, int64_t batch, int64_t width, int64_t value, int extra,
+                               int32_t* first, void* stream) {
+    const char* fn = "mrl_first_match";
+    MRL_REQUIRE(batch >= 0 && width >= 0 && width <= 0x7fffffffLL, MRL_ERR_INVALID_ARG, "%s: batch=%lld width=%lld", fn,
+                (long long)batch, (long long)width);
+    MRL_REQUIRE(elem_bytes == 4 || elem_bytes == 8, MRL_ERR_UNSUPPORTED, "%s: elem_bytes=%d (want 4 or 8)", fn, elem_bytes);
+    MRL_REQUIRE(extra == 0 || extra == 1, MRL_ERR_INVALID_ARG, "%s: extra=%d", fn, extra);
+    if (batch == 0) return MRL_OK;
+    MRL_REQUIRE(first != nullptr && (rows != nullptr || width == 0), MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+    const dim3 grid((unsigned)((batch + 3) / 4)), block(256);
+    hipStream_t s = mrl::as_stream(stream);
+    if (elem_bytes == 8)
+        hipLaunchKernelGGL(first_match_kernel<int64_t>, grid, block, 0, s, (const int64_t*)rows, batch, width, value, extra,
+                           first);
+    else
+        hipLaunchKernelGGL(first_match_kernel<int32_t>, grid, block, 0, s, (const int32_t*)rows, batch, width,
+                           (int32_t)value, extra, first);
     return mrl::check_launch(fn);
 }

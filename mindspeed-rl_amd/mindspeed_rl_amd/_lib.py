@@ -58,6 +58,8 @@ SIGNATURES = {
     "mrl_scale_rows": [_vp, _int, _i64, _i64, _i64, _vp, _f32, _vp],
     "mrl_lmhead_workspace_bytes": [_i64, _i64],
     "mrl_lmhead_logprob_fwd": [_vp, _vp, _i64, _i64, _i64, _vp, _int, _f32, _vp, _vp, _vp, _vp, _i64, _vp],
+    "mrl_group_standardize": [_vp, _int, _i64, _i64, ctypes.c_double, _vp, _vp],
+    "mrl_first_match": [_vp, _int, _i64, _i64, _i64, _int, _vp, _vp],
     "mrl_kl_token_rewards": [_vp, _vp, _vp, _int, _vp, _i64, _i64, _int, _f32, _vp, _vp, _vp],
     "mrl_gae_scan": [_vp, _vp, _i64, _i64, _f32, _f32, _vp, _vp, _vp],
     "mrl_masked_whiten": [_vp, _vp, _int, _i64, _int, _vp, _vp, _vp],

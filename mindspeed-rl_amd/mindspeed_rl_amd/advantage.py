@@ -51,6 +51,24 @@ def compute_group_norm_advantage_return(token_level_rewards, eos_mask, response_
     return adv, ret
 
 
+def get_last_reward(rm_scores, n_sample_batch: int):
+    """Reference: ``trainer/utils/compute_utils.py:277-291``: every reward standardised inside its
+    group of ``n_sample_batch`` consecutive samples, ``(r - mean) / (std + 1e-8)`` with the unbiased
+    standard deviation; same shape as ``rm_scores``, fp32."""
+    dev = _lib.require_device(rm_scores)
+    rewards = rm_scores.detach()
+    if rewards.dtype not in (torch.float32, torch.float64):
+        rewards = rewards.to(torch.float32)
+    flat = rewards.reshape(-1).contiguous()
+    n = flat.numel()
+    if n % n_sample_batch != 0:
+        raise RuntimeError("shape '[-1, %d]' is invalid for input of size %d" % (n_sample_batch, n))
+    out = torch.empty(n, dtype=torch.float32, device=dev)
+    _lib.call("mrl_group_standardize", _lib.ptr(flat), _lib.dtype_code(flat), n, int(n_sample_batch), 1e-8, _lib.ptr(out),
+              _lib.stream(dev))
+    return out.view(rm_scores.shape)
+
+
 def dynamic_sampling_keep_mask(metric_values, n_samples_per_prompt):
     """uint8 ``[N]`` device mask: 1 for the rows of every group the DAPO filter keeps
     (``numpy.std(group) > 0`` or a single-member group), following numpy's arithmetic in the

@@ -16,3 +16,8 @@ def masked_sum(values, mask, axis=None):
 
 def masked_mean(values, mask, axis=None, epsilon=1e-8):
     return masked_sum(values, mask, axis) / (mask.sum(axis=axis) + epsilon)
+
+
+def clip_by_value(x, tensor_min, tensor_max):
+    """Reference: ``torch_functional.py:22-35``: ``max(min(x, tensor_max), tensor_min)``."""
+    return torch.max(torch.min(x, tensor_max), tensor_min)

@@ -573,3 +573,21 @@ class ReferenceLossFunc(BaseLossFunc):
         if forward_only:
             return log_probs
         return None
+
+
+@LossFuncFactory.register_loss("ray_grpo", "reward")
+@LossFuncFactory.register_loss("ray_ppo", "reward")
+class RewardLossFunc(BaseLossFunc):
+    """Reference: ``reward_loss_func.py:11-31``: the reward model's scores, unpacked to
+    ``[B, seq_len, ...]`` when the batch was packed."""
+
+    def __init__(self):
+        super(RewardLossFunc, self).__init__()
+
+    def compute_loss(self, output: torch.Tensor, batch: Dict[str, torch.Tensor], forward_only=False,
+                     non_loss_data=True, **kwargs) -> Tuple[torch.Tensor, Dict]:
+        if kwargs.get("use_remove_padding", False):
+            output = postprocess_packed_seqs(output=output, seqlens_in_batch=kwargs.get("seqlens_in_batch", None),
+                                             cu_seqlens_padded=kwargs.get("cu_seqlens_padded", None),
+                                             seq_len=kwargs.get("seq_len", None))
+        return output

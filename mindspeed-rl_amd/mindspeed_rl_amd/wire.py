@@ -164,3 +164,91 @@ def truncate_rows(tensor, index_tensor, left_pad=False):
             rows.append(host[lo:lo + n])
         lo += n
     return rows
+
+
+def _ragged_to_padded(flat, sizes, width, pad, dev):
+    """flat 1-D device tensor holding the samples back to back -> [n, width]."""
+    n = len(sizes)
+    cu = torch.zeros(n + 1, dtype=torch.int32)
+    cu[1:] = torch.cumsum(torch.tensor(sizes, dtype=torch.int64), 0).to(torch.int32)
+    cu = cu.to(dev)
+    out = torch.empty((n, width), dtype=flat.dtype, device=dev)
+    if flat.element_size() not in (2, 4, 8):
+        raise TypeError("unsupported element size %d" % flat.element_size())
+    _lib.call("mrl_ragged_to_padded", _lib.ptr(flat), flat.element_size(), 1, max(flat.shape[0], 1), _lib.ptr(cu), n,
+              width, _pad_bits(flat.dtype, pad), _lib.ptr(out), _lib.stream(dev))
+    return out
+
+
+def pad_multiple(data_list, pad_id, multiple=1):
+    """Reference: ``utils/pad_process.py:65-71``.  A list of 1-D device tensors -> ``[n, L]`` padded
+    with ``pad_id``, ``L`` the longest sample rounded up to ``multiple``.  The lengths come from
+    the shapes (no device read); one concatenation and one gather launch."""
+    dev = _lib.require_device(data_list[0])
+    sizes = [int(t.shape[0]) for t in data_list]
+    width = (max(sizes) + multiple - 1) // multiple * multiple
+    return _ragged_to_padded(torch.cat(list(data_list)).contiguous(), sizes, width, pad_id, dev)
+
+
+def padding_dict_to_tensor_dict(experience_data):
+    """Reference: ``utils/pad_process.py:13-25``, returning a plain dict (the reference wraps it in a
+    TensorDict): each column, a list of 1-D device tensors, becomes a zero-padded ``[n, max_len]``
+    tensor; ``original_length`` (int64, on the device) lists the sample lengths column after column."""
+    batch, lengths, dev = {}, [], None
+    for column, value in experience_data.items():
+        dev = _lib.require_device(value[0])
+        sizes = [int(t.shape[0]) for t in value]
+        batch[column] = _ragged_to_padded(torch.cat(list(value)).contiguous(), sizes, max(sizes), 0, dev)
+        lengths.extend(sizes)
+    batch["original_length"] = torch.tensor(lengths, dtype=torch.int64).to(dev)
+    return batch
+
+
+def remove_padding_tensor_dict_to_dict(data_dict):
+    """Reference: ``utils/pad_process.py:28-40``: the inverse of :func:`padding_dict_to_tensor_dict`,
+    lists of CPU rows (see :func:`truncate_rows`)."""
+    out = {}
+    if data_dict is None:
+        return out
+    if "original_length" not in data_dict.keys():
+        return data_dict
+    data_lengths = data_dict["original_length"]
+    for idx, (key, value) in enumerate(data_dict.items()):
+        if key == "original_length":
+            continue
+        out[key] = truncate_rows(value, data_lengths[idx * len(value):(idx + 1) * len(value)])
+    return out
+
+
+def remove_padding_and_split_to_list(responses, eos_token_id, pad_token_id, to_list=False):
+    """Reference: ``utils/pad_process.py:44-62``: every row of the integer ``[B, L]`` tensor cut at
+    its first ``pad_token_id`` (the pad token itself is kept when it is also the end-of-sequence
+    token).  Returns device tensors, or python lists without the last token when ``to_list``.  One
+    search launch, one packing launch and one host read of the ``B`` lengths replace the
+    reference's ``nonzero`` per row."""
+    dev = _lib.require_device(responses)
+    src = responses.contiguous()
+    if src.dim() != 2 or src.is_floating_point() or src.element_size() not in (4, 8):
+        raise TypeError("responses must be a [B, L] tensor of 4- or 8-byte integers")
+    batch, width = src.shape
+    first = torch.empty(batch, dtype=torch.int32, device=dev)
+    stream = _lib.stream(dev)
+    _lib.call("mrl_first_match", _lib.ptr(src), src.element_size(), batch, width, int(pad_token_id),
+              1 if pad_token_id == eos_token_id else 0, _lib.ptr(first), stream)
+    cu = torch.empty(batch + 1, dtype=torch.int32, device=dev)
+    info = torch.empty(2, dtype=torch.int64, device=dev)
+    _lib.call("mrl_ragged_layout", _lib.ptr(first), _lib.I32, batch, 1, None, src.element_size(), width, 0, None,
+              _lib.ptr(cu), _lib.ptr(info), stream)
+    lens = first.cpu().tolist()
+    total = sum(lens)
+    flat = torch.empty(total, dtype=src.dtype, device=dev)
+    _lib.call("mrl_padded_to_ragged", _lib.ptr(src), src.element_size(), batch, width, _lib.ptr(cu), 0, total,
+              _lib.ptr(flat), stream)
+    if to_list:
+        host = flat.cpu().tolist()
+        out, lo = [], 0
+        for n in lens:
+            out.append(host[lo:lo + n][:-1])
+            lo += n
+        return out
+    return list(torch.split(flat, lens))

@@ -101,3 +101,10 @@ def compute_gae_advantage_return(token_level_rewards, values, eos_mask, gamma, l
         returns = advantages + values
         advantages = loss.masked_whiten(advantages, eos_mask)
     return advantages, returns
+
+
+def get_last_reward(rm_scores, n_sample_batch):
+    """``compute_utils.py:277-291``."""
+    reward = rm_scores.reshape(-1, n_sample_batch)
+    last_reward = (reward - reward.mean(dim=1, keepdim=True)) / (reward.std(dim=1, keepdim=True) + 1e-8)
+    return last_reward.reshape(rm_scores.shape)

@@ -181,3 +181,55 @@ def truncate_rows(tensor, index_tensor, left_pad=False):
             row = tensor[i, -n:].cpu() if left_pad else tensor[i, :n].cpu()
         rows.append(row)
     return rows
+
+
+def pad_multiple(data_list, pad_id, multiple=1):
+    """``utils/pad_process.py:65-71``: right-pad to the longest sample, rounded up to ``multiple``."""
+    padded = torch.nn.utils.rnn.pad_sequence(data_list, batch_first=True, padding_value=pad_id)
+    max_len = padded.size(1)
+    target_len = ((max_len + multiple - 1) // multiple) * multiple
+    return torch.nn.functional.pad(padded, (0, target_len - max_len), value=pad_id)
+
+
+def remove_padding_and_split_to_list(responses, eos_token_id, pad_token_id, to_list=False):
+    """``utils/pad_process.py:44-62``: cut every row at its first pad token (keeping it when the pad
+    token is also the end-of-sequence token)."""
+    output = []
+    for i in range(responses.shape[0]):
+        response = responses[i]
+        nonzeros = torch.nonzero(response == pad_token_id, as_tuple=False)
+        first_pad_index = nonzeros[0][0] if len(nonzeros) != 0 else len(response)
+        response = response[:first_pad_index + 1] if pad_token_id == eos_token_id else response[:first_pad_index]
+        if to_list:
+            response = response[:-1].cpu().numpy().tolist()
+        output.append(response)
+    return output
+
+
+def padding_dict_to_tensor_dict(experience_data):
+    """``utils/pad_process.py:13-25`` with a plain dict in place of the TensorDict: every column
+    (a list of 1-D samples) becomes a zero-padded ``[n, max_len]`` tensor; ``original_length`` holds
+    the sample lengths column after column."""
+    batch, lengths = {}, []
+    for column, value in experience_data.items():
+        max_length = max(len(exp) for exp in value)
+        batch[column] = torch.stack([torch.nn.functional.pad(exp, (0, max_length - len(exp)), mode="constant", value=0)
+                                     for exp in value], dim=0)
+        lengths.extend([torch.tensor(len(exp)) for exp in value])
+    batch["original_length"] = torch.stack(lengths)
+    return batch
+
+
+def remove_padding_tensor_dict_to_dict(data_dict):
+    """``utils/pad_process.py:28-40``."""
+    out = {}
+    if data_dict is None:
+        return out
+    if "original_length" not in data_dict.keys():
+        return data_dict
+    data_lengths = data_dict["original_length"]
+    for idx, (key, value) in enumerate(data_dict.items()):
+        if key == "original_length":
+            continue
+        out[key] = truncate_rows(value, data_lengths[idx * len(value):(idx + 1) * len(value)])
+    return out

@@ -389,6 +389,66 @@ def test_wire_format_bit_exact(dev):
         mrl.pack_experience_columns("actor_train", {"responses": samples["responses"]}, batch - 1)
 
 
+def test_pad_process_parity(dev, reference_vectors):
+    """The rest of pad_process.py and the small helpers around the path, against the oracle."""
+    v = reference_vectors["remove_padding_and_split_to_list"]
+    out = mrl.remove_padding_and_split_to_list(torch.tensor(v["responses"]).to(dev), v["eos_token_id"], v["pad_token_id"])
+    assert [o.tolist() for o in out] == v["expected"] and out[0].device.type == "cuda"
+    m = reference_vectors["pad_multiple"]
+    got = mrl.pad_multiple([torch.tensor(x).to(dev) for x in m["data_list"]], m["pad_id"], m["multiple"])
+    assert got.tolist() == m["expected"]
+    gen = torch.Generator().manual_seed(71)
+    batch, width = 41, 130
+    resp = torch.randint(1, 50, (batch, width), generator=gen)
+    lens = torch.randint(0, width + 1, (batch,), generator=gen)
+    lens[0], lens[1] = 0, width
+    for i in range(batch):
+        resp[i, int(lens[i]):] = 7
+    resp[5, 3] = 7                                      # a pad token inside the response: the row is cut there
+    for eos, pad in ((99, 7), (7, 7)):
+        for cast in (torch.int64, torch.int32):
+            for to_list in (False, True):
+                want = o_pack.remove_padding_and_split_to_list(resp.to(cast), eos, pad, to_list)
+                got = mrl.remove_padding_and_split_to_list(resp.to(cast).to(dev), eos, pad, to_list)
+                assert len(got) == batch
+                for a, b in zip(got, want):
+                    if to_list:
+                        assert a == b
+                    else:
+                        assert a.dtype == b.dtype and torch.equal(a.cpu(), b)
+    cols = {"ids": [torch.randint(0, 9, (int(n),), generator=gen) for n in torch.randint(1, 20, (9,), generator=gen)],
+            "lp": [torch.randn(int(n), generator=gen) for n in torch.randint(1, 33, (9,), generator=gen)]}
+    want = o_pack.padding_dict_to_tensor_dict(cols)
+    got = mrl.padding_dict_to_tensor_dict({k: [t.to(dev) for t in v_] for k, v_ in cols.items()})
+    assert list(got) == list(want)
+    for k in want:
+        assert got[k].dtype == want[k].dtype and torch.equal(got[k].cpu(), want[k]), k
+    back = mrl.remove_padding_tensor_dict_to_dict(got)
+    for k in cols:
+        assert all(torch.equal(a, b) for a, b in zip(back[k], cols[k]))
+    assert mrl.remove_padding_tensor_dict_to_dict(None) == {}
+    for k in (1, 2, 8):
+        want = o_pack.pad_multiple(cols["lp"], 0.5, k)
+        assert torch.equal(mrl.pad_multiple([t.to(dev) for t in cols["lp"]], 0.5, k).cpu(), want)
+    # get_last_reward, clip_by_value, the reward model's loss object
+    scores = torch.randn(24, 1, generator=gen)
+    assert (mrl.get_last_reward(scores.to(dev), 8).cpu() - o_adv.get_last_reward(scores, 8)).abs().max().item() < 1e-5
+    x = torch.randn(5, 6, generator=gen)
+    assert torch.equal(mrl.clip_by_value(x.to(dev), torch.tensor(-0.5, device=dev), torch.tensor(0.25, device=dev)).cpu(),
+                       torch.clamp(x, -0.5, 0.25))
+    rw = mrl.LossFuncFactory.get_instance("ray_grpo", "reward")
+    assert isinstance(rw, mrl.RewardLossFunc) and isinstance(mrl.LossFuncFactory.get_instance("ray_ppo", "reward"),
+                                                                mrl.RewardLossFunc)
+    seqlens = torch.tensor([3, 5], dtype=torch.int32)
+    cu = torch.tensor([0, 4, 12], dtype=torch.int32)
+    packed = torch.randn(1, 12, 1, generator=gen)
+    got = rw.compute_loss(packed.to(dev), {}, forward_only=True, use_remove_padding=True, seqlens_in_batch=seqlens.to(dev),
+                          cu_seqlens_padded=cu.to(dev), seq_len=6)
+    assert torch.equal(got.cpu(), o_pack.postprocess_packed_seqs(packed, seqlens, cu, 6))
+    plain = packed.to(dev)
+    assert rw.compute_loss(plain, {}) is plain
+
+
 # --------------------------------------------------------------------------------- PPO value side
 def test_value_side_reference_vectors_on_device(dev, reference_vectors):
     w = reference_vectors["masked_whiten"]

@@ -532,3 +532,30 @@ def test_value_side_closed_forms():
         "responses": torch.zeros(2, 3), "prompt_length": torch.tensor([[2], [1]]),
         "response_length": torch.tensor([[3], [2]])}, forward_only=True)
     assert out.squeeze(-1).tolist() == [[1.0, 2.0, 3.0], [6.0, 7.0, 0.0]]
+
+
+def test_pad_process_reference_vectors(reference_vectors):
+    """remove_padding_and_split_to_list and pad_multiple (tests/ut/utils/test_pad_process.py:18-46), the
+    TensorDict round trip by construction, get_last_reward against its closed form."""
+    v = reference_vectors["remove_padding_and_split_to_list"]
+    out = packing.remove_padding_and_split_to_list(torch.tensor(v["responses"]), v["eos_token_id"], v["pad_token_id"])
+    assert [o.tolist() for o in out] == v["expected"]
+    # pad token == eos token: the first pad token is kept; to_list drops the last token
+    out = packing.remove_padding_and_split_to_list(torch.tensor(v["responses"]), 0, 0)
+    assert [o.tolist() for o in out] == [[1, 2, 3, 4, 0], [4, 5, 6, 1, 1, 0]]
+    assert packing.remove_padding_and_split_to_list(torch.tensor(v["responses"]), 0, 0, to_list=True) == \
+        [[1, 2, 3, 4], [4, 5, 6, 1, 1]]
+    m = reference_vectors["pad_multiple"]
+    got = packing.pad_multiple([torch.tensor(x) for x in m["data_list"]], m["pad_id"], m["multiple"])
+    assert got.tolist() == m["expected"]
+    cols = {"a": [torch.tensor([1, 2, 3]), torch.tensor([4])], "b": [torch.tensor([5.0]), torch.tensor([6.0, 7.0])]}
+    packed = packing.padding_dict_to_tensor_dict(cols)
+    assert packed["a"].tolist() == [[1, 2, 3], [4, 0, 0]] and packed["b"].tolist() == [[5.0, 0.0], [6.0, 7.0]]
+    assert packed["original_length"].tolist() == [3, 1, 1, 2]
+    back = packing.remove_padding_tensor_dict_to_dict(packed)
+    for k in cols:
+        assert [r.tolist() for r in back[k]] == [c.tolist() for c in cols[k]]
+    assert packing.remove_padding_tensor_dict_to_dict(None) == {}
+    r = torch.tensor([[1.0], [3.0], [2.0], [2.0]])
+    got = advantage.get_last_reward(r, 2)
+    assert torch.allclose(got, torch.tensor([[-0.70710677], [0.70710677], [0.0], [0.0]]), atol=1e-6)
