@@ -145,7 +145,9 @@ class _FusedLmHeadLoss(torch.autograd.Function):
             if cfg["fp32_dw_gemm"]:
                 d_weight32.addmm_(z.t().float(), h2d[c0:c1].float())
             else:
-                _accumulate_fp32(d_weight32, z.t(), h2d[c0:c1])
+                # the hidden chunk goes in as the transpose of an [H, rows] copy: the library picks a faster
+                # kernel for that operand layout (7.5 against 8.7 ms per chunk), the copy is 59 MB
+                _accumulate_fp32(d_weight32, z.t(), h2d[c0:c1].t().contiguous().t())
         _lib.call("mrl_fused_loss_reduce", _lib.ptr(row_terms), _lib.ptr(row_start), _lib.ptr(row_count), n_seq, width,
                   _lib.ptr(old), _lib.ptr(ref), _lib.ptr(adv), _lib.ptr(mask_t), mdt, _lib.ptr(resp), rdt,
                   cfg["clip_lo"], cfg["clip_hi"], cfg["kl_penalty"], cfg["kl_coef"], cfg["entropy_coeff"],
