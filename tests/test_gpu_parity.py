@@ -1075,6 +1075,35 @@ def test_fused_sweep_persistent_with_skipped_rows(dev):
             ((dz.float().cpu() != 0) <= (dz_o != 0)).all().item()      # nothing outside the response rows
 
 
+def test_fused_sweep_persistent_full_vocab(dev):
+    """The persistent fused sweep at the Qwen2.5 vocabulary (19 vectors per thread, the last one partly
+    past the end of the row) on more than 2 x CU-count rows, against the oracle end to end."""
+    gen = torch.Generator().manual_seed(33)
+    logits, b, kw, _, _ = _make_batch(gen, 2, 4, 120, 150, 152064, torch.bfloat16, 3.0, 1, prompt_hi=2)
+    assert logits.shape[1] > 2 * 256 + 300
+    meta = dict(clip_ratio=0.2, kl_coef=0.001, kl_penalty="low_var_kl", entropy_coeff=0.001)
+    zo = logits.float().requires_grad_()
+    want, want_stats = o_loss.grpo_compute_loss(zo, b, meta, **kw)
+    (dz_o,) = torch.autograd.grad(want, zo)
+    f = mrl.LossFuncFactory.get_instance("ray_grpo", "actor")
+    f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.001), "kl_penalty": "low_var_kl",
+                          "entropy_coeff": 0.001})
+    zd = logits.to(dev).requires_grad_()
+    got, got_stats = f.compute_loss(zd, _to_dev(b, dev), fused=True, grad_inplace=False, **_to_dev(kw, dev))
+    (dz,) = torch.autograd.grad(got, zd)
+    assert abs(got.item() - want.item()) <= TOL_LOSS_REL * abs(want.item()) + 1e-7
+    for k in want_stats:
+        assert abs(got_stats[k] - want_stats[k]) <= TOL_LOSS_REL * abs(want_stats[k]) + 1e-6, k
+    err = (dz.float().cpu() - dz_o).abs().max().item()
+    assert err < TOL_DLOGITS and err <= 2 ** -8 * dz_o.abs().max().item() + 1e-9
+    # the split kernels on the same batch (persistent backward) agree with the fused sweep
+    zs = logits.to(dev).requires_grad_()
+    loss_s, _ = f.compute_loss(zs, _to_dev(b, dev), fused=False, **_to_dev(kw, dev))
+    (dz_s,) = torch.autograd.grad(loss_s, zs)
+    assert loss_s.item() == pytest.approx(got.item(), rel=5e-5)
+    assert (dz_s.float() - dz.float()).abs().max().item() <= 2 ** -7 * dz.float().abs().max().item()
+
+
 @pytest.mark.parametrize("tokens,vocab,hdim", [(300, 1000, 128), (129, 256, 64), (64, 4096 + 24, 256),
                                                (517, 2 * 2048 + 256, 3584)])
 def test_lmhead_logprob_forward(dev, tokens, vocab, hdim):
