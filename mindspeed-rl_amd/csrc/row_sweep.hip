@@ -452,41 +452,62 @@ __global__ __launch_bounds__(kBlock) void bwd_rows_kernel(
 // runs while the following row is on its way.
 template <int DT, int NV, bool kEntropy>
 __global__ __launch_bounds__(kBlock) void bwd_rows_persistent_kernel(
-    const typename Elem<DT>::T* logits, int64_t row_stride, int vocab, int64_t n_rows,
+    const typename Elem<DT>::T* logits, int64_t row_stride, int vocab, int64_t n_rows, int seg_elems, int n_seg,
     const void* __restrict__ labels, int labels_dtype, float inv_t, const float* __restrict__ lse_in,
     const float* __restrict__ ent_in, const float* __restrict__ g_logp, const float* __restrict__ g_entropy,
     typename Elem<DT>::T* dlogits, int64_t d_stride) {
     using E = Elem<DT>;
     using T = typename E::T;
-    const uint32_t row_bytes = (uint32_t)vocab * (uint32_t)sizeof(T);
+    // The unit of work is a SEGMENT of a row: the backward needs no whole-row state (the log-sum-exp
+    // is an input), so a row that does not fit the registers of a workgroup (fp32 at V = 152064) is
+    // handled as n_seg independent pieces of seg_elems entries.  Units are numbered row-major.
+    const int64_t n_units = n_rows * n_seg;
     const int64_t step = gridDim.x;
+    const int64_t step_r = step / n_seg;
+    const int step_s = (int)(step % n_seg);
     auto grad_lp = [&](int64_t r) { return g_logp ? g_logp[r] : 0.f; };
     auto grad_h = [&](int64_t r) { return (kEntropy && g_entropy) ? g_entropy[r] : 0.f; };
+    auto seg_bytes = [&](int s) {
+        const int left = vocab - s * seg_elems;
+        return (uint32_t)(left < seg_elems ? left : seg_elems) * (uint32_t)sizeof(T);
+    };
 
     u32x4 v[NV];
-    int64_t r = blockIdx.x;
+    int64_t u = blockIdx.x;
+    int64_t r = u / n_seg;
+    int s = (int)(u - r * n_seg);
     int64_t y = 0;
     uint32_t zy_bits = 0;
-    if (r < n_rows) {
+    if (u < n_units) {
         const bool live = grad_lp(r) != 0.f || grad_h(r) != 0.f;
         const T* row = logits + r * row_stride;
         y = load_label(labels, labels_dtype, r);
         zy_bits = E::load_bits(row + ((y >= 0 && y < (int64_t)vocab) ? y : 0));
         vector_fence();
-        load_row<NV>(v, row_ref(row, live ? row_bytes : 0u));
+        load_row<NV>(v, row_ref(row + (int64_t)s * seg_elems, live ? seg_bytes(s) : 0u));
     }
-    for (; r < n_rows; r += step) {
-        const RowRef dst = row_ref(dlogits + r * d_stride, row_bytes);
+    for (; u < n_units; u += step) {
+        const uint32_t bytes = seg_bytes(s);
+        const RowRef dst = row_ref(dlogits + r * d_stride + (int64_t)s * seg_elems, bytes);
         const float g_lp = grad_lp(r), g_h = grad_h(r);
-        const bool y_ok = (y >= 0) && (y < (int64_t)vocab);
-        const int64_t r2 = r + step;
-        const bool has_next = r2 < n_rows;
+        // the label in coordinates of this segment (outside it: no one-hot term here)
+        const int64_t y_local = y - (int64_t)s * seg_elems;
+        const bool y_here = (y >= 0) && (y < (int64_t)vocab) && y_local >= 0 && y_local < (int64_t)seg_elems;
+        // the next unit of this workgroup
+        int64_t r2 = r + step_r;
+        int s2 = s + step_s;
+        if (s2 >= n_seg) {
+            s2 -= n_seg;
+            ++r2;
+        }
+        const bool has_next = u + step < n_units;
         const int64_t rn = has_next ? r2 : r;
+        const int sn = has_next ? s2 : s;
         const bool next_live = has_next && (grad_lp(rn) != 0.f || grad_h(rn) != 0.f);
         const T* nrow = logits + rn * row_stride;
         const int64_t y_next = load_label(labels, labels_dtype, rn);
         const T* zy_next_ptr = nrow + ((y_next >= 0 && y_next < (int64_t)vocab) ? y_next : 0);
-        const RowRef nxt = row_ref(nrow, next_live ? row_bytes : 0u);
+        const RowRef nxt = row_ref(nrow + (int64_t)sn * seg_elems, next_live ? seg_bytes(sn) : 0u);
         uint32_t zy_next = 0;
         bool wrote = false;
         if (g_lp != 0.f || g_h != 0.f) {
@@ -502,7 +523,7 @@ __global__ __launch_bounds__(kBlock) void bwd_rows_persistent_kernel(
                 mrl::buf_store_nt(grad_vec<DT, kEntropy>(v[q], g), vec_rsrc(dst, q), lane_offset());
                 vector_fence();
             }
-            store_label_grad<DT, kEntropy>(dst, g, y_ok, y, E::from_bits(zy_bits));
+            store_label_grad<DT, kEntropy>(dst, g, y_here, y_local, E::from_bits(zy_bits));
             // the refill is written out on both paths: after a join the compiler would wait for
             // every store of the row before the first load of the next
             zy_next = E::load_bits(zy_next_ptr);
@@ -518,6 +539,8 @@ __global__ __launch_bounds__(kBlock) void bwd_rows_persistent_kernel(
         }
         zy_bits = zy_next;
         y = y_next;
+        r = r2;
+        s = s2;
     }
 }
 
@@ -628,13 +651,16 @@ template <int DT, int NV>
 int launch_bwd_rows_nv(const mrl::BwdArgs& a) {
     using T = typename Elem<DT>::T;
     const dim3 block(kBlock);
-    const int cus = persistent_enabled() ? cu_count() : 0;
-    if (cus > 0 && a.n_rows > 2 * (int64_t)cus) {
-        const dim3 pgrid((unsigned)cus);
+    const int seg_elems = a.seg_vec * Elem<DT>::kVec;
+    const int cus = persistent_enabled() || a.n_seg > 1 ? cu_count() : 0;
+    if (a.n_seg > 1 || (cus > 0 && a.n_rows > 2 * (int64_t)cus)) {
+        const int64_t units = a.n_rows * a.n_seg;
+        const int64_t want = cus > 0 ? cus : 256;
+        const dim3 pgrid((unsigned)(units < want ? units : want));
 #define MRL_BWDP_LAUNCH(ENT)                                                                                      \
     hipLaunchKernelGGL((bwd_rows_persistent_kernel<DT, NV, ENT>), pgrid, block, 0, a.stream, (const T*)a.logits,  \
-                       a.row_stride, (int)a.vocab, a.n_rows, a.labels, a.labels_dtype, a.inv_t, a.lse, a.entropy, \
-                       a.g_logp, a.g_entropy, (T*)a.dlogits, a.d_stride)
+                       a.row_stride, (int)a.vocab, a.n_rows, seg_elems, a.n_seg, a.labels, a.labels_dtype, a.inv_t,   \
+                       a.lse, a.entropy, a.g_logp, a.g_entropy, (T*)a.dlogits, a.d_stride)
         if (a.g_entropy != nullptr) MRL_BWDP_LAUNCH(true);
         else MRL_BWDP_LAUNCH(false);
 #undef MRL_BWDP_LAUNCH
@@ -657,13 +683,28 @@ int bwd_rows_by_nv(int nv, const mrl::BwdArgs& a) { MRL_NV_SWITCH(launch_bwd_row
 
 namespace mrl {
 
-int launch_bwd_rows(const BwdArgs& a) {
-    const int nv = pick_nv(a.vocab / (16 / float_dtype_bytes(a.dtype)));
+int launch_bwd_rows(const BwdArgs& a0) {
+    BwdArgs a = a0;
+    const int64_t n_vec = a.vocab / (16 / float_dtype_bytes(a.dtype));
+    a.n_seg = (int)((n_vec + (int64_t)kMaxVecPerThread * kBlock - 1) / ((int64_t)kMaxVecPerThread * kBlock));
+    a.seg_vec = (int)((n_vec + a.n_seg - 1) / a.n_seg);
+    const int nv = pick_nv(a.seg_vec);
     switch (a.dtype) {
         case MRL_F32: return bwd_rows_by_nv<MRL_F32>(nv, a);
         case MRL_BF16: return bwd_rows_by_nv<MRL_BF16>(nv, a);
         default: return bwd_rows_by_nv<MRL_F16>(nv, a);
     }
+}
+
+bool bwd_rows_supported(int dtype, int64_t vocab, const void* in, int64_t in_stride, const void* out,
+                        int64_t out_stride, int64_t n_rows) {
+    const int eb = float_dtype_bytes(dtype);
+    if (eb == 0) return false;
+    const int64_t per_vec = 16 / eb;
+    if (vocab % per_vec != 0 || vocab * eb < 16 * 1024 || vocab > (1LL << 30)) return false;
+    if (!aligned(in, 16) || !aligned(out, 16)) return false;
+    if (n_rows > 1 && ((in_stride * eb) % 16 != 0 || (out_stride * eb) % 16 != 0)) return false;
+    return true;
 }
 
 bool row_sweep_supported(int dtype, int64_t vocab, const void* in, int64_t in_stride, const void* out,

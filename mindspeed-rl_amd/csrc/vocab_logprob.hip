@@ -428,11 +428,12 @@ extern "C" int mrl_vocab_logprob_bwd(const void* logits, int logits_dtype, int64
     }
     hipStream_t s = mrl::as_stream(stream);
     const int v = (int)vocab;
-    // rows that fill a 1024-thread workgroup and fit its register file take the row-in-registers kernel
-    if (dlogits_dtype == logits_dtype && sweep_rows_enabled() && vocab * ib >= 16 * 1024 &&
-        mrl::row_sweep_supported(logits_dtype, vocab, logits, row_stride, dlogits, dlogits_row_stride, n_rows)) {
+    // rows that fill a 1024-thread workgroup take the row-in-registers kernel (in segments if a row is
+    // larger than the register file of a workgroup)
+    if (dlogits_dtype == logits_dtype && sweep_rows_enabled() &&
+        mrl::bwd_rows_supported(logits_dtype, vocab, logits, row_stride, dlogits, dlogits_row_stride, n_rows)) {
         const mrl::BwdArgs a = {logits, logits_dtype, n_rows, vocab, row_stride, labels, labels_dtype, inv_temperature,
-                                lse, entropy, g_logp, g_entropy, dlogits, dlogits_row_stride, s};
+                                lse, entropy, g_logp, g_entropy, dlogits, dlogits_row_stride, s, 1, 0};
         return mrl::launch_bwd_rows(a);
     }
 #define MRL_BWD(DI, DO)                                                                                      \

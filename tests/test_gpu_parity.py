@@ -1041,6 +1041,35 @@ def test_persistent_row_sweeps(dev, dtype, vocab):
     assert (zin.float().cpu() - dz_lp_o).abs().max().item() < tol
 
 
+@pytest.mark.parametrize("rows", [5, 600])
+def test_backward_rows_in_segments(dev, rows):
+    """fp32 rows of 152064 entries (608 KiB) exceed the registers of a workgroup: the backward handles
+    them as two independent segments; labels in either segment, at the seam and outside the vocabulary."""
+    torch.manual_seed(rows)
+    vocab = 152064
+    z = (torch.randn(rows, vocab, device=dev) * 3)
+    y = torch.randint(0, vocab, (rows,), device=dev)
+    seam = (vocab // 4 + 2 * 1024 * 19 - 1) // (2 * 1024 * 19)    # vectors per segment are ceil(n_vec / 2)
+    half = ((vocab // 4 + 1) // 2) * 4
+    y[0], y[1], y[2], y[3], y[4] = half - 1, half, 0, vocab - 1, -100
+    assert seam == 1
+    g_lp = torch.randn(rows, device=dev) * 0.1
+    g_h = torch.randn(rows, device=dev) * 0.01
+    g_lp[2], g_h[2] = 0.0, 0.0
+    zr = z.clone().requires_grad_()
+    lp, h, lse = mrl.vocab_logprob_entropy(zr, y)
+    (dz,) = torch.autograd.grad([lp, h], zr, [g_lp, g_h])
+    ref = torch.log_softmax(z, -1)
+    p = ref.exp()
+    y_ok = (y >= 0) & (y < vocab)
+    onehot = torch.zeros_like(z)
+    onehot[y_ok, y[y_ok]] = 1.0
+    closed = g_lp[:, None] * (onehot - p) - g_h[:, None] * p * (z - (p * z).sum(-1, keepdim=True))
+    assert (dz - closed).abs().max().item() < 1e-5
+    assert not dz[2].any().item()
+    assert torch.equal(zr.detach(), z)
+
+
 def test_fused_sweep_persistent_with_skipped_rows(dev):
     """The fused sweep on more than 2 x CU-count rows: prompt rows, alignment padding and sequences
     without a response are rows it must not read but must zero."""
