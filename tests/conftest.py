@@ -19,3 +19,9 @@ def pytest_configure(config):
 def reference_vectors():
     with open(os.path.join(ROOT, "tests", "golden", "reference_vectors.json")) as f:
         return json.load(f)
+
+
+@pytest.fixture(scope="session")
+def oracle_vectors():
+    with open(os.path.join(ROOT, "tests", "golden", "oracle_vectors.json")) as f:
+        return json.load(f)

@@ -36,6 +36,51 @@ def _logits(gen, rows, vocab, dtype, scale=3.0):
     return (torch.randn(rows, vocab, generator=gen) * scale).to(dtype)
 
 
+def test_against_committed_oracle_vectors(dev, oracle_vectors):
+    """Fixed vectors (tests/golden/oracle_vectors.json, written by this repository's oracle) through the
+    HIP path: sweeps, index maps, advantages and the [B, L] policy losses."""
+    v = oracle_vectors["vocab"]
+    for dtype in (torch.float32, torch.bfloat16):
+        z = torch.tensor(v["logits"]).to(dtype).to(dev).requires_grad_()          # the logits are bf16-representable
+        lp, h, _ = mrl.vocab_logprob_entropy(z, torch.tensor(v["labels"]).to(dev))
+        assert (lp.cpu() - torch.tensor(v["logp"])).abs().max().item() < 1e-5
+        assert (h.cpu() - torch.tensor(v["entropy"])).abs().max().item() < 1e-5
+        (dz,) = torch.autograd.grad([lp, h], z, [torch.tensor(v["g_logp"]).to(dev), torch.tensor(v["g_entropy"]).to(dev)])
+        tol = 1e-6 if dtype == torch.float32 else TOL_DLOGITS
+        assert (dz.float().cpu() - torch.tensor(v["dlogits"])).abs().max().item() < tol
+    pk = oracle_vectors["packing"]
+    ids, labels = torch.tensor(pk["input_ids"]).to(dev), torch.tensor(pk["labels"]).to(dev)
+    mask = torch.tensor(pk["attention_mask"]).to(dev)
+    plen = torch.tensor(pk["prompt_length"], dtype=torch.int32).to(dev)
+    for align, want in pk["by_alignment"].items():
+        p_ids, p_pos, p_lab, seqlens, cu = mrl.preprocess_packed_seqs(ids, labels, mask, int(align))
+        assert p_ids.cpu().tolist() == want["ids"] and p_pos.cpu().tolist() == want["position_ids"]
+        assert p_lab.cpu().tolist() == want["labels"] and seqlens.cpu().tolist() == want["seqlens"]
+        assert cu.cpu().tolist() == want["cu_seqlens_padded"]
+        rows = torch.arange(p_ids.shape[1], dtype=torch.float32, device=dev).unsqueeze(0)
+        got = mrl.postprocess_packed_seqs(rows, seqlens, cu, 5, prompt_length=plen)
+        assert got.cpu().tolist() == want["unpacked_rows"]
+    a = oracle_vectors["advantage"]
+    rl = torch.tensor(a["response_length"]).to(dev)
+    m = mrl.generate_mask(torch.zeros(8, 3, device=dev), rl)
+    adv, _ = mrl.compute_group_norm_advantage_return(torch.tensor(a["rewards"]).to(dev), m, rl, a["group"])
+    assert (adv.cpu() - torch.tensor(a["advantages"])).abs().max().item() < 1e-6
+    pl = oracle_vectors["policy_loss"]
+    t = {k: torch.tensor(pl[k]).to(dev) for k in ("log_prob", "old_log_prob", "ref_log_prob", "advantages", "entropy", "mask")}
+    runs = {"grpo": dict(ref_log_prob=t["ref_log_prob"], clip_low=0.2, clip_high=0.2, kl_penalty="low_var_kl", kl_coef=0.01,
+                         entropy_coeff=0.003, token_level_loss=True),
+            "dapo_token": dict(ref_log_prob=None, clip_low=0.2, clip_high=0.28, entropy_coeff=0.003, token_level_loss=True),
+            "dapo_seq": dict(ref_log_prob=None, clip_low=0.2, clip_high=0.28, entropy_coeff=0.003, token_level_loss=False)}
+    for name, kwargs in runs.items():
+        want = pl["cases"][name]
+        lp = t["log_prob"].clone().requires_grad_()
+        ref = kwargs.pop("ref_log_prob")
+        loss, out = mrl.policy_loss(lp, t["entropy"], t["old_log_prob"], ref, t["advantages"], mask=t["mask"], **kwargs)
+        assert loss.item() == pytest.approx(want["outputs"][0], rel=TOL_LOSS_REL, abs=1e-7), name
+        (g,) = torch.autograd.grad(loss, lp)
+        assert (g.cpu() - torch.tensor(want["g_log_prob"])).abs().max().item() < 1e-6, name
+
+
 # --------------------------------------------------------------------------------- vocab sweep
 @pytest.mark.parametrize("dtype,vocab,rows", [
     (torch.float32, 32000, 64), (torch.bfloat16, 152064, 24), (torch.bfloat16, 129280, 16),

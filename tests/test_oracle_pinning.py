@@ -559,3 +559,68 @@ def test_pad_process_reference_vectors(reference_vectors):
     r = torch.tensor([[1.0], [3.0], [2.0], [2.0]])
     got = advantage.get_last_reward(r, 2)
     assert torch.allclose(got, torch.tensor([[-0.70710677], [0.70710677], [0.0], [0.0]]), atol=1e-6)
+
+
+def test_oracle_reproduces_its_golden_vectors(oracle_vectors):
+    """tests/golden/oracle_vectors.json was written by tests/golden/make_oracle_vectors.py from this
+    repository's oracle; replaying the script must give the same numbers (drift guard)."""
+    import importlib.util
+    import os
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "make_oracle_vectors.py")
+    spec = importlib.util.spec_from_file_location("make_oracle_vectors", path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    fresh = mod.build()
+
+    def close(a, b, where):
+        if isinstance(a, dict):
+            assert set(a) == set(b), where
+            for k in a:
+                close(a[k], b[k], where + "/" + k)
+        elif isinstance(a, list):
+            assert len(a) == len(b), where
+            for i, (x, y) in enumerate(zip(a, b)):
+                close(x, y, where + "[%d]" % i)
+        elif isinstance(a, float):
+            assert a == pytest.approx(b, rel=1e-6, abs=1e-9), where
+        else:
+            assert a == b, where
+
+    close(fresh, oracle_vectors, "")
+
+
+def test_pack_maps_property_based():
+    """Random ragged batches: packing then unpacking returns every valid position, padded sequence
+    starts are multiples of the alignment, and the index maps agree with a direct restatement."""
+    from hypothesis import given, settings, strategies as st
+
+    @settings(max_examples=60, deadline=None)
+    @given(st.lists(st.tuples(st.integers(1, 5), st.integers(0, 9)), min_size=1, max_size=6),
+           st.sampled_from([1, 2, 4, 8]), st.integers(0, 10 ** 6))
+    def check(lengths, align, seed):
+        gen = torch.Generator().manual_seed(seed)
+        batch = len(lengths)
+        plen = torch.tensor([[p] for p, _ in lengths], dtype=torch.int32)
+        rlen = torch.tensor([[r] for _, r in lengths], dtype=torch.int32)
+        width = int((plen + rlen).max())
+        ids = torch.randint(1, 1000, (batch, width), generator=gen)
+        mask = packing.generate_mask(ids, plen + rlen)
+        ids = ids * mask
+        p_ids, p_pos, _, seqlens, cu = packing.preprocess_packed_seqs(ids, ids, mask, align)
+        assert seqlens.tolist() == (plen + rlen).flatten().tolist()
+        assert all(int(c) % align == 0 for c in cu) and int(cu[-1]) == p_ids.shape[1]
+        for i in range(batch):
+            n, lo = int(seqlens[i]), int(cu[i])
+            assert p_ids[0, lo:lo + n].tolist() == ids[i, :n].tolist()
+            assert p_pos[0, lo:lo + n].tolist() == list(range(n))
+            assert not p_ids[0, lo + n:int(cu[i + 1])].any()
+        back = packing.postprocess_packed_seqs(p_ids.float(), seqlens, cu, width)
+        assert torch.equal(back.long() * mask, ids)
+        resp_w = max(int(rlen.max()), 1)
+        cut = packing.postprocess_packed_seqs(p_ids.float(), seqlens, cu, resp_w, prompt_length=plen)
+        for i in range(batch):
+            p, r = int(plen[i]), int(rlen[i])
+            want = ids[i, p - 1:p - 1 + r].tolist()
+            assert cut[i, :r].long().tolist() == want
+
+    check()
