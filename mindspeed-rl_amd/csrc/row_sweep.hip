@@ -2,16 +2,19 @@
 //
 // One workgroup of 1024 threads (16 wavefronts, one workgroup per CU) owns one logits row and
 // keeps ALL of it in registers: up to 19 16-byte vectors per thread = 311 296 bytes, enough for a
-// 152 064-entry bf16 row.  The row is loaded once (every load issued before the first use), the
-// softmax statistics and the token's loss gradient are computed from registers, and dlogits are
-// written from the same registers - one HBM read and one HBM write per element for the whole
-// forward + backward of the log-prob / policy-loss path.  Reads and writes of a workgroup are
-// separated in time, which is also the access pattern that the HBM system serves best for a
-// read+write stream.
+// 152 064-entry bf16 row.  The row is requested in one burst, the softmax statistics are taken
+// vector by vector as the data arrives, the token's loss gradient follows from them, and dlogits
+// are written from the same registers in one burst - one HBM read and one HBM write per element
+// for the whole forward + backward of the log-prob / policy-loss path.  Reads and writes of a
+// workgroup are separated in time, which is also the access pattern that the HBM system serves
+// best for a read+write stream.  All accesses are range-checked buffer accesses, so the unrolled
+// bodies contain no branch (see mrl_internal.h for why that matters).
 //
 // fused_sweep_kernel launches one workgroup per row; fused_sweep_persistent_kernel (the default
-// for large batches) launches one workgroup per CU that walks its rows, which removes the
-// workgroup launch gap between rows.
+// for large batches) launches one workgroup per CU that walks its rows and requests its next row
+// right after the stores of the current one.  bwd_rows_kernel / bwd_rows_persistent_kernel are the
+// same sweep for the split path's backward (upstream gradients and the log-sum-exp are inputs, so
+// there is no statistics pass and a row may be cut into independent segments).
 #include <stdlib.h>
 
 #include "mrl_internal.h"
