@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the actor log-prob + GRPO loss hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c0|c4chunk]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c0|c2|c4chunk|c3|c3fwd]
 
 One step = one pass of the path over one synthetic packed batch resident in HBM: the fused
 vocabulary sweep (log-prob + entropy + logsumexp), the unpack to [B, L], the fused policy loss
@@ -31,6 +31,10 @@ WORKLOADS = {
     # name: prompts, group, r_lo, r_hi, vocab, dtype, sigma, description
     "c1": dict(prompts=16, group=8, r_lo=512, r_hi=2048, vocab=152064, dtype="bf16", sigma=3.0,
                desc="configs[1]: Qwen2.5-7B-shaped GRPO actor step, 16x8 responses, R~U[512,2048], V=152064 bf16"),
+    "c2": dict(prompts=16, group=8, r_lo=512, r_hi=2048, vocab=152064, dtype="bf16", sigma=3.0, layout="padded",
+               empty_group=5, equal_group=3,
+               desc="configs[2]: the configs[1] batch as padded [B,S,V] logits (S = longest sequence), one group of "
+                    "empty responses and one group of all-equal rewards"),
     "c0": dict(prompts=4, group=4, r_lo=64, r_hi=256, vocab=32000, dtype="f32", sigma=2.0,
                desc="configs[0]: 4x4 responses, R~U[64,256], V=32000 fp32"),
     "c4chunk": dict(prompts=1, group=4, r_lo=8192, r_hi=24576, vocab=129280, dtype="bf16", sigma=3.0, loss="dapo",
@@ -66,6 +70,11 @@ def make_lengths(torch, w, seed):
     plen = torch.ones(batch, 1, dtype=torch.int32)       # the path needs prompt_length >= 1
     p = torch.rand(w["prompts"], 1, generator=gen).repeat(1, w["group"]).reshape(batch, 1)
     rewards = torch.bernoulli(p, generator=gen)
+    g = w["group"]
+    if "empty_group" in w:
+        rlen[w["empty_group"] * g:(w["empty_group"] + 1) * g] = 0
+    if "equal_group" in w:
+        rewards[w["equal_group"] * g:(w["equal_group"] + 1) * g] = 1.0
     return plen, rlen, rewards
 
 
@@ -78,6 +87,11 @@ def build_device_batch(torch, mrl, w, plen, rlen, rewards, dev, seed):
     total = int(cu[-1])
     vocab = w["vocab"]
     tdtype = torch.bfloat16 if w["dtype"] == "bf16" else torch.float32
+    padded = w.get("layout") == "padded"
+    if padded:
+        # [B, S, V] with S the longest sequence; rows past a sequence's end hold noise like the rest
+        width = int(seqlens.max())
+        total = batch * width
     logits = torch.empty(1, total, vocab, dtype=tdtype, device=dev)
     labels = torch.empty(1, total, dtype=torch.int64, device=dev)
     g = torch.Generator(device=dev).manual_seed(seed)
@@ -99,6 +113,10 @@ def build_device_batch(torch, mrl, w, plen, rlen, rewards, dev, seed):
     }
     kw = dict(use_remove_padding=True, seqlens_in_batch=seqlens.to(dev), cu_seqlens_padded=cu.to(dev),
               seq_len=int(seqlens.max()))
+    if padded:
+        logits = logits.view(batch, width, vocab)
+        b["labels"] = labels.view(batch, width)
+        kw = {}
     rmask = mrl.generate_mask(b["responses"], b["response_length"])
     if w.get("loss") == "dapo":
         # configs[4]: the chunk holds the first rows of a 16-response group; rewards Bernoulli(p), p~Beta(.5,.5);
@@ -433,7 +451,8 @@ def main():
         "dtype": w["dtype"],
         "data": "synthetic",
         "config": {
-            "workload": w["desc"], "responses": int(plen.shape[0]), "packed_rows": total, "response_tokens": tokens,
+            "workload": w["desc"], "responses": int(plen.shape[0]), "layout": w.get("layout", "packed"),
+            "packed_rows": total, "response_tokens": tokens,
             "vocab": vocab, "accumulate": "f32", "loss_kind": w.get("loss", "grpo: clip 0.2, low_var_kl 0.001"),
             "entropy_coeff": args.entropy_coeff, "loss": "token-mean", "path": args.path,
         },

@@ -931,6 +931,62 @@ def test_padded_vs_packed_and_dapo_bf16(dev, fused):
 
 
 @pytest.mark.parametrize("fused", [True, False])
+def test_padded_vs_packed_full_vocab_grpo(dev, fused):
+    """configs[2] at the configs[1] row shape (V=152064, bf16), batch scaled down: GRPO loss on the
+    padded [B,S,V] layout and on the packed one, with a group of empty responses and a group whose
+    rewards are all equal (std 0: the eps keeps its advantages at exactly zero, so only the KL
+    term drives those rows)."""
+    gen = torch.Generator().manual_seed(22)
+    group, vocab = 4, 152064
+    logits, b, kw, rewards, (ids, labels, mask1d) = _make_batch(gen, 3, group, 6, 30, vocab, torch.bfloat16, 3.0, 1)
+    rewards[:group] = 1.0                                   # all-equal group
+    rewards[2 * group:, 0] = torch.tensor([1.0, 0.0, 0.0, 1.0])
+    b["response_length"][group:2 * group] = 0               # group of empty responses
+    rmask = o_pack.generate_mask(b["responses"], b["response_length"])
+    b["advantages"], _ = o_adv.compute_group_norm_advantage_return(rewards, rmask, b["response_length"], group)
+    assert torch.equal(b["advantages"][:group], torch.zeros_like(b["advantages"][:group]))
+    assert b["advantages"][2 * group:].abs().max() > 0.5
+    adv_d, _ = mrl.compute_group_norm_advantage_return(rewards.to(dev), rmask.to(dev), b["response_length"].to(dev),
+                                                       group)
+    assert (adv_d.cpu() - b["advantages"]).abs().max().item() < TOL_LOGP
+    assert torch.equal(adv_d[:2 * group].cpu(), torch.zeros_like(b["advantages"][:2 * group]))
+    meta = dict(clip_ratio=0.2, kl_coef=0.001, kl_penalty="low_var_kl", entropy_coeff=0.001)
+    zo = logits.float().requires_grad_()
+    want_loss, want_stats = o_loss.grpo_compute_loss(zo, b, meta, **kw)
+    (dz_o,) = torch.autograd.grad(want_loss, zo)
+    f = mrl.LossFuncFactory.get_instance("ray_grpo", "actor")
+    f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.001), "kl_penalty": "low_var_kl",
+                          "entropy_coeff": 0.001})
+    bd, kwd = _to_dev(b, dev), _to_dev(kw, dev)
+    zd = logits.to(dev).requires_grad_()
+    loss, stats = f.compute_loss(zd, bd, fused=fused, **kwd)
+    assert abs(loss.item() - want_loss.item()) <= TOL_LOSS_REL * abs(want_loss.item()) + 1e-7
+    for k in want_stats:
+        assert abs(stats[k] - want_stats[k]) <= TOL_LOSS_REL * abs(want_stats[k]) + 1e-6, k
+    (dz,) = torch.autograd.grad(loss, zd)
+    assert (dz.float().cpu() - dz_o).abs().max().item() < TOL_DLOGITS
+    # rows of the empty-response group carry no gradient at all
+    seqlens, cu = kw["seqlens_in_batch"], kw["cu_seqlens_padded"]
+    for i in range(group, 2 * group):
+        assert not dz[0, cu[i]:cu[i] + seqlens[i]].any().item()
+    # the same responses in the padded layout: same loss and statistics, bit-identical gradient rows,
+    # zero gradient on the padding rows
+    batch, width = ids.shape
+    padded = torch.randn(batch, width, vocab, generator=gen).to(torch.bfloat16)     # padding rows hold noise
+    for i in range(batch):
+        padded[i, :seqlens[i]] = logits[0, cu[i]:cu[i] + seqlens[i]]
+    zp = padded.to(dev).requires_grad_()
+    loss_p, stats_p = f.compute_loss(zp, dict(bd, labels=labels.to(dev)), fused=fused)
+    assert loss_p.item() == pytest.approx(loss.item(), rel=1e-6)
+    for k in stats:
+        assert stats_p[k] == pytest.approx(stats[k], rel=1e-6, abs=1e-9)
+    (dzp,) = torch.autograd.grad(loss_p, zp)
+    for i in range(batch):
+        assert torch.equal(dzp[i, :seqlens[i]], dz[0, cu[i]:cu[i] + seqlens[i]])
+        assert not dzp[i, seqlens[i]:].any().item()
+
+
+@pytest.mark.parametrize("fused", [True, False])
 def test_ppo_actor_loss_parity(dev, fused):
     """PPO actor (the GRPO surrogate without KL, four statistics), end to end and as a stand-alone op."""
     gen = torch.Generator().manual_seed(17)
