@@ -41,6 +41,11 @@ __device__ __forceinline__ void buf_store_b16(uint16_t v, rsrc_t r, uint32_t byt
 __device__ __forceinline__ void buf_store_b32(uint32_t v, rsrc_t r, uint32_t byte_off) {
     __builtin_amdgcn_raw_buffer_store_b32(v, r, (int)byte_off, 0, 2);
 }
+// device-scope fetch-and-add through a descriptor: lanes whose offset is outside the range take no
+// part (and get 0 back), so "one lane of the workgroup" needs no branch around the instruction
+__device__ __forceinline__ uint32_t buf_atomic_add_u32(rsrc_t r, uint32_t byte_off, uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_raw_ptr_buffer_atomic_add_i32((int)v, r, (int)byte_off, 0, 0);
+}
 #else   // the host pass only has to parse the kernels
 struct rsrc_t {};
 __device__ inline rsrc_t make_rsrc(const void*, uint32_t) { return rsrc_t(); }
@@ -48,6 +53,7 @@ __device__ inline u32x4 buf_load_nt(rsrc_t, uint32_t) { return make_u32x4(0, 0, 
 __device__ inline void buf_store_nt(u32x4, rsrc_t, uint32_t) {}
 __device__ inline void buf_store_b16(uint16_t, rsrc_t, uint32_t) {}
 __device__ inline void buf_store_b32(uint32_t, rsrc_t, uint32_t) {}
+__device__ inline uint32_t buf_atomic_add_u32(rsrc_t, uint32_t, uint32_t) { return 0; }
 #endif
 
 // Single IEEE operations that stay single: HIP compiles with floating-point contraction on, and its

@@ -17,6 +17,8 @@
 // there is no statistics pass and a row may be cut into independent segments).
 #include <stdlib.h>
 
+#include <atomic>
+
 #include "mrl_internal.h"
 #include "policy_terms.h"
 #include "row_sweep.h"
@@ -136,6 +138,26 @@ __device__ __forceinline__ void zero_row(const RowRef& dst) {
     for (int q = 0; q < NV; ++q) mrl::buf_store_nt(zero, vec_rsrc(dst, q), lane_offset());
 }
 
+// Vectors [A, B) of a row: loads, zero stores.
+template <int A, int B, int NV>
+__device__ __forceinline__ void load_part(u32x4 (&v)[NV], const RowRef& src) {
+#pragma unroll
+    for (int q = A; q < B; ++q) {
+        v[q] = mrl::buf_load_nt(vec_rsrc(src, q), lane_offset());
+        vector_fence();
+    }
+}
+
+template <int A, int B>
+__device__ __forceinline__ void zero_part(const RowRef& dst) {
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int q = A; q < B; ++q) {
+        mrl::buf_store_nt(zero, vec_rsrc(dst, q), lane_offset());
+        vector_fence();
+    }
+}
+
 // Online-softmax statistics of the vectors one thread holds.  A vector past the end of the row
 // (zeros from the range-checked load) is processed like any other and its result discarded, which
 // costs three selects on the few vectors that can be affected and keeps the pass free of branches.
@@ -185,6 +207,16 @@ __device__ __forceinline__ u32x4 grad_vec(const u32x4& v, const RowGrad& g) {
 #pragma unroll
     for (int i = 0; i < kVec; ++i) d[i] = grad_elem<kEntropy>(g, z[i]);
     return E::pack(d);
+}
+
+// dlogits of vectors [A, B) of the row in registers, stored as they are computed.
+template <int DT, bool kEntropy, int A, int B, int NV>
+__device__ __forceinline__ void grad_part(const u32x4 (&v)[NV], const RowGrad& g, const RowRef& dst) {
+#pragma unroll
+    for (int q = A; q < B; ++q) {
+        mrl::buf_store_nt(grad_vec<DT, kEntropy>(v[q], g), vec_rsrc(dst, q), lane_offset());
+        vector_fence();
+    }
 }
 
 // The label's entry gets the one-hot term on top of the softmax term.  The thread that has just
@@ -310,58 +342,117 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_kernel(
     }
 }
 
-// Persistent variant of the fused sweep: one workgroup per CU walks rows r, r + grid, ... and, once
-// it has turned the registers of row r into dlogits, refills them with its NEXT row.  The loads of
-// row r+grid are in flight while the row's scalars are written and the loop turns over, and the
-// statistics pass of the next row starts on its first vectors while the last are still arriving -
-// the register file never has to hold two rows.  With kInterleave each register is refilled right
-// after its own store instead of after the last store.
-template <int DT, int NV, bool kEntropy, bool kInterleave>
+// ------------------------------------------------------------------------------ row tickets
+// The persistent kernels hand out rows through a counter: a workgroup that has finished a row takes
+// the next unclaimed one.  With a fixed stride (row r, r + grid, ...) the workgroups drift apart and
+// the rows in flight spread over a wide stretch of memory; with tickets the rows in flight are always
+// the most recent `grid` consecutive ones, which the HBM system serves about a tenth faster.
+// The counters live in device memory of the library (one array per GPU); a launch takes the next
+// slot round-robin and resets it with ticket_reset_kernel on the same stream, so launches that are
+// in flight together on different streams do not share a counter (up to kTicketSlots of them).
+constexpr int kTicketSlots = 256;
+__device__ unsigned int g_row_ticket[kTicketSlots];
+
+__global__ void ticket_reset_kernel(int slot, unsigned int first) {
+    if (threadIdx.x == 0) g_row_ticket[slot] = first;
+}
+
+// Thread 0 passes its ticket to the workgroup through LDS.  The fences order LDS accesses only and
+// the barrier is the bare instruction: __syncthreads() carries a fence over global memory as well,
+// which would wait for every outstanding store of the row that was just written.
+__device__ __forceinline__ uint32_t broadcast_ticket(uint32_t mine, uint32_t* slot) {
+    // every wavefront picks its (unused) result up here, not only the one that passes it on: a
+    // result left pending on the other path would make the next fetch-and-add wait for everything
+    asm volatile("" : "+v"(mine));
+    if (threadIdx.x == 0) *slot = mine;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    return (uint32_t)__builtin_amdgcn_readfirstlane((int)*slot);
+}
+
+// Persistent variant of the fused sweep: one workgroup per CU walks rows and, as it turns the
+// registers of a row into dlogits, refills them with its NEXT row, so the statistics pass of the next
+// row starts on its first vectors while the last are still arriving - the register file never has to
+// hold two rows.
+// kTicket: the next row is the next unclaimed one (see "row tickets" above), taken while the row is
+// being written; otherwise row r is followed by r + grid.
+template <int DT, int NV, bool kEntropy, bool kTicket>
 __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
     const typename Elem<DT>::T* logits, int64_t row_stride, int vocab, int64_t n_rows,
     const void* __restrict__ labels, int labels_dtype, float inv_t, const float* __restrict__ row_ops, int has_old,
     Params p, float grad_scale, typename Elem<DT>::T* dlogits, int64_t d_stride, float* __restrict__ logp,
-    float* __restrict__ entropy, float* __restrict__ row_terms) {
+    float* __restrict__ entropy, float* __restrict__ row_terms, int ticket_slot) {
     using E = Elem<DT>;
     using T = typename E::T;
     constexpr int kVec = E::kVec;
     __shared__ Stats lds[kWaves + 1];
+    __shared__ uint32_t next_row[2];
 
     const int tid = threadIdx.x;
     const int n_vec = vocab / kVec;
     const uint32_t row_bytes = (uint32_t)vocab * (uint32_t)sizeof(T);
     const float k = inv_t * kLog2e;
     const int64_t step = gridDim.x;
+    // the counter as a 4-byte buffer: only the lane with offset 0 (thread 0) is inside it
+    const mrl::rsrc_t ticket = mrl::make_rsrc(&g_row_ticket[ticket_slot], 4u);
 
-    // A row that is not a response token is never read: its descriptor gets zero bytes, so the
-    // (unconditional) loads return zeros without touching memory.  The label of a row and the logit
-    // at the label are requested BEFORE the row itself: loads return in order, so a request behind
-    // the row could only be used once the whole row has arrived.
-    u32x4 v[NV];
+    // What a workgroup needs to know of the row it fetches next.  A row that is not a response token
+    // is never read: its descriptor gets zero bytes, so the (unconditional) loads return zeros
+    // without touching memory; the same happens past the last row.
+    struct Next {
+        int64_t r;              // >= n_rows: none
+        int64_t y;
+        const T* zy_ptr;
+        RowRef row;
+    };
     int64_t r = blockIdx.x;
+    auto plan = [&](int64_t r2) {
+        Next n;
+        n.r = r2;
+        const bool has = r2 < n_rows;
+        const int64_t rn = has ? r2 : r;
+        const bool live = has && (row_ops[rn * MRL_ROW_OPS + MRL_OP_MASK] != 0.f);
+        const T* nrow = logits + rn * row_stride;
+        n.row = row_ref(nrow, live ? row_bytes : 0u);
+        n.y = load_label(labels, labels_dtype, rn);
+        n.zy_ptr = nrow + ((n.y >= 0 && n.y < (int64_t)vocab) ? n.y : 0);
+        return n;
+    };
+
+    // The next row is requested in two bursts: its first H vectors once the first H vectors of the
+    // current row have been written (they arrive while the rest of the gradient is computed, so the
+    // statistics pass of the next row starts without waiting for memory), the others behind the last
+    // store.  A larger H costs bandwidth: a row's requests are served best when they are issued
+    // together.  The logit at the label comes last; it is not needed before the row is reduced.
+    constexpr int H = NV >= 8 ? 4 : NV / 2;
+    u32x4 v[NV];
     int64_t y = 0;
     uint32_t zy_bits = 0;                   // the logit at the label as loaded; converted where it is used
     if (r < n_rows) {
-        const bool live = row_ops[r * MRL_ROW_OPS + MRL_OP_MASK] != 0.f;
-        const T* row = logits + r * row_stride;
-        y = load_label(labels, labels_dtype, r);
-        zy_bits = E::load_bits(row + ((y >= 0 && y < (int64_t)vocab) ? y : 0));
-        vector_fence();
-        load_row<NV>(v, row_ref(row, live ? row_bytes : 0u));
+        const Next first = plan(r);
+        y = first.y;
+        // the same sequence of operations as one turn of the loop leaves behind (with stores that
+        // write nothing), so that the number of operations outstanding at the top of the loop - which
+        // the compiler has to assume when it places the waits of the statistics pass - is the same
+        // on every path into it
+        const RowRef none = row_ref(dlogits, 0u);
+        mrl::buf_atomic_add_u32(mrl::make_rsrc(dlogits, 0u), lane_offset(), 0u);
+        zero_part<0, H>(none);
+        load_part<0, H>(v, first.row);
+        zero_part<H, NV>(none);
+        mrl::buf_store_b32(0u, mrl::make_rsrc(dlogits, 0u), 0u);
+        load_part<H, NV>(v, first.row);
+        zy_bits = E::load_bits(first.zy_ptr);
     }
-    for (; r < n_rows; r += step) {
+    int parity = 0;
+    while (r < n_rows) {
         const RowRef dst = row_ref(dlogits + r * d_stride, row_bytes);
         const float* ops = row_ops + r * MRL_ROW_OPS;
         const float m = ops[MRL_OP_MASK];
         const bool y_ok = (y >= 0) && (y < (int64_t)vocab);
-        const int64_t r2 = r + step;
-        const bool has_next = r2 < n_rows;
-        const int64_t rn = has_next ? r2 : r;
-        const bool next_live = has_next && (row_ops[rn * MRL_ROW_OPS + MRL_OP_MASK] != 0.f);
-        const T* nrow = logits + rn * row_stride;
-        const RowRef nxt = row_ref(nrow, next_live ? row_bytes : 0u);
-        const int64_t y_next = load_label(labels, labels_dtype, rn);
-        const T* zy_next_ptr = nrow + ((y_next >= 0 && y_next < (int64_t)vocab) ? y_next : 0);
+        Next nx;
+        if (!kTicket) nx = plan(r + step);
         uint32_t zy_next = 0;
 
         bool wrote = false;                 // dlogits of row r written and the next row requested
@@ -374,35 +465,37 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
             if (tid == 0) write_row_outputs(r, s, m, logp, entropy, row_terms);
             if (s.g_lp != 0.f || s.g_h != 0.f) {
                 const RowGrad g = row_grad<kEntropy>(s, k, inv_t, lse);
-                if (kInterleave) {
-                    zy_next = E::load_bits(zy_next_ptr);
-                    vector_fence();
-                }
-#pragma unroll
-                for (int q = 0; q < NV; ++q) {
-                    mrl::buf_store_nt(grad_vec<DT, kEntropy>(v[q], g), vec_rsrc(dst, q), lane_offset());
-                    if (kInterleave) v[q] = mrl::buf_load_nt(vec_rsrc(nxt, q), lane_offset());
-                    vector_fence();
-                }
+                // the ticket is asked for ahead of the stores and picked up behind the first H of
+                // them: it is older than every store, so waiting for it does not wait for them
+                uint32_t mine = 0;
+                if (kTicket) mine = mrl::buf_atomic_add_u32(ticket, lane_offset(), 1u);
+                grad_part<DT, kEntropy, 0, H>(v, g, dst);
+                if (kTicket) nx = plan((int64_t)broadcast_ticket(mine, &next_row[parity]));
+                load_part<0, H>(v, nx.row);
+                grad_part<DT, kEntropy, H, NV>(v, g, dst);
                 store_label_grad<DT, kEntropy>(dst, g, y_ok, y, z_y);
-                if (!kInterleave) {
-                    zy_next = E::load_bits(zy_next_ptr);
-                    vector_fence();
-                    load_row<NV>(v, nxt);
-                }
+                load_part<H, NV>(v, nx.row);
+                zy_next = E::load_bits(nx.zy_ptr);
                 wrote = true;
             }
         } else if (tid == 0) {
             write_masked_row_outputs(r, logp, entropy, row_terms);
         }
-        if (!wrote) {                       // no gradient for this row: zeros, then fetch the next row
-            zero_row<NV>(dst);
-            zy_next = E::load_bits(zy_next_ptr);
-            vector_fence();
-            load_row<NV>(v, nxt);
+        if (!wrote) {                       // no gradient for this row: zeros, same order of operations
+            uint32_t mine = 0;
+            if (kTicket) mine = mrl::buf_atomic_add_u32(ticket, lane_offset(), 1u);
+            zero_part<0, H>(dst);
+            if (kTicket) nx = plan((int64_t)broadcast_ticket(mine, &next_row[parity]));
+            load_part<0, H>(v, nx.row);
+            zero_part<H, NV>(dst);
+            mrl::buf_store_b32(0u, mrl::make_rsrc(dlogits, 0u), 0u);
+            load_part<H, NV>(v, nx.row);
+            zy_next = E::load_bits(nx.zy_ptr);
         }
-        y = y_next;
+        y = nx.y;
         zy_bits = zy_next;
+        r = nx.r;
+        parity ^= 1;
     }
 }
 
@@ -450,24 +543,25 @@ __global__ __launch_bounds__(kBlock) void bwd_rows_kernel(
     store_label_grad<DT, kEntropy>(dst, g, y_ok, y, E::from_bits(zy_bits));
 }
 
-// Persistent form of bwd_rows_kernel: one workgroup per CU walks rows r, r + grid, ... and requests
-// its next row right after the stores of the current one, so that the gradient arithmetic of a row
-// runs while the following row is on its way.
-template <int DT, int NV, bool kEntropy>
+// Persistent form of bwd_rows_kernel: one workgroup per CU walks units of work in ticket order (or
+// with a fixed stride) and refills its registers with the next unit in two bursts, like the fused
+// sweep above, so that the gradient arithmetic of a unit runs while the following one is on its way.
+template <int DT, int NV, bool kEntropy, bool kTicket>
 __global__ __launch_bounds__(kBlock) void bwd_rows_persistent_kernel(
-    const typename Elem<DT>::T* logits, int64_t row_stride, int vocab, int64_t n_rows, int seg_elems, int n_seg,
+    const typename Elem<DT>::T* logits, int64_t row_stride, int vocab, int64_t n_rows, int seg_elems, int seg_shift,
     const void* __restrict__ labels, int labels_dtype, float inv_t, const float* __restrict__ lse_in,
     const float* __restrict__ ent_in, const float* __restrict__ g_logp, const float* __restrict__ g_entropy,
-    typename Elem<DT>::T* dlogits, int64_t d_stride) {
+    typename Elem<DT>::T* dlogits, int64_t d_stride, int ticket_slot) {
     using E = Elem<DT>;
     using T = typename E::T;
+    __shared__ uint32_t next_unit[2];
     // The unit of work is a SEGMENT of a row: the backward needs no whole-row state (the log-sum-exp
     // is an input), so a row that does not fit the registers of a workgroup (fp32 at V = 152064) is
-    // handled as n_seg independent pieces of seg_elems entries.  Units are numbered row-major.
-    const int64_t n_units = n_rows * n_seg;
+    // handled as 2^seg_shift independent pieces of seg_elems entries.  Units are numbered row-major.
+    const int64_t n_units = n_rows << seg_shift;
     const int64_t step = gridDim.x;
-    const int64_t step_r = step / n_seg;
-    const int step_s = (int)(step % n_seg);
+    const mrl::rsrc_t ticket = mrl::make_rsrc(&g_row_ticket[ticket_slot], 4u);
+    constexpr int H = NV >= 8 ? 4 : NV / 2;
     auto grad_lp = [&](int64_t r) { return g_logp ? g_logp[r] : 0.f; };
     auto grad_h = [&](int64_t r) { return (kEntropy && g_entropy) ? g_entropy[r] : 0.f; };
     auto seg_bytes = [&](int s) {
@@ -475,43 +569,64 @@ __global__ __launch_bounds__(kBlock) void bwd_rows_persistent_kernel(
         return (uint32_t)(left < seg_elems ? left : seg_elems) * (uint32_t)sizeof(T);
     };
 
-    u32x4 v[NV];
+    struct Next {
+        int64_t u;              // >= n_units: none
+        int64_t r;
+        int s;
+        int64_t y;
+        const T* zy_ptr;
+        RowRef row;
+    };
     int64_t u = blockIdx.x;
-    int64_t r = u / n_seg;
-    int s = (int)(u - r * n_seg);
+    int64_t r = 0;
+    int s = 0;
+    auto plan = [&](int64_t u2) {
+        Next n;
+        n.u = u2;
+        const bool has = u2 < n_units;
+        const int64_t un = has ? u2 : u;
+        n.r = un >> seg_shift;
+        n.s = (int)(un & ((1 << seg_shift) - 1));
+        const bool live = has && (grad_lp(n.r) != 0.f || grad_h(n.r) != 0.f);
+        const T* nrow = logits + n.r * row_stride;
+        n.y = load_label(labels, labels_dtype, n.r);
+        n.zy_ptr = nrow + ((n.y >= 0 && n.y < (int64_t)vocab) ? n.y : 0);
+        n.row = row_ref(nrow + (int64_t)n.s * seg_elems, live ? seg_bytes(n.s) : 0u);
+        return n;
+    };
+
+    u32x4 v[NV];
     int64_t y = 0;
     uint32_t zy_bits = 0;
     if (u < n_units) {
-        const bool live = grad_lp(r) != 0.f || grad_h(r) != 0.f;
-        const T* row = logits + r * row_stride;
-        y = load_label(labels, labels_dtype, r);
-        zy_bits = E::load_bits(row + ((y >= 0 && y < (int64_t)vocab) ? y : 0));
-        vector_fence();
-        load_row<NV>(v, row_ref(row + (int64_t)s * seg_elems, live ? seg_bytes(s) : 0u));
+        const Next first = plan(u);
+        r = first.r;
+        s = first.s;
+        y = first.y;
+        // same order of operations as one turn of the loop (see the fused sweep)
+        const RowRef none = row_ref(dlogits, 0u);
+        mrl::buf_atomic_add_u32(mrl::make_rsrc(dlogits, 0u), lane_offset(), 0u);
+        zero_part<0, H>(none);
+        load_part<0, H>(v, first.row);
+        zero_part<H, NV>(none);
+        mrl::buf_store_b32(0u, mrl::make_rsrc(dlogits, 0u), 0u);
+        load_part<H, NV>(v, first.row);
+        zy_bits = E::load_bits(first.zy_ptr);
     }
-    for (; u < n_units; u += step) {
+    int parity = 0;
+    while (u < n_units) {
         const uint32_t bytes = seg_bytes(s);
         const RowRef dst = row_ref(dlogits + r * d_stride + (int64_t)s * seg_elems, bytes);
         const float g_lp = grad_lp(r), g_h = grad_h(r);
         // the label in coordinates of this segment (outside it: no one-hot term here)
         const int64_t y_local = y - (int64_t)s * seg_elems;
         const bool y_here = (y >= 0) && (y < (int64_t)vocab) && y_local >= 0 && y_local < (int64_t)seg_elems;
-        // the next unit of this workgroup
-        int64_t r2 = r + step_r;
-        int s2 = s + step_s;
-        if (s2 >= n_seg) {
-            s2 -= n_seg;
-            ++r2;
-        }
-        const bool has_next = u + step < n_units;
-        const int64_t rn = has_next ? r2 : r;
-        const int sn = has_next ? s2 : s;
-        const bool next_live = has_next && (grad_lp(rn) != 0.f || grad_h(rn) != 0.f);
-        const T* nrow = logits + rn * row_stride;
-        const int64_t y_next = load_label(labels, labels_dtype, rn);
-        const T* zy_next_ptr = nrow + ((y_next >= 0 && y_next < (int64_t)vocab) ? y_next : 0);
-        const RowRef nxt = row_ref(nrow + (int64_t)sn * seg_elems, next_live ? seg_bytes(sn) : 0u);
+        Next nx;
+        if (!kTicket) nx = plan(u + step);
         uint32_t zy_next = 0;
+        // both paths are written out in full (after a join the compiler would wait for every store of
+        // the unit before the first load of the next), and as "done / not done" rather than if / else,
+        // which keeps the register allocator from copying the row at the join
         bool wrote = false;
         if (g_lp != 0.f || g_h != 0.f) {
             const float lse = lse_in[r];
@@ -521,29 +636,34 @@ __global__ __launch_bounds__(kBlock) void bwd_rows_persistent_kernel(
             g.c0 = kEntropy ? inv_t * (-g_lp + g_h * (lse - ent_in[r])) : -g_lp * inv_t;
             g.c1 = kEntropy ? -g_h * inv_t * inv_t : 0.f;
             g.onehot = g_lp * inv_t;
-#pragma unroll
-            for (int q = 0; q < NV; ++q) {
-                mrl::buf_store_nt(grad_vec<DT, kEntropy>(v[q], g), vec_rsrc(dst, q), lane_offset());
-                vector_fence();
-            }
+            uint32_t mine = 0;
+            if (kTicket) mine = mrl::buf_atomic_add_u32(ticket, lane_offset(), 1u);
+            grad_part<DT, kEntropy, 0, H>(v, g, dst);
+            if (kTicket) nx = plan((int64_t)broadcast_ticket(mine, &next_unit[parity]));
+            load_part<0, H>(v, nx.row);
+            grad_part<DT, kEntropy, H, NV>(v, g, dst);
             store_label_grad<DT, kEntropy>(dst, g, y_here, y_local, E::from_bits(zy_bits));
-            // the refill is written out on both paths: after a join the compiler would wait for
-            // every store of the row before the first load of the next
-            zy_next = E::load_bits(zy_next_ptr);
-            vector_fence();
-            load_row<NV>(v, nxt);
+            load_part<H, NV>(v, nx.row);
+            zy_next = E::load_bits(nx.zy_ptr);
             wrote = true;
         }
         if (!wrote) {
-            zero_row<NV>(dst);
-            zy_next = E::load_bits(zy_next_ptr);
-            vector_fence();
-            load_row<NV>(v, nxt);
+            uint32_t mine = 0;
+            if (kTicket) mine = mrl::buf_atomic_add_u32(ticket, lane_offset(), 1u);
+            zero_part<0, H>(dst);
+            if (kTicket) nx = plan((int64_t)broadcast_ticket(mine, &next_unit[parity]));
+            load_part<0, H>(v, nx.row);
+            zero_part<H, NV>(dst);
+            mrl::buf_store_b32(0u, mrl::make_rsrc(dlogits, 0u), 0u);
+            load_part<H, NV>(v, nx.row);
+            zy_next = E::load_bits(nx.zy_ptr);
         }
         zy_bits = zy_next;
-        y = y_next;
-        r = r2;
-        s = s2;
+        y = nx.y;
+        u = nx.u;
+        r = nx.r;
+        s = nx.s;
+        parity ^= 1;
     }
 }
 
@@ -598,13 +718,22 @@ bool persistent_enabled() {
     return on;
 }
 
-// MRL_SWEEP_INTERLEAVE=1 refills each register right after its own store (a tuning switch).
-bool interleave_enabled() {
+// MRL_SWEEP_TICKET=0 walks rows with a fixed stride instead of tickets (a tuning switch).
+bool ticket_enabled() {
     static const bool on = [] {
-        const char* e = getenv("MRL_SWEEP_INTERLEAVE");
-        return e && e[0] == '1';
+        const char* e = getenv("MRL_SWEEP_TICKET");
+        return !(e && e[0] == '0');
     }();
     return on;
+}
+
+// Next counter slot, reset on the launch stream to the first row that is not handed out by
+// blockIdx (the workgroups start on rows 0 .. grid-1).
+int take_ticket_slot(unsigned first_ticket, hipStream_t stream) {
+    static std::atomic<unsigned> next{0};
+    const int slot = (int)(next.fetch_add(1u) % (unsigned)kTicketSlots);
+    hipLaunchKernelGGL(ticket_reset_kernel, dim3(1), dim3(64), 0, stream, slot, first_ticket);
+    return slot;
 }
 
 template <int DT, int NV>
@@ -615,14 +744,15 @@ int launch_fused(const mrl::FusedArgs& a) {
     const int cus = persistent_enabled() ? cu_count() : 0;
     if (cus > 0 && a.n_rows > 2 * (int64_t)cus) {
         const dim3 pgrid((unsigned)cus);
-#define MRL_FUSEDP_LAUNCH(ENT, IL)                                                                                \
-    hipLaunchKernelGGL((fused_sweep_persistent_kernel<DT, NV, ENT, IL>), pgrid, block, 0, a.stream, (const T*)a.logits, \
+#define MRL_FUSEDP_LAUNCH(ENT, TK)                                                                                \
+    hipLaunchKernelGGL((fused_sweep_persistent_kernel<DT, NV, ENT, TK>), pgrid, block, 0, a.stream, (const T*)a.logits, \
                        a.row_stride, (int)a.vocab, a.n_rows, a.labels, a.labels_dtype, a.inv_t, a.row_ops,         \
-                       a.has_old, p, a.grad_scale, (T*)a.dlogits, a.d_stride, a.logp, a.entropy, a.row_terms)
-        const bool il = interleave_enabled();
-        if (a.with_entropy && il) MRL_FUSEDP_LAUNCH(true, true);
+                       a.has_old, p, a.grad_scale, (T*)a.dlogits, a.d_stride, a.logp, a.entropy, a.row_terms, slot)
+        const bool tk = ticket_enabled();
+        const int slot = tk ? take_ticket_slot((unsigned)cus, a.stream) : 0;
+        if (a.with_entropy && tk) MRL_FUSEDP_LAUNCH(true, true);
         else if (a.with_entropy) MRL_FUSEDP_LAUNCH(true, false);
-        else if (il) MRL_FUSEDP_LAUNCH(false, true);
+        else if (tk) MRL_FUSEDP_LAUNCH(false, true);
         else MRL_FUSEDP_LAUNCH(false, false);
 #undef MRL_FUSEDP_LAUNCH
         return mrl::check_launch("mrl_fused_logprob_loss");
@@ -660,12 +790,18 @@ int launch_bwd_rows_nv(const mrl::BwdArgs& a) {
         const int64_t units = a.n_rows * a.n_seg;
         const int64_t want = cus > 0 ? cus : 256;
         const dim3 pgrid((unsigned)(units < want ? units : want));
-#define MRL_BWDP_LAUNCH(ENT)                                                                                      \
-    hipLaunchKernelGGL((bwd_rows_persistent_kernel<DT, NV, ENT>), pgrid, block, 0, a.stream, (const T*)a.logits,  \
-                       a.row_stride, (int)a.vocab, a.n_rows, seg_elems, a.n_seg, a.labels, a.labels_dtype, a.inv_t,   \
-                       a.lse, a.entropy, a.g_logp, a.g_entropy, (T*)a.dlogits, a.d_stride)
-        if (a.g_entropy != nullptr) MRL_BWDP_LAUNCH(true);
-        else MRL_BWDP_LAUNCH(false);
+#define MRL_BWDP_LAUNCH(ENT, TK)                                                                                  \
+    hipLaunchKernelGGL((bwd_rows_persistent_kernel<DT, NV, ENT, TK>), pgrid, block, 0, a.stream, (const T*)a.logits, \
+                       a.row_stride, (int)a.vocab, a.n_rows, seg_elems, seg_shift, a.labels, a.labels_dtype, a.inv_t, \
+                       a.lse, a.entropy, a.g_logp, a.g_entropy, (T*)a.dlogits, a.d_stride, slot)
+        int seg_shift = 0;
+        while ((1 << seg_shift) < a.n_seg) ++seg_shift;
+        const bool tk = ticket_enabled();
+        const int slot = tk ? take_ticket_slot(pgrid.x, a.stream) : 0;
+        if (a.g_entropy != nullptr && tk) MRL_BWDP_LAUNCH(true, true);
+        else if (a.g_entropy != nullptr) MRL_BWDP_LAUNCH(true, false);
+        else if (tk) MRL_BWDP_LAUNCH(false, true);
+        else MRL_BWDP_LAUNCH(false, false);
 #undef MRL_BWDP_LAUNCH
         return mrl::check_launch("mrl_vocab_logprob_bwd");
     }
@@ -689,7 +825,8 @@ namespace mrl {
 int launch_bwd_rows(const BwdArgs& a0) {
     BwdArgs a = a0;
     const int64_t n_vec = a.vocab / (16 / float_dtype_bytes(a.dtype));
-    a.n_seg = (int)((n_vec + (int64_t)kMaxVecPerThread * kBlock - 1) / ((int64_t)kMaxVecPerThread * kBlock));
+    a.n_seg = 1;          // a power of two, so that a unit number splits into row and segment by shifting
+    while ((int64_t)a.n_seg * kMaxVecPerThread * kBlock < n_vec) a.n_seg *= 2;
     a.seg_vec = (int)((n_vec + a.n_seg - 1) / a.n_seg);
     const int nv = pick_nv(a.seg_vec);
     switch (a.dtype) {
