@@ -469,14 +469,16 @@ def main():
         "stats": {k: float(v) for k, v in stats.items()},
         "loss": float(loss.detach()),
     }
-    # practical ceilings on this box with the sweeps' access pattern (one workgroup per 152064-entry bf16 row)
+    # practical ceilings on this box: with the sweeps' access pattern (one workgroup per 152064-entry bf16
+    # row) and with the pattern the HBM system serves best (one vector per thread, small workgroups)
     del dz
     probe_rows, probe_row_bytes = 32768, 304128
     nbytes = probe_rows * probe_row_bytes
     src = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     dst = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     ceilings = {}
-    for mode, name, passes in ((0, "read_GBps", 1), (1, "write_GBps", 1), (2, "copy_GBps", 2)):
+    for mode, name, passes in ((0, "read_GBps", 1), (1, "write_GBps", 1), (2, "copy_GBps", 2),
+                               (3, "stream_read_GBps", 1), (4, "stream_write_GBps", 1), (5, "stream_copy_GBps", 2)):
         s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         for _ in range(2):
             _lib.call("mrl_bandwidth_probe", mode, src.data_ptr(), dst.data_ptr(), probe_rows, probe_row_bytes,
@@ -491,9 +493,10 @@ def main():
     del src, dst
     result["measured_ceiling"] = ceilings
     # a read+write stream of R read bytes and W written bytes cannot beat R/read + W/write on this box
+    best_copy = max(ceilings["copy_GBps"], ceilings["stream_copy_GBps"])
     for k in kernels.values():
-        k["frac_of_measured_copy"] = k["GBps"] / ceilings["copy_GBps"]
-    result["roofline"]["frac_of_measured_copy_ceiling"] = kernels[dominant]["GBps"] / ceilings["copy_GBps"]
+        k["frac_of_measured_copy"] = k["GBps"] / best_copy
+    result["roofline"]["frac_of_measured_copy_ceiling"] = kernels[dominant]["GBps"] / best_copy
     dz = None
     del dz
     if not args.no_cpu_baseline:

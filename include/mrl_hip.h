@@ -410,9 +410,11 @@ int mrl_copy_bytes(const void* src, void* dst, int64_t n_bytes, void* stream);
 /* Bandwidth probes with the sweeps' access pattern (one 1024-thread workgroup per row of row_bytes
  * bytes, a multiple of 16, at most 311 296): mode 0 reads n_rows rows from src (dst: 4 writable
  * bytes, never written in practice), mode 1 writes n_rows rows to dst, mode 2 copies src to dst with
- * the whole row in registers (all loads of a workgroup before its stores).  They measure the
- * practical read / write / copy ceilings that the roofline fractions are also quoted against.  No
- * counterpart in the reference. */
+ * the whole row in registers (all loads of a workgroup before its stores).  Modes 3, 4, 5 are the
+ * same read / write / copy of n_rows * row_bytes bytes as one vector per thread in small
+ * workgroups that retire at once: the requests in flight cover one compact stretch of memory,
+ * which is the pattern the HBM system serves best.  They measure the practical ceilings that the
+ * roofline fractions are also quoted against.  No counterpart in the reference. */
 int mrl_bandwidth_probe(int mode, const void* src, void* dst, int64_t n_rows, int64_t row_bytes,
                         void* stream);
 

@@ -71,6 +71,30 @@ __global__ __launch_bounds__(kProbeBlock) void probe_copy_kernel(const u32x4* __
     for (int q = 0; q < kProbeMaxVec; ++q) mrl::buf_store_nt(v[q], d, (uint32_t)(q * kProbeBlock + threadIdx.x) * 16u);
 }
 
+// The same three streams with the pattern the HBM system serves best: small workgroups that each
+// touch ONE vector per thread and retire, so that the requests in flight at any moment cover one
+// compact, advancing stretch of memory.  These are the ceilings of the machine rather than of the
+// row-per-workgroup pattern.
+__global__ __launch_bounds__(1024) void stream_read_kernel(const u32x4* __restrict__ src, int64_t n_vec,
+                                                           unsigned* __restrict__ sink) {
+    const int64_t i = (int64_t)blockIdx.x * 1024 + threadIdx.x;
+    if (i >= n_vec) return;
+    const u32x4 v = __builtin_nontemporal_load(src + i);
+    if ((v.x ^ v.y ^ v.z ^ v.w) == 0x9e3779b9u) sink[0] = v.x;
+}
+
+__global__ __launch_bounds__(256) void stream_write_kernel(u32x4* __restrict__ dst, int64_t n_vec) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const u32x4 v = {1u, 2u, 3u, 4u};
+    if (i < n_vec) dst[i] = v;
+}
+
+__global__ __launch_bounds__(64) void stream_copy_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst,
+                                                         int64_t n_vec) {
+    const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (i < n_vec) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+
 }  // namespace
 
 extern "C" int mrl_version(void) { return MRL_VERSION; }
@@ -95,19 +119,37 @@ extern "C" int mrl_copy_bytes(const void* src, void* dst, int64_t n_bytes, void*
 extern "C" int mrl_bandwidth_probe(int mode, const void* src, void* dst, int64_t n_rows, int64_t row_bytes,
                                    void* stream) {
     const char* fn = "mrl_bandwidth_probe";
-    MRL_REQUIRE(mode >= 0 && mode <= 2, MRL_ERR_INVALID_ARG, "%s: mode=%d (0 read, 1 write, 2 copy)", fn, mode);
+    MRL_REQUIRE(mode >= 0 && mode <= 5, MRL_ERR_INVALID_ARG,
+                "%s: mode=%d (0 read, 1 write, 2 copy by rows; 3 read, 4 write, 5 copy streaming)", fn, mode);
     MRL_REQUIRE(n_rows >= 0 && n_rows <= 0x7fffffffLL && row_bytes > 0 && row_bytes % 16 == 0, MRL_ERR_INVALID_ARG,
                 "%s: n_rows=%lld row_bytes=%lld (row_bytes must be a positive multiple of 16)", fn, (long long)n_rows,
                 (long long)row_bytes);
     MRL_REQUIRE(row_bytes / 16 <= (int64_t)kProbeMaxVec * kProbeBlock, MRL_ERR_UNSUPPORTED,
                 "%s: row_bytes=%lld exceeds %d bytes", fn, (long long)row_bytes, kProbeMaxVec * kProbeBlock * 16);
     if (n_rows == 0) return MRL_OK;
-    MRL_REQUIRE((mode == 1 || src != nullptr) && dst != nullptr, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+    MRL_REQUIRE((mode == 1 || mode == 4 || src != nullptr) && dst != nullptr, MRL_ERR_INVALID_ARG, "%s: NULL pointer",
+                fn);
     MRL_REQUIRE(mrl::aligned(src, 16) && mrl::aligned(dst, 16), MRL_ERR_MISALIGNED, "%s: pointers must be 16-byte aligned",
                 fn);
     hipStream_t s = mrl::as_stream(stream);
     const dim3 grid((unsigned)n_rows), block(kProbeBlock);
     const int64_t row_vec = row_bytes / 16;
+    const int64_t n_vec = n_rows * row_vec;
+    if (mode >= 3) {
+        const int64_t per = mode == 3 ? 1024 : (mode == 4 ? 256 : 64);
+        const int64_t blocks = (n_vec + per - 1) / per;
+        MRL_REQUIRE(blocks <= 0x7fffffffLL, MRL_ERR_UNSUPPORTED, "%s: %lld bytes are too many for one launch", fn,
+                    (long long)(n_vec * 16));
+        const dim3 sgrid((unsigned)blocks);
+        if (mode == 3) {
+            hipLaunchKernelGGL(stream_read_kernel, sgrid, dim3(1024), 0, s, (const u32x4*)src, n_vec, (unsigned*)dst);
+        } else if (mode == 4) {
+            hipLaunchKernelGGL(stream_write_kernel, sgrid, dim3(256), 0, s, (u32x4*)dst, n_vec);
+        } else {
+            hipLaunchKernelGGL(stream_copy_kernel, sgrid, dim3(64), 0, s, (const u32x4*)src, (u32x4*)dst, n_vec);
+        }
+        return mrl::check_launch(fn);
+    }
     if (mode == 0) {
         hipLaunchKernelGGL(probe_read_kernel, grid, block, 0, s, (const u32x4*)src, row_vec, (unsigned*)dst);
     } else if (mode == 1) {

@@ -1298,3 +1298,24 @@ def test_copy_kernel_moves_bytes(dev):
     dst = torch.zeros_like(src)
     _lib.call("mrl_copy_bytes", src.data_ptr(), dst.data_ptr(), src.numel(), _lib.stream(dev))
     assert torch.equal(src, dst)
+
+
+def test_bandwidth_probes_touch_exactly_their_range(dev):
+    """The probes the roofline is quoted against: both copy patterns copy exactly n_rows * row_bytes
+    bytes, both write patterns write exactly that many, the read patterns write nothing."""
+    rows, row_bytes = 37, 19 * 1024 * 16 - 4096 + 16
+    n = rows * row_bytes
+    src = torch.randint(0, 255, (n + 64,), dtype=torch.uint8, device=dev)
+    for mode in (2, 5):
+        dst = torch.full((n + 64,), 7, dtype=torch.uint8, device=dev)
+        _lib.call("mrl_bandwidth_probe", mode, src.data_ptr(), dst.data_ptr(), rows, row_bytes, _lib.stream(dev))
+        assert torch.equal(dst[:n], src[:n]) and (dst[n:] == 7).all().item()
+    for mode in (1, 4):
+        dst = torch.full((n + 64,), 7, dtype=torch.uint8, device=dev)
+        _lib.call("mrl_bandwidth_probe", mode, 0, dst.data_ptr(), rows, row_bytes, _lib.stream(dev))
+        want = torch.tensor([1, 2, 3, 4], dtype=torch.int32).view(torch.uint8).repeat(n // 16).to(dev)
+        assert torch.equal(dst[:n], want) and (dst[n:] == 7).all().item()
+    for mode in (0, 3):
+        sink = torch.full((64,), 7, dtype=torch.uint8, device=dev)
+        _lib.call("mrl_bandwidth_probe", mode, src.data_ptr(), sink.data_ptr(), rows, row_bytes, _lib.stream(dev))
+        assert (sink == 7).all().item()

@@ -106,7 +106,7 @@ def test_argument_validation_launches_nothing():
     assert lib.mrl_value_loss_fwd(p, p, p, None, 0, None, 0, 2, 4, 0.5, 1.0, p, None) == -1  # no mask, no lengths
     assert lib.mrl_value_loss_bwd(p, p, p, p, _lib.F32, None, 0, 2, 4, 0.5, 1.0, p, None, p, None) == -1
     # bandwidth probe
-    assert lib.mrl_bandwidth_probe(3, p, p, 1, 1024, None) == -1
+    assert lib.mrl_bandwidth_probe(6, p, p, 1, 1024, None) == -1
     assert lib.mrl_bandwidth_probe(2, p, p, 1, 1000, None) == -1
     assert lib.mrl_bandwidth_probe(2, p, p, 1, 19 * 1024 * 16 + 16, None) == -2
     assert lib.mrl_bandwidth_probe(2, None, p, 1, 1024, None) == -1
