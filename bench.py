@@ -420,7 +420,7 @@ def main():
         "mrl_vocab_logprob_bwd": live_rows * 2 * row_bytes + dead_rows * row_bytes,
         "mrl_fused_logprob_loss": live_rows * 2 * row_bytes + dead_rows * row_bytes,
     }
-    kernel_symbol = {"mrl_vocab_logprob_fwd": "vocab_fwd_kernel", "mrl_vocab_logprob_bwd": "bwd_rows_persistent_kernel",
+    kernel_symbol = {"mrl_vocab_logprob_fwd": "vocab_fwd_kernel", "mrl_vocab_logprob_bwd": "bwd_chunk_kernel",
                      "mrl_fused_logprob_loss": "fused_sweep_persistent_kernel"}
     kernels = {}
     for name, nbytes in kernel_bytes.items():

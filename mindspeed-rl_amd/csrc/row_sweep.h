@@ -32,14 +32,13 @@ struct BwdArgs {
     const float* lse; const float* entropy; const float* g_logp; const float* g_entropy;
     void* dlogits; int64_t d_stride;
     hipStream_t stream;
-    int n_seg, seg_vec;     // filled in by launch_bwd_rows: segments per row, 16-byte vectors per segment
 };
 
 // Backward of log-prob / entropy for given per-row upstream gradients, dlogits in the dtype of the
-// logits, one workgroup per row segment with the segment in registers.  Call only if bwd_rows_supported().
-int launch_bwd_rows(const BwdArgs& a);
-bool bwd_rows_supported(int dtype, int64_t vocab, const void* in, int64_t in_stride, const void* out,
-                        int64_t out_stride, int64_t n_rows);
+// logits, as a stream of 16-byte vectors.  Call only if bwd_chunks_supported().
+int launch_bwd_chunks(const BwdArgs& a);
+bool bwd_chunks_supported(int dtype, int64_t vocab, const void* in, int64_t in_stride, const void* out,
+                          int64_t out_stride, int64_t n_rows);
 
 // True if rows of this dtype / vocab / alignment fit the row-in-registers kernels.
 bool row_sweep_supported(int dtype, int64_t vocab, const void* in, int64_t in_stride, const void* out,

@@ -11,10 +11,10 @@
 // bodies contain no branch (see mrl_internal.h for why that matters).
 //
 // fused_sweep_kernel launches one workgroup per row; fused_sweep_persistent_kernel (the default
-// for large batches) launches one workgroup per CU that walks its rows and requests its next row
-// right after the stores of the current one.  bwd_rows_kernel / bwd_rows_persistent_kernel are the
-// same sweep for the split path's backward (upstream gradients and the log-sum-exp are inputs, so
-// there is no statistics pass and a row may be cut into independent segments).
+// for large batches) launches one workgroup per CU that takes rows in ticket order and requests
+// its next row while it writes the current one.  bwd_chunk_kernel is the split path's backward
+// (upstream gradients and the log-sum-exp are inputs, so there is no statistics pass and nothing
+// has to stay on chip): a plain stream of one vector per thread.
 #include <stdlib.h>
 
 #include <atomic>
@@ -31,14 +31,14 @@ using namespace mrl_loss;
 
 // Vectors of the next row that are requested early (see fused_sweep_persistent_kernel); build-time
 // tuning constants, measured on the 152064-entry bf16 row.  The fused sweep gains 4 % from an early
-// burst of 4 (its statistics pass then starts without waiting for memory); the split backward has
-// no such pass and is, within the noise, as fast with one burst behind the last store (0) as with
-// any split.
+// burst of 4: its statistics pass then starts without waiting for memory.
 #ifndef MRL_SWEEP_HEAD
 #define MRL_SWEEP_HEAD 4
 #endif
-#ifndef MRL_BWD_HEAD
-#define MRL_BWD_HEAD 0
+// Workgroup size of the streaming backward (bwd_chunk_kernel): 256 measured best (64: +2 %, 128:
+// +14 %, 1024: +8 % in time).
+#ifndef MRL_BWD_CHUNK_THREADS
+#define MRL_BWD_CHUNK_THREADS 256
 #endif
 #ifndef MRL_SWEEP_HEAD2
 #define MRL_SWEEP_HEAD2 0
@@ -521,35 +521,38 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
     }
 }
 
-// Backward for given upstream gradients (the split path): the row is loaded into registers in one
-// burst, turned into dlogits and stored in one burst - the access pattern of the copy probe, which
-// a streaming loop of loads and stores does not reach.
-template <int DT, int NV, bool kEntropy>
-__global__ __launch_bounds__(kBlock) void bwd_rows_kernel(
-    const typename Elem<DT>::T* logits, int64_t row_stride, int vocab, const void* __restrict__ labels,
-    int labels_dtype, float inv_t, const float* __restrict__ lse_in, const float* __restrict__ ent_in,
-    const float* __restrict__ g_logp, const float* __restrict__ g_entropy, typename Elem<DT>::T* dlogits,
-    int64_t d_stride) {
+// Backward of the split path as a plain stream: one 16-byte vector per thread, small workgroups that
+// retire at once.  The backward needs no whole-row state (the log-sum-exp is an input), so nothing
+// has to stay on chip, and this is the access pattern the HBM system serves best: the requests in
+// flight always cover one compact, advancing stretch of the logits and of dlogits.  Grid: x walks
+// the row in chunks of kThreads vectors, (y, z) number the rows; x is dispatched fastest, so the
+// workgroups in flight are neighbours in memory.  A row with no incoming gradient is zero-filled
+// without being read; a vector past the end of the row is neither read nor written (range checks).
+constexpr int kChunkRowsY = 32768;      // rows per grid.y; grid.z carries the rest
+
+template <int DT, bool kEntropy, int kThreads>
+__global__ __launch_bounds__(kThreads) void bwd_chunk_kernel(
+    const typename Elem<DT>::T* logits, int64_t row_stride, int vocab, int64_t n_rows,
+    const void* __restrict__ labels, int labels_dtype, float inv_t, const float* __restrict__ lse_in,
+    const float* __restrict__ ent_in, const float* __restrict__ g_logp, const float* __restrict__ g_entropy,
+    typename Elem<DT>::T* dlogits, int64_t d_stride) {
     using E = Elem<DT>;
     using T = typename E::T;
-    const int64_t r = blockIdx.x;
+    constexpr int kVec = E::kVec;
+    const int64_t r = (int64_t)blockIdx.z * kChunkRowsY + blockIdx.y;
+    if (r >= n_rows) return;
     const uint32_t row_bytes = (uint32_t)vocab * (uint32_t)sizeof(T);
-    const T* row = logits + r * row_stride;
-    const RowRef dst = row_ref(dlogits + r * d_stride, row_bytes);
-
+    const uint32_t first = blockIdx.x * (uint32_t)kThreads;           // first vector of this workgroup
+    const uint32_t off = (first + threadIdx.x) * 16u;
+    const mrl::rsrc_t dst = mrl::make_rsrc(dlogits + r * d_stride, row_bytes);
     const float g_lp = g_logp ? g_logp[r] : 0.f;
     const float g_h = (kEntropy && g_entropy) ? g_entropy[r] : 0.f;
-    if (g_lp == 0.f && g_h == 0.f) {      // nothing flows into this row: zeros, the logits are not read
-        zero_row<NV>(dst);
+    if (g_lp == 0.f && g_h == 0.f) {
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+        mrl::buf_store_nt(zero, dst, off);
         return;
     }
-    const int64_t y = load_label(labels, labels_dtype, r);
-    const bool y_ok = (y >= 0) && (y < (int64_t)vocab);
-    const uint32_t zy_bits = E::load_bits(row + (y_ok ? y : 0));
-    vector_fence();
-    u32x4 v[NV];
-    load_row<NV>(v, row_ref(row, row_bytes));
-
+    const u32x4 v = mrl::buf_load_nt(mrl::make_rsrc(logits + r * row_stride, row_bytes), off);
     const float lse = lse_in[r];
     RowGrad g;
     g.k = inv_t * kLog2e;
@@ -557,137 +560,22 @@ __global__ __launch_bounds__(kBlock) void bwd_rows_kernel(
     g.c0 = kEntropy ? inv_t * (-g_lp + g_h * (lse - ent_in[r])) : -g_lp * inv_t;
     g.c1 = kEntropy ? -g_h * inv_t * inv_t : 0.f;
     g.onehot = g_lp * inv_t;
+    mrl::buf_store_nt(grad_vec<DT, kEntropy>(v, g), dst, off);
+    // the entry at the label: written once more, with the one-hot term, by the thread that holds it
+    // (stores of one thread to the same address stay in program order)
+    const int64_t y = load_label(labels, labels_dtype, r);
+    if (y >= 0 && y < (int64_t)vocab) {
+        const uint32_t yv = (uint32_t)y / (uint32_t)kVec;
+        if (yv >= first && yv < first + (uint32_t)kThreads) {        // uniform over the workgroup
+            float z[kVec];
+            E::unpack(v, z);
+            const int e = (int)((uint32_t)y % (uint32_t)kVec);
+            float z_y = z[0];
 #pragma unroll
-    for (int q = 0; q < NV; ++q) {
-        mrl::buf_store_nt(grad_vec<DT, kEntropy>(v[q], g), vec_rsrc(dst, q), lane_offset());
-        vector_fence();
-    }
-    store_label_grad<DT, kEntropy>(dst, g, y_ok, y, E::from_bits(zy_bits));
-}
-
-// Persistent form of bwd_rows_kernel: one workgroup per CU walks units of work in ticket order (or
-// with a fixed stride) and refills its registers with the next unit in two bursts, like the fused
-// sweep above, so that the gradient arithmetic of a unit runs while the following one is on its way.
-template <int DT, int NV, bool kEntropy, bool kTicket>
-__global__ __launch_bounds__(kBlock) void bwd_rows_persistent_kernel(
-    const typename Elem<DT>::T* logits, int64_t row_stride, int vocab, int64_t n_rows, int seg_elems, int seg_shift,
-    const void* __restrict__ labels, int labels_dtype, float inv_t, const float* __restrict__ lse_in,
-    const float* __restrict__ ent_in, const float* __restrict__ g_logp, const float* __restrict__ g_entropy,
-    typename Elem<DT>::T* dlogits, int64_t d_stride, int ticket_slot) {
-    using E = Elem<DT>;
-    using T = typename E::T;
-    __shared__ uint32_t next_unit[2];
-    // The unit of work is a SEGMENT of a row: the backward needs no whole-row state (the log-sum-exp
-    // is an input), so a row that does not fit the registers of a workgroup (fp32 at V = 152064) is
-    // handled as 2^seg_shift independent pieces of seg_elems entries.  Units are numbered row-major.
-    const int64_t n_units = n_rows << seg_shift;
-    const int64_t step = gridDim.x;
-    const mrl::rsrc_t ticket = mrl::make_rsrc(&g_row_ticket[ticket_slot], 4u);
-    constexpr int H = NV >= 8 ? MRL_BWD_HEAD : NV / 2;
-    auto grad_lp = [&](int64_t r) { return g_logp ? g_logp[r] : 0.f; };
-    auto grad_h = [&](int64_t r) { return (kEntropy && g_entropy) ? g_entropy[r] : 0.f; };
-    auto seg_bytes = [&](int s) {
-        const int left = vocab - s * seg_elems;
-        return (uint32_t)(left < seg_elems ? left : seg_elems) * (uint32_t)sizeof(T);
-    };
-
-    struct Next {
-        int64_t u;              // >= n_units: none
-        int64_t r;
-        int s;
-        int64_t y;
-        const T* zy_ptr;
-        RowRef row;
-    };
-    int64_t u = blockIdx.x;
-    int64_t r = 0;
-    int s = 0;
-    auto plan = [&](int64_t u2) {
-        Next n;
-        n.u = u2;
-        const bool has = u2 < n_units;
-        const int64_t un = has ? u2 : u;
-        n.r = un >> seg_shift;
-        n.s = (int)(un & ((1 << seg_shift) - 1));
-        const bool live = has && (grad_lp(n.r) != 0.f || grad_h(n.r) != 0.f);
-        const T* nrow = logits + n.r * row_stride;
-        n.y = load_label(labels, labels_dtype, n.r);
-        n.zy_ptr = nrow + ((n.y >= 0 && n.y < (int64_t)vocab) ? n.y : 0);
-        n.row = row_ref(nrow + (int64_t)n.s * seg_elems, live ? seg_bytes(n.s) : 0u);
-        return n;
-    };
-
-    u32x4 v[NV];
-    int64_t y = 0;
-    uint32_t zy_bits = 0;
-    if (u < n_units) {
-        const Next first = plan(u);
-        r = first.r;
-        s = first.s;
-        y = first.y;
-        // same order of operations as one turn of the loop (see the fused sweep)
-        const RowRef none = row_ref(dlogits, 0u);
-        mrl::buf_atomic_add_u32(mrl::make_rsrc(dlogits, 0u), lane_offset(), 0u);
-        zero_part<0, H>(none);
-        load_part<0, H>(v, first.row);
-        zero_part<H, NV>(none);
-        mrl::buf_store_b32(0u, mrl::make_rsrc(dlogits, 0u), 0u);
-        load_part<H, NV>(v, first.row);
-        zy_bits = E::load_bits(first.zy_ptr);
-    }
-    int parity = 0;
-    while (u < n_units) {
-        const uint32_t bytes = seg_bytes(s);
-        const RowRef dst = row_ref(dlogits + r * d_stride + (int64_t)s * seg_elems, bytes);
-        const float g_lp = grad_lp(r), g_h = grad_h(r);
-        // the label in coordinates of this segment (outside it: no one-hot term here)
-        const int64_t y_local = y - (int64_t)s * seg_elems;
-        const bool y_here = (y >= 0) && (y < (int64_t)vocab) && y_local >= 0 && y_local < (int64_t)seg_elems;
-        Next nx;
-        if (!kTicket) nx = plan(u + step);
-        uint32_t zy_next = 0;
-        // both paths are written out in full (after a join the compiler would wait for every store of
-        // the unit before the first load of the next), and as "done / not done" rather than if / else,
-        // which keeps the register allocator from copying the row at the join
-        bool wrote = false;
-        if (g_lp != 0.f || g_h != 0.f) {
-            const float lse = lse_in[r];
-            RowGrad g;
-            g.k = inv_t * kLog2e;
-            g.lse2 = lse * kLog2e;
-            g.c0 = kEntropy ? inv_t * (-g_lp + g_h * (lse - ent_in[r])) : -g_lp * inv_t;
-            g.c1 = kEntropy ? -g_h * inv_t * inv_t : 0.f;
-            g.onehot = g_lp * inv_t;
-            uint32_t mine = 0;
-            if (kTicket) mine = mrl::buf_atomic_add_u32(ticket, lane_offset(), 1u);
-            grad_part<DT, kEntropy, 0, H>(v, g, dst);
-            if (kTicket && H > 0) nx = plan((int64_t)broadcast_ticket(mine, &next_unit[parity]));
-            load_part<0, H>(v, nx.row);
-            grad_part<DT, kEntropy, H, NV>(v, g, dst);
-            store_label_grad<DT, kEntropy>(dst, g, y_here, y_local, E::from_bits(zy_bits));
-            if (kTicket && H == 0) nx = plan((int64_t)broadcast_ticket(mine, &next_unit[parity]));
-            load_part<H, NV>(v, nx.row);
-            zy_next = E::load_bits(nx.zy_ptr);
-            wrote = true;
+            for (int i = 1; i < kVec; ++i) z_y = (e == i) ? z[i] : z_y;
+            const uint32_t y_off = (yv - first == threadIdx.x) ? (uint32_t)y * (uint32_t)sizeof(T) : 0x80000000u;
+            E::buf_store(dst, y_off, grad_elem<kEntropy>(g, z_y) + g.onehot);
         }
-        if (!wrote) {
-            uint32_t mine = 0;
-            if (kTicket) mine = mrl::buf_atomic_add_u32(ticket, lane_offset(), 1u);
-            zero_part<0, H>(dst);
-            if (kTicket && H > 0) nx = plan((int64_t)broadcast_ticket(mine, &next_unit[parity]));
-            load_part<0, H>(v, nx.row);
-            zero_part<H, NV>(dst);
-            mrl::buf_store_b32(0u, mrl::make_rsrc(dlogits, 0u), 0u);
-            if (kTicket && H == 0) nx = plan((int64_t)broadcast_ticket(mine, &next_unit[parity]));
-            load_part<H, NV>(v, nx.row);
-            zy_next = E::load_bits(nx.zy_ptr);
-        }
-        zy_bits = zy_next;
-        y = nx.y;
-        u = nx.u;
-        r = nx.r;
-        s = nx.s;
-        parity ^= 1;
     }
 }
 
@@ -804,69 +692,45 @@ int launch_fused(const mrl::FusedArgs& a) {
 template <int DT>
 int fused_by_nv(int nv, const mrl::FusedArgs& a) { MRL_NV_SWITCH(launch_fused, DT, nv, a) }
 
-template <int DT, int NV>
-int launch_bwd_rows_nv(const mrl::BwdArgs& a) {
-    using T = typename Elem<DT>::T;
-    const dim3 block(kBlock);
-    const int seg_elems = a.seg_vec * Elem<DT>::kVec;
-    const int cus = persistent_enabled() || a.n_seg > 1 ? cu_count() : 0;
-    if (a.n_seg > 1 || (cus > 0 && a.n_rows > 2 * (int64_t)cus)) {
-        const int64_t units = a.n_rows * a.n_seg;
-        const int64_t want = cus > 0 ? cus : 256;
-        const dim3 pgrid((unsigned)(units < want ? units : want));
-#define MRL_BWDP_LAUNCH(ENT, TK)                                                                                  \
-    hipLaunchKernelGGL((bwd_rows_persistent_kernel<DT, NV, ENT, TK>), pgrid, block, 0, a.stream, (const T*)a.logits, \
-                       a.row_stride, (int)a.vocab, a.n_rows, seg_elems, seg_shift, a.labels, a.labels_dtype, a.inv_t, \
-                       a.lse, a.entropy, a.g_logp, a.g_entropy, (T*)a.dlogits, a.d_stride, slot)
-        int seg_shift = 0;
-        while ((1 << seg_shift) < a.n_seg) ++seg_shift;
-        // tickets are 32-bit and every workgroup draws one past the end
-        const bool tk = ticket_enabled() && units < 0xffff0000LL;
-        const int slot = tk ? take_ticket_slot(pgrid.x, a.stream) : 0;
-        if (a.g_entropy != nullptr && tk) MRL_BWDP_LAUNCH(true, true);
-        else if (a.g_entropy != nullptr) MRL_BWDP_LAUNCH(true, false);
-        else if (tk) MRL_BWDP_LAUNCH(false, true);
-        else MRL_BWDP_LAUNCH(false, false);
-#undef MRL_BWDP_LAUNCH
-        return mrl::check_launch("mrl_vocab_logprob_bwd");
-    }
-    const dim3 grid((unsigned)a.n_rows);
-#define MRL_BWDR_LAUNCH(ENT)                                                                                   \
-    hipLaunchKernelGGL((bwd_rows_kernel<DT, NV, ENT>), grid, block, 0, a.stream, (const T*)a.logits, a.row_stride, \
-                       (int)a.vocab, a.labels, a.labels_dtype, a.inv_t, a.lse, a.entropy, a.g_logp, a.g_entropy,   \
-                       (T*)a.dlogits, a.d_stride)
-    if (a.g_entropy != nullptr) MRL_BWDR_LAUNCH(true);
-    else MRL_BWDR_LAUNCH(false);
-#undef MRL_BWDR_LAUNCH
-    return mrl::check_launch("mrl_vocab_logprob_bwd");
-}
-
-template <int DT>
-int bwd_rows_by_nv(int nv, const mrl::BwdArgs& a) { MRL_NV_SWITCH(launch_bwd_rows_nv, DT, nv, a) }
 }  // namespace
 
 namespace mrl {
 
-int launch_bwd_rows(const BwdArgs& a0) {
-    BwdArgs a = a0;
-    const int64_t n_vec = a.vocab / (16 / float_dtype_bytes(a.dtype));
-    a.n_seg = 1;          // a power of two, so that a unit number splits into row and segment by shifting
-    while ((int64_t)a.n_seg * kMaxVecPerThread * kBlock < n_vec) a.n_seg *= 2;
-    a.seg_vec = (int)((n_vec + a.n_seg - 1) / a.n_seg);
-    const int nv = pick_nv(a.seg_vec);
+template <int DT>
+static int launch_bwd_chunk(const BwdArgs& a) {
+    using T = typename Elem<DT>::T;
+    constexpr int kThreads = MRL_BWD_CHUNK_THREADS;
+    const int64_t n_vec = a.vocab / Elem<DT>::kVec;
+    const int64_t gy = a.n_rows < kChunkRowsY ? a.n_rows : kChunkRowsY;
+    const int64_t gz = (a.n_rows + kChunkRowsY - 1) / kChunkRowsY;
+    const dim3 grid((unsigned)((n_vec + kThreads - 1) / kThreads), (unsigned)gy, (unsigned)gz);
+#define MRL_BWDC_LAUNCH(ENT)                                                                                     \
+    hipLaunchKernelGGL((bwd_chunk_kernel<DT, ENT, kThreads>), grid, dim3(kThreads), 0, a.stream, (const T*)a.logits, \
+                       a.row_stride, (int)a.vocab, a.n_rows, a.labels, a.labels_dtype, a.inv_t, a.lse, a.entropy,  \
+                       a.g_logp, a.g_entropy, (T*)a.dlogits, a.d_stride)
+    if (a.g_entropy != nullptr) MRL_BWDC_LAUNCH(true);
+    else MRL_BWDC_LAUNCH(false);
+#undef MRL_BWDC_LAUNCH
+    return check_launch("mrl_vocab_logprob_bwd");
+}
+
+int launch_bwd_chunks(const BwdArgs& a) {
     switch (a.dtype) {
-        case MRL_F32: return bwd_rows_by_nv<MRL_F32>(nv, a);
-        case MRL_BF16: return bwd_rows_by_nv<MRL_BF16>(nv, a);
-        default: return bwd_rows_by_nv<MRL_F16>(nv, a);
+        case MRL_F32: return launch_bwd_chunk<MRL_F32>(a);
+        case MRL_BF16: return launch_bwd_chunk<MRL_BF16>(a);
+        default: return launch_bwd_chunk<MRL_F16>(a);
     }
 }
 
-bool bwd_rows_supported(int dtype, int64_t vocab, const void* in, int64_t in_stride, const void* out,
-                        int64_t out_stride, int64_t n_rows) {
+bool bwd_chunks_supported(int dtype, int64_t vocab, const void* in, int64_t in_stride, const void* out,
+                          int64_t out_stride, int64_t n_rows) {
     const int eb = float_dtype_bytes(dtype);
     if (eb == 0) return false;
     const int64_t per_vec = 16 / eb;
-    if (vocab % per_vec != 0 || vocab * eb < 16 * 1024 || vocab > (1LL << 30)) return false;
+    // rows of whole vectors, at least 16 KiB (below that the loop kernel with one workgroup per row has
+    // less to launch), below 2 GiB (32-bit range checks), and a grid.z within its limit
+    if (vocab % per_vec != 0 || vocab * eb < 16 * 1024 || vocab * eb >= (1LL << 31)) return false;
+    if (n_rows > (int64_t)kChunkRowsY * 65535) return false;
     if (!aligned(in, 16) || !aligned(out, 16)) return false;
     if (n_rows > 1 && ((in_stride * eb) % 16 != 0 || (out_stride * eb) % 16 != 0)) return false;
     return true;

@@ -317,10 +317,11 @@ int launch_bwd(const void* logits, int64_t n_rows, int vocab, int64_t row_stride
     return mrl::check_launch("mrl_vocab_logprob_bwd");
 }
 
-// MRL_BWD_ROWS=0 keeps the streaming backward kernel for every shape (a tuning / debugging switch).
-bool sweep_rows_enabled() {
+// MRL_BWD_CHUNK=0 keeps the one-workgroup-per-row backward kernel for every shape (a tuning /
+// debugging switch).
+bool bwd_chunks_enabled() {
     static const bool on = [] {
-        const char* e = getenv("MRL_BWD_ROWS");
+        const char* e = getenv("MRL_BWD_CHUNK");
         return !(e && e[0] == '0');
     }();
     return on;
@@ -428,13 +429,12 @@ extern "C" int mrl_vocab_logprob_bwd(const void* logits, int logits_dtype, int64
     }
     hipStream_t s = mrl::as_stream(stream);
     const int v = (int)vocab;
-    // rows that fill a 1024-thread workgroup take the row-in-registers kernel (in segments if a row is
-    // larger than the register file of a workgroup)
-    if (dlogits_dtype == logits_dtype && sweep_rows_enabled() &&
-        mrl::bwd_rows_supported(logits_dtype, vocab, logits, row_stride, dlogits, dlogits_row_stride, n_rows)) {
+    // rows from 16 KiB on, same dtype in and out: the streaming kernel (one vector per thread)
+    if (dlogits_dtype == logits_dtype && bwd_chunks_enabled() &&
+        mrl::bwd_chunks_supported(logits_dtype, vocab, logits, row_stride, dlogits, dlogits_row_stride, n_rows)) {
         const mrl::BwdArgs a = {logits, logits_dtype, n_rows, vocab, row_stride, labels, labels_dtype, inv_temperature,
-                                lse, entropy, g_logp, g_entropy, dlogits, dlogits_row_stride, s, 1, 0};
-        return mrl::launch_bwd_rows(a);
+                                lse, entropy, g_logp, g_entropy, dlogits, dlogits_row_stride, s};
+        return mrl::launch_bwd_chunks(a);
     }
 #define MRL_BWD(DI, DO)                                                                                      \
     (labels_dtype == MRL_I32                                                                                 \

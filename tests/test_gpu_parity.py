@@ -1103,10 +1103,10 @@ def test_fused_sweep_vocab_sizes(dev, dtype, vocab):
 
 @pytest.mark.parametrize("dtype,vocab", [(torch.bfloat16, 8200), (torch.float32, 4100), (torch.float16, 40960)])
 def test_persistent_row_sweeps(dev, dtype, vocab):
-    """More rows than twice the CU count: the persistent row-in-registers kernels (one workgroup per
-    CU walking rows) of the split backward and of the fused sweep, with rows that are skipped (no
-    gradient / no response token) next to each other, at the ends and a whole grid stride apart,
-    labels outside the vocabulary, a row tail that does not fill the last vector of every thread."""
+    """More rows than twice the CU count, rows from 16 KiB on: the streaming backward of the split
+    path (one vector per thread, workgroups of 256 vectors), with rows that are skipped (no gradient)
+    next to each other, at the ends and 256 rows apart, labels outside the vocabulary and in the last
+    chunk of a row, a row length that does not fill the last workgroup."""
     gen = torch.Generator().manual_seed(vocab)
     rows = 700
     z = _logits(gen, rows, vocab, dtype)
@@ -1143,17 +1143,16 @@ def test_persistent_row_sweeps(dev, dtype, vocab):
 
 
 @pytest.mark.parametrize("rows", [5, 600])
-def test_backward_rows_in_segments(dev, rows):
-    """fp32 rows of 152064 entries (608 KiB) exceed the registers of a workgroup: the backward handles
-    them as two independent segments; labels in either segment, at the seam and outside the vocabulary."""
+def test_backward_fp32_full_vocab(dev, rows):
+    """fp32 rows of 152064 entries (608 KiB, more than a workgroup's registers hold) through the split
+    backward against the closed form; labels on both sides of a workgroup's chunk boundary (256 vectors
+    of 4 entries), first, last and outside the vocabulary."""
     torch.manual_seed(rows)
     vocab = 152064
     z = (torch.randn(rows, vocab, device=dev) * 3)
     y = torch.randint(0, vocab, (rows,), device=dev)
-    seam = (vocab // 4 + 2 * 1024 * 19 - 1) // (2 * 1024 * 19)    # vectors per segment are ceil(n_vec / 2)
-    half = ((vocab // 4 + 1) // 2) * 4
+    half = 74 * 1024
     y[0], y[1], y[2], y[3], y[4] = half - 1, half, 0, vocab - 1, -100
-    assert seam == 1
     g_lp = torch.randn(rows, device=dev) * 0.1
     g_h = torch.randn(rows, device=dev) * 0.01
     g_lp[2], g_h[2] = 0.0, 0.0
