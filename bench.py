@@ -339,8 +339,8 @@ def run_lmhead_train(args):
 # HBM bytes per launch of the dominant kernel from the committed rocprofv3 --pmc summary
 # (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for the copy probe); only
 # the default workload has been profiled that way, every other run reports null.
-PROFILED_TRAFFIC_BYTES = {("c1", "fused", "mrl_fused_logprob_loss"): 104.06e9,
-                          ("c1", "split", "mrl_vocab_logprob_bwd"): 104.31e9}
+PROFILED_TRAFFIC_BYTES = {("c1", "fused", "mrl_fused_logprob_loss"): 104.05e9,
+                          ("c1", "split", "mrl_vocab_logprob_bwd"): 104.06e9}
 
 
 def _profiled_traffic(args, w, dominant):
