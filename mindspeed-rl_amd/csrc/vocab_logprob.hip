@@ -18,9 +18,15 @@ namespace {
 
 using namespace mrl_vocab;
 
-constexpr int kBlock = 256;
+#ifndef MRL_VOCAB_BLOCK
+#define MRL_VOCAB_BLOCK 256
+#endif
+#ifndef MRL_VOCAB_UNROLL
+#define MRL_VOCAB_UNROLL 4
+#endif
+constexpr int kBlock = MRL_VOCAB_BLOCK;
 constexpr int kWaves = kBlock / 64;
-constexpr int kUnroll = 4;
+constexpr int kUnroll = MRL_VOCAB_UNROLL;
 // Splits a row of `vocab` elements starting at `row` into head scalars, aligned 16-byte
 // vectors and tail scalars.
 template <typename T, int kVec>

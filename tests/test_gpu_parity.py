@@ -1318,3 +1318,68 @@ def test_bandwidth_probes_touch_exactly_their_range(dev):
         sink = torch.full((64,), 7, dtype=torch.uint8, device=dev)
         _lib.call("mrl_bandwidth_probe", mode, src.data_ptr(), sink.data_ptr(), rows, row_bytes, _lib.stream(dev))
         assert (sink == 7).all().item()
+
+
+def _raw_fused_sweep(z, y, row_ops, dz, ent, terms, stream):
+    rows, vocab = z.shape
+    _lib.call("mrl_fused_logprob_loss", z.data_ptr(), _lib.dtype_code(z), rows, vocab, vocab, y.data_ptr(), _lib.I64,
+              1.0, row_ops.data_ptr(), 1, 0.8, 1.2, 3, 0.01, 0.002, 1.0, dz.data_ptr(), vocab, None, ent.data_ptr(),
+              terms.data_ptr(), stream)
+
+
+def _raw_fused_case(dev, seed, rows, vocab):
+    gen = torch.Generator().manual_seed(seed)
+    z = _logits(gen, rows, vocab, torch.bfloat16).to(dev)
+    y = torch.randint(0, vocab, (rows,), generator=gen).to(dev)
+    ops = torch.zeros(rows, 8)
+    ops[:, 0] = -torch.rand(rows, generator=gen) * 8                   # old log-prob
+    ops[:, 1] = -torch.rand(rows, generator=gen) * 8                   # ref log-prob
+    ops[:, 2] = torch.randn(rows, generator=gen)                       # advantage
+    ops[:, 3] = (torch.rand(rows, generator=gen) > 0.2).float()        # mask: a fifth of the rows is skipped
+    ops[:, 4] = 1.0 / rows
+    ops[:, 5] = 1.0 / rows
+    return z, y, ops.to(dev)
+
+
+def test_fused_sweep_on_two_streams_and_in_a_graph(dev):
+    """The persistent sweep hands out rows through a counter that a launch resets on its own stream:
+    two sweeps in flight on two streams (different counters) and a captured sweep replayed several
+    times (the reset is a kernel, so it is part of the graph) give the results of a lone eager call,
+    bit for bit - every row's result is independent of the order in which rows are taken."""
+    rows, vocab = 1500, 8200
+    cases = [_raw_fused_case(dev, 50 + i, rows, vocab) for i in range(2)]
+    want = []
+    for z, y, ops in cases:
+        dz, ent, terms = torch.empty_like(z), torch.empty(rows, device=dev), torch.empty(rows, 8, device=dev)
+        _raw_fused_sweep(z, y, ops, dz, ent, terms, _lib.stream(dev))
+        torch.cuda.synchronize()
+        want.append((dz, ent, terms))
+        assert dz.float().abs().max().item() > 0 and not dz[ops[:, 3] == 0].any().item()
+    # two streams at once, several rounds
+    streams = [torch.cuda.Stream(device=dev) for _ in cases]
+    outs = [(torch.empty_like(c[0]), torch.empty(rows, device=dev), torch.empty(rows, 8, device=dev)) for c in cases]
+    torch.cuda.synchronize()
+    for _ in range(4):
+        for (z, y, ops), (dz, ent, terms), s in zip(cases, outs, streams):
+            _raw_fused_sweep(z, y, ops, dz, ent, terms, s.cuda_stream)
+    torch.cuda.synchronize()
+    for got, ref in zip(outs, want):
+        for a, b in zip(got, ref):
+            assert torch.equal(a, b)
+    # captured once, replayed with eager work in between
+    z, y, ops = cases[0]
+    dz, ent, terms = torch.zeros_like(z), torch.zeros(rows, device=dev), torch.zeros(rows, 8, device=dev)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _raw_fused_sweep(z, y, ops, dz, ent, terms, _lib.stream(dev))
+    for i in range(3):
+        dz.zero_()
+        ent.zero_()
+        terms.zero_()
+        other = torch.empty_like(cases[1][0])
+        _raw_fused_sweep(cases[1][0], cases[1][1], cases[1][2], other, torch.empty(rows, device=dev),
+                         torch.empty(rows, 8, device=dev), _lib.stream(dev))      # eager sweep between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(dz, want[0][0]) and torch.equal(ent, want[0][1]) and torch.equal(terms, want[0][2]), i
+        assert torch.equal(other, want[1][0])
