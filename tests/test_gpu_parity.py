@@ -1389,3 +1389,74 @@ def test_fused_sweep_on_two_streams_and_in_a_graph(dev):
         torch.cuda.synchronize()
         assert torch.equal(dz, want[0][0]) and torch.equal(ent, want[0][1]) and torch.equal(terms, want[0][2]), i
         assert torch.equal(other, want[1][0])
+
+
+def test_full_size_config1_properties(dev):
+    """configs[1] at its full size (128 responses, about 171 k packed rows x 152064 bf16 = 52 GB of
+    logits), where the oracle cannot follow: the fused sweep and the split kernels (independent code)
+    agree on loss, statistics and dlogits; every dlogits row sums to zero (the softmax gradient is
+    orthogonal to the constant vector); rows without a response token are exactly zero; and a random
+    sample of rows matches the oracle's closed forms."""
+    free, _ = torch.cuda.mem_get_info(dev)
+    if free < 190 * 2 ** 30:
+        pytest.skip("needs 190 GB of free HBM")
+    import bench
+    w = bench.WORKLOADS["c1"]
+    plen, rlen, rewards = bench.make_lengths(torch, w, 0)
+    logits, b, kw, total = bench.build_device_batch(torch, mrl, w, plen, rlen, rewards, dev, 0)
+    vocab = w["vocab"]
+    f = mrl.LossFuncFactory.get_instance("ray_grpo", "actor")
+    f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.001), "kl_penalty": "low_var_kl",
+                          "entropy_coeff": 0.001})
+    z1 = logits.detach().requires_grad_()
+    loss_f, stats_f = f.compute_loss(z1, b, fused=True, **kw)
+    (dz_f,) = torch.autograd.grad(loss_f, z1)
+    z2 = logits.detach().requires_grad_()
+    loss_s, stats_s = f.compute_loss(z2, b, fused=False, **kw)
+    (dz_s,) = torch.autograd.grad(loss_s, z2)
+    assert loss_s.item() == pytest.approx(loss_f.item(), rel=TOL_LOSS_REL)
+    for k in stats_f:
+        # ppo_kl is a mean of 171 k differences of about +-0.05 that nearly cancels (5e-6): the absolute
+        # term covers the rounding of the log-probs (ulp 1e-6 at -10) in two different summation orders
+        assert stats_s[k] == pytest.approx(stats_f[k], rel=TOL_LOSS_REL, abs=2e-6), k
+    rows_per = 8192
+    scale, worst_sum, worst_diff = 0.0, 0.0, 0.0
+    for lo in range(0, total, rows_per):
+        a = dz_f[0, lo:lo + rows_per].float()
+        scale = max(scale, a.abs().max().item())
+        worst_diff = max(worst_diff, (a - dz_s[0, lo:lo + rows_per].float()).abs().max().item())
+        worst_sum = max(worst_sum, a.sum(-1).abs().max().item())
+        del a
+    assert scale > 0
+    assert worst_diff <= 2 ** -7 * scale
+    assert worst_sum <= 0.02 * scale                    # 152 k bf16 roundings against a one-hot entry of `scale`
+    # rows that are no response token (the last row of every sequence here: prompt length 1)
+    cu = kw["cu_seqlens_padded"].cpu()
+    last = (cu[1:] - 1).long().to(dev)
+    assert not dz_f[0, last].any().item() and not dz_s[0, last].any().item()
+    del dz_s, z2
+    # a sample of rows against the oracle: log-prob, entropy, and the gradient implied by them
+    gen = torch.Generator().manual_seed(5)
+    pick = torch.randint(0, total, (48,), generator=gen)
+    zs = logits[0, pick.to(dev)].float().cpu()
+    ys = b["labels"][0, pick.to(dev)].cpu()
+    lp, h, lse = mrl.vocab_logprob_entropy(logits[0], b["labels"][0])
+    want_lp = o_vocab.compute_log_probs(zs, ys)
+    want_h = o_vocab.vocab_parallel_entropy(zs)
+    assert (lp[pick.to(dev)].cpu() - want_lp).abs().max().item() < TOL_LOGP
+    assert (h[pick.to(dev)].cpu() - want_h).abs().max().item() < TOL_LOGP
+    # dlogits of a live row is c0 * (onehot - p) - c1 * p * (z - E z): recover c0 from the label entry and
+    # check the rest of the row against the oracle's softmax with it (entropy coefficient folded into c1)
+    p = torch.softmax(zs, -1)
+    got = dz_f[0, pick.to(dev)].float().cpu()
+    ent_term = p * (zs - (p * zs).sum(-1, keepdim=True))
+    onehot = torch.zeros_like(p)
+    onehot[torch.arange(len(ys)), ys] = 1.0
+    basis0, basis1 = onehot - p, -ent_term
+    for i in range(len(pick)):
+        if not got[i].any():
+            continue
+        a = torch.stack([basis0[i], basis1[i]], 1).double()
+        coef = torch.linalg.lstsq(a, got[i].double().unsqueeze(1)).solution
+        resid = (a @ coef).squeeze(1) - got[i].double()
+        assert resid.abs().max().item() <= 2 ** -8 * got[i].abs().max().item() + 1e-12, i
