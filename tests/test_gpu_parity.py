@@ -1391,23 +1391,29 @@ def test_fused_sweep_on_two_streams_and_in_a_graph(dev):
         assert torch.equal(other, want[1][0])
 
 
-def test_full_size_config1_properties(dev):
+@pytest.mark.parametrize("workload", ["c1", "c4chunk"])
+def test_full_size_properties(dev, workload):
     """configs[1] at its full size (128 responses, about 171 k packed rows x 152064 bf16 = 52 GB of
-    logits), where the oracle cannot follow: the fused sweep and the split kernels (independent code)
-    agree on loss, statistics and dlogits; every dlogits row sums to zero (the softmax gradient is
-    orthogonal to the constant vector); rows without a response token are exactly zero; and a random
-    sample of rows matches the oracle's closed forms."""
-    free, _ = torch.cuda.mem_get_info(dev)
-    if free < 190 * 2 ** 30:
-        pytest.skip("needs 190 GB of free HBM")
+    logits) and one 64 k-row chunk of configs[4] (DAPO clip-higher, no KL, V = 129280), where the
+    oracle cannot follow: the fused sweep and the split kernels (independent code) agree on loss,
+    statistics and dlogits; every dlogits row sums to zero (the softmax gradient is orthogonal to the
+    constant vector); rows without a response token are exactly zero; and a random sample of rows
+    matches the oracle's closed forms."""
     import bench
-    w = bench.WORKLOADS["c1"]
+    w = bench.WORKLOADS[workload]
+    free, _ = torch.cuda.mem_get_info(dev)
+    if free < (190 if workload == "c1" else 70) * 2 ** 30:
+        pytest.skip("needs more free HBM")
     plen, rlen, rewards = bench.make_lengths(torch, w, 0)
     logits, b, kw, total = bench.build_device_batch(torch, mrl, w, plen, rlen, rewards, dev, 0)
-    vocab = w["vocab"]
-    f = mrl.LossFuncFactory.get_instance("ray_grpo", "actor")
-    f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.001), "kl_penalty": "low_var_kl",
-                          "entropy_coeff": 0.001})
+    if w.get("loss") == "dapo":
+        f = mrl.LossFuncFactory.get_instance("ray_dapo", "actor")
+        f.add_loss_meta_info({"clip_ratio": 0.2, "clip_higher_enable": True, "clip_ratio_low": 0.2,
+                              "clip_ratio_high": 0.28, "token_level_loss": True, "entropy_coeff": 0.001})
+    else:
+        f = mrl.LossFuncFactory.get_instance("ray_grpo", "actor")
+        f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.001), "kl_penalty": "low_var_kl",
+                              "entropy_coeff": 0.001})
     z1 = logits.detach().requires_grad_()
     loss_f, stats_f = f.compute_loss(z1, b, fused=True, **kw)
     (dz_f,) = torch.autograd.grad(loss_f, z1)
