@@ -2,13 +2,12 @@
 //
 // One workgroup of 1024 threads (16 wavefronts, one workgroup per CU) owns one logits row and
 // keeps ALL of it in registers: up to 19 16-byte vectors per thread = 311 296 bytes, enough for a
-// 152 064-entry bf16 row.  The row is requested in one burst, the softmax statistics are taken
-// vector by vector as the data arrives, the token's loss gradient follows from them, and dlogits
-// are written from the same registers in one burst - one HBM read and one HBM write per element
-// for the whole forward + backward of the log-prob / policy-loss path.  Reads and writes of a
-// workgroup are separated in time, which is also the access pattern that the HBM system serves
-// best for a read+write stream.  All accesses are range-checked buffer accesses, so the unrolled
-// bodies contain no branch (see mrl_internal.h for why that matters).
+// 152 064-entry bf16 row.  The softmax statistics are taken vector by vector as the data arrives,
+// the token's loss gradient follows from them, and dlogits are written from the same registers -
+// one HBM read and one HBM write per element for the whole forward + backward of the log-prob /
+// policy-loss path.  The requests of a row are issued together (the HBM system serves a row best
+// that way) and all accesses are range-checked buffer accesses, so the unrolled bodies contain no
+// branch (see mrl_internal.h for why that matters).
 //
 // fused_sweep_kernel launches one workgroup per row; fused_sweep_persistent_kernel (the default
 // for large batches) launches one workgroup per CU that takes rows in ticket order and requests
@@ -39,9 +38,6 @@ using namespace mrl_loss;
 // +14 %, 1024: +8 % in time).
 #ifndef MRL_BWD_CHUNK_THREADS
 #define MRL_BWD_CHUNK_THREADS 256
-#endif
-#ifndef MRL_SWEEP_HEAD2
-#define MRL_SWEEP_HEAD2 0
 #endif
 
 constexpr int kBlock = 1024;
@@ -358,7 +354,7 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_kernel(
 }
 
 // ------------------------------------------------------------------------------ row tickets
-// The persistent kernels hand out rows through a counter: a workgroup that has finished a row takes
+// The persistent kernel hands out rows through a counter: a workgroup that has finished a row takes
 // the next unclaimed one.  With a fixed stride (row r, r + grid, ...) the workgroups drift apart and
 // the rows in flight spread over a wide stretch of memory; with tickets the rows in flight are always
 // the most recent `grid` consecutive ones, which the HBM system serves about a tenth faster.
@@ -402,6 +398,8 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
     using T = typename E::T;
     constexpr int kVec = E::kVec;
     __shared__ Stats lds[kWaves + 1];
+    // two slots used in turn: thread 0 may write the ticket of the following row while a slow
+    // wavefront has yet to read this one's (one barrier per row separates a slot's reuse)
     __shared__ uint32_t next_row[2];
 
     const int tid = threadIdx.x;
@@ -441,7 +439,6 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
     // store.  A larger H costs bandwidth: a row's requests are served best when they are issued
     // together.  The logit at the label comes last; it is not needed before the row is reduced.
     constexpr int H = NV >= 8 ? MRL_SWEEP_HEAD : NV / 2;
-    constexpr int H2 = (NV >= 16 && MRL_SWEEP_HEAD2 > H) ? MRL_SWEEP_HEAD2 : H;   // H2 == H: two bursts
     u32x4 v[NV];
     int64_t y = 0;
     uint32_t zy_bits = 0;                   // the logit at the label as loaded; converted where it is used
@@ -456,11 +453,9 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
         mrl::buf_atomic_add_u32(mrl::make_rsrc(dlogits, 0u), lane_offset(), 0u);
         zero_part<0, H>(none);
         load_part<0, H>(v, first.row);
-        zero_part<H, H2>(none);
-        load_part<H, H2>(v, first.row);
-        zero_part<H2, NV>(none);
+        zero_part<H, NV>(none);
         mrl::buf_store_b32(0u, mrl::make_rsrc(dlogits, 0u), 0u);
-        load_part<H2, NV>(v, first.row);
+        load_part<H, NV>(v, first.row);
         zy_bits = E::load_bits(first.zy_ptr);
     }
     int parity = 0;
@@ -490,11 +485,9 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
                 grad_part<DT, kEntropy, 0, H>(v, g, dst);
                 if (kTicket) nx = plan((int64_t)broadcast_ticket(mine, &next_row[parity]));
                 load_part<0, H>(v, nx.row);
-                grad_part<DT, kEntropy, H, H2>(v, g, dst);
-                load_part<H, H2>(v, nx.row);
-                grad_part<DT, kEntropy, H2, NV>(v, g, dst);
+                grad_part<DT, kEntropy, H, NV>(v, g, dst);
                 store_label_grad<DT, kEntropy>(dst, g, y_ok, y, z_y);
-                load_part<H2, NV>(v, nx.row);
+                load_part<H, NV>(v, nx.row);
                 zy_next = E::load_bits(nx.zy_ptr);
                 wrote = true;
             }
@@ -507,11 +500,9 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
             zero_part<0, H>(dst);
             if (kTicket) nx = plan((int64_t)broadcast_ticket(mine, &next_row[parity]));
             load_part<0, H>(v, nx.row);
-            zero_part<H, H2>(dst);
-            load_part<H, H2>(v, nx.row);
-            zero_part<H2, NV>(dst);
+            zero_part<H, NV>(dst);
             mrl::buf_store_b32(0u, mrl::make_rsrc(dlogits, 0u), 0u);
-            load_part<H2, NV>(v, nx.row);
+            load_part<H, NV>(v, nx.row);
             zy_next = E::load_bits(nx.zy_ptr);
         }
         y = nx.y;
