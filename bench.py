@@ -54,6 +54,8 @@ def parse_args():
     ap.add_argument("--tokens", type=int, default=163840, help="rows of the c3fwd workload")
     ap.add_argument("--entropy-coeff", type=float, default=0.001,
                     help="non-zero so that the forward computes entropy and the backward its gradient")
+    ap.add_argument("--chunk-rows", type=int, default=32768,
+                    help="c3 only: logits rows that exist at a time (chunk of the GEMM -> sweep -> GEMMs loop)")
     ap.add_argument("--path", default="fused", choices=["fused", "split"],
                     help="fused: one sweep computes log-prob, loss and dlogits (1 read + 1 write of [T,V]); "
                          "split: forward sweep, then the backward sweep from the saved logsumexp (2 reads + 1 write)")
@@ -266,7 +268,7 @@ def run_lmhead(args):
 
 def run_lmhead_train(args):
     """configs[3]: GRPO loss as in configs[1] but from hidden [T, 3584] and W [152064, 3584]; backward yields
-    dHidden and dW.  Logits exist for 8192 rows at a time."""
+    dHidden and dW.  Logits exist for --chunk-rows rows at a time."""
     import torch
     import mindspeed_rl_amd as mrl
     from mindspeed_rl_amd import vocab_ops
@@ -301,7 +303,7 @@ def run_lmhead_train(args):
         loss, out = mrl.fused_lmhead_policy_loss(h, wt, b, packed=True, seqlens=seqlens_d, cu_seqlens=cu_d,
                                                  ref_log_prob=ref_lp, clip_low=0.2, clip_high=0.2,
                                                  kl_penalty="low_var_kl", kl_coef=0.001,
-                                                 entropy_coeff=args.entropy_coeff)
+                                                 entropy_coeff=args.entropy_coeff, chunk_rows=args.chunk_rows)
         stats = out.cpu().tolist()
         dh, dw = torch.autograd.grad(loss, [h, wt])
         return loss, stats, dh, dw
@@ -326,7 +328,7 @@ def run_lmhead_train(args):
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "configs[3]: hidden [%d,3584] x W [152064,3584], GRPO loss as configs[1], logits only for "
-                               "8192 rows at a time" % total, "response_tokens": tokens, "accumulate": "f32",
+                               "%d rows at a time" % (total, args.chunk_rows), "response_tokens": tokens, "accumulate": "f32",
                    "gemm": "library (hipBLASLt via torch.mm)", "sweep": "fused_sweep_persistent_kernel in place"},
         "roofline": {"kernel": "whole step (3 library GEMMs + fused sweeps)", "bound": "mfma", "achieved": tflops,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS,

@@ -127,7 +127,7 @@ class _FusedLmHeadLoss(torch.autograd.Function):
         w_t = w.t()
         # The library's GEMM for dlogits_c @ W is a third faster when W is laid out [H, V] (6.7 against
         # 9.4 ms per 8192-row chunk at V = 152064, H = 3584), so one transposed copy is made per step.
-        w_hv = w_t.contiguous() if n_rows > chunk else None
+        w_hv = w_t.contiguous() if n_rows > 8192 else None
         for c0 in range(0, n_rows, chunk):
             c1 = min(n_rows, c0 + chunk)
             rows = c1 - c0
@@ -173,7 +173,7 @@ class _FusedLmHeadLoss(torch.autograd.Function):
 def fused_lmhead_policy_loss(hidden, weight, batch, *, packed, seqlens=None, cu_seqlens=None, mask=None,
                              ref_log_prob=None, clip_low, clip_high, kl_penalty=None, kl_coef=0.0, entropy_coeff=0.0,
                              token_level_loss=True, loss_scale=1.0, inv_temperature=1.0, expected_upstream=1.0,
-                             chunk_rows=8192, fp32_dw_gemm=False):
+                             chunk_rows=32768, fp32_dw_gemm=False):
     """Policy loss straight from the hidden states: ``hidden`` is packed ``[1, T, H]`` (or padded
     ``[B, S, H]``) bf16, ``weight`` the ``[V, H]`` bf16 lm_head weight; ``batch`` as for
     :func:`mindspeed_rl_amd.fused_logprob_policy_loss` (``labels, responses, response_length,
