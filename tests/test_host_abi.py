@@ -33,6 +33,24 @@ def test_library_exports_every_declared_symbol():
     assert os.path.dirname(_lib.library_path()).startswith(ROOT), "the library must live in-tree"
 
 
+def test_header_is_plain_c_and_arities_match(tmp_path):
+    """The boundary is a C ABI: the header must compile as C99 without any other include path, and the
+    ctypes table must pass as many arguments as each declaration takes."""
+    import shutil
+    import subprocess
+    header = os.path.join(ROOT, "include", "mrl_hip.h")
+    gcc = shutil.which("gcc")
+    if gcc:
+        src = tmp_path / "use_header.c"
+        src.write_text('#include "mrl_hip.h"\nint (*probe)(void) = mrl_version;\nint main(void) { return probe == 0; }\n')
+        subprocess.run([gcc, "-std=c99", "-pedantic", "-Wall", "-Werror", "-fsyntax-only", "-I",
+                        os.path.dirname(header), str(src)], check=True)
+    text = re.sub(r"/\*.*?\*/", "", open(header).read(), flags=re.S)
+    for name, params in re.findall(r"\b(mrl_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", text):
+        n = 0 if params.strip() in ("", "void") else params.count(",") + 1
+        assert len(_lib.SIGNATURES[name]) == n, name
+
+
 def test_argument_validation_launches_nothing():
     lib = _lib.load()
     # NULL logits
