@@ -1466,3 +1466,142 @@ def test_full_size_properties(dev, workload):
         coef = torch.linalg.lstsq(a, got[i].double().unsqueeze(1)).solution
         resid = (a @ coef).squeeze(1) - got[i].double()
         assert resid.abs().max().item() <= 2 ** -8 * got[i].abs().max().item() + 1e-12, i
+
+
+def _random_fused_case(i, rnd):
+    """One random case of the raw fused sweep against an fp32 torch chain on the device; returns a
+    description of the mismatch or None."""
+    dts = {torch.bfloat16: 8, torch.float16: 8, torch.float32: 4}
+    dtype = rnd.choice(list(dts))
+    per = dts[dtype]
+    max_vec = 19 * 1024
+    nvec = rnd.choice([rnd.randint(1, 64), rnd.randint(1, max_vec),
+                       rnd.choice([1024 * k + d for k in (4, 8, 12, 16, 19) for d in (-1, 0, 1)])])
+    nvec = max(1, min(nvec, max_vec))
+    vocab = nvec * per
+    rows = rnd.choice([1, 3, 257, 511, 513, 600, 777, 1100])
+    inv_t = rnd.choice([1.0, 0.7, 1.3])
+    ent_c = rnd.choice([0.0, 0.003])
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(i)
+    z = (torch.randn(rows, vocab, generator=g, device=dev) * 3).to(dtype)
+    y = torch.randint(0, vocab, (rows,), generator=g, device=dev)
+    if rows > 2:
+        y[1] = -100
+        y[2] = vocab + 3
+    ops = torch.zeros(rows, 8, device=dev)
+    ops[:, 0] = -torch.rand(rows, generator=g, device=dev) * 8
+    ops[:, 1] = -torch.rand(rows, generator=g, device=dev) * 8
+    ops[:, 2] = torch.randn(rows, generator=g, device=dev)
+    ops[:, 3] = (torch.rand(rows, generator=g, device=dev) > 0.25).float()
+    ops[:, 4] = 1.0 / rows
+    ops[:, 5] = 1.0 / rows
+    dz = torch.full_like(z, 7.0)
+    ent = torch.zeros(rows, device=dev)
+    lp = torch.zeros(rows, device=dev)
+    terms = torch.zeros(rows, 8, device=dev)
+    clip_lo, clip_hi, kl_kind, kl_coef = 0.8, 1.25, 4, 0.01
+    _lib.call("mrl_fused_logprob_loss", z.data_ptr(), _lib.dtype_code(z), rows, vocab, vocab, y.data_ptr(), _lib.I64,
+              inv_t, ops.data_ptr(), 1, clip_lo, clip_hi, kl_kind, kl_coef, ent_c, 1.0, dz.data_ptr(), vocab,
+              lp.data_ptr(), ent.data_ptr() if ent_c != 0 else None, terms.data_ptr(), _lib.stream(dev))
+    zr = (z.float() * inv_t).requires_grad_()
+    logsm = torch.log_softmax(zr, -1)
+    y_ok = (y >= 0) & (y < vocab)
+    yc = y.clamp(0, vocab - 1)
+    # a label outside the vocabulary scores the row maximum and has no one-hot term (Megatron's masked gather)
+    lp_ref = torch.where(y_ok, logsm.gather(-1, yc[:, None])[:, 0], zr.max(-1).values.detach() - torch.logsumexp(zr, -1))
+    p = logsm.exp()
+    h_ref = -(p * logsm).sum(-1)
+    old, ref, adv, m, wpg, invtok = [ops[:, k] for k in range(6)]
+    ratio = torch.exp(lp_ref - old)
+    pg = torch.maximum(-adv * ratio, -adv * ratio.clamp(clip_lo, clip_hi))
+    c = (ref - lp_ref).clamp(-20, 20)
+    k3 = (torch.exp(c) - c - 1).clamp(-10, 10)
+    loss = (pg * m * wpg).sum() + kl_coef * (k3 * m * invtok).sum() - ent_c * (h_ref * m * invtok).sum()
+    (g_ref,) = torch.autograd.grad(loss, zr)
+    g_ref = g_ref * inv_t
+    live = m != 0
+    e_lp = (lp[live] - lp_ref.detach()[live]).abs().max().item() if live.any() else 0.0
+    scale = g_ref.abs().max().item() + 1e-12
+    err = (dz.float() - g_ref).abs().max().item()
+    rel = 2 ** -7 if dtype != torch.float32 else 2e-5
+    ok = e_lp < 2e-4 and err <= rel * scale + 1e-9 and not dz[~live].any().item()
+    if ent_c != 0 and live.any():
+        ok = ok and (ent[live] - h_ref.detach()[live]).abs().max().item() < 2e-4
+    return None if ok else (i, dtype, rows, vocab, inv_t, ent_c, e_lp, err, scale)
+
+
+def test_fused_sweep_random_shapes(dev):
+    """Randomised differential test of the fused sweep (all three logits dtypes, row lengths around
+    every register-tile boundary, one-row to persistent batches, temperature, entropy on and off,
+    skipped rows, labels outside the vocabulary) against an fp32 torch chain on the device."""
+    import random
+    rnd = random.Random(1234)
+    failures = [f for f in (_random_fused_case(i, rnd) for i in range(60)) if f is not None]
+    assert not failures, failures
+
+
+def _random_split_case(i, rnd):
+    """One random case of the split forward + backward against an fp32 torch chain on the device."""
+    dev = torch.device("cuda:0")
+    dtype = rnd.choice([torch.bfloat16, torch.float16, torch.float32])
+    vocab = rnd.choice([rnd.randint(1, 300), rnd.randint(300, 40000), rnd.choice([8192, 8200, 16384, 32000, 129280, 152064]),
+                        rnd.randint(1, 2500) * 8 + rnd.choice([0, 0, 1, 3, 5])])
+    rows = rnd.choice([1, 2, 17, 300, 700])
+    if rows * vocab > 60_000_000:
+        rows = max(1, 60_000_000 // vocab)
+    inv_t = rnd.choice([1.0, 0.5, 1.7])
+    pad = rnd.choice([0, 0, 8, 24])
+    g = torch.Generator(device=dev).manual_seed(1000 + i)
+    wide = (torch.randn(rows, vocab + pad, generator=g, device=dev) * 3).to(dtype)
+    z = wide[:, :vocab] if pad else wide
+    y = torch.randint(0, vocab, (rows,), generator=g, device=dev)
+    if rows > 2:
+        y[0] = -100
+        y[1] = vocab
+    g_lp = torch.randn(rows, generator=g, device=dev) * 0.1
+    g_h = torch.randn(rows, generator=g, device=dev) * 0.01
+    mode = rnd.choice(["both", "lp", "h"])
+    if rows > 2:
+        g_lp[2] = 0.0
+        g_h[2] = 0.0
+    zd = z.detach().requires_grad_()
+    lp, h, lse = mrl.vocab_logprob_entropy(zd, y, inv_temperature=inv_t)
+    outs, gs = [], []
+    if mode in ("both", "lp"):
+        outs.append(lp); gs.append(g_lp)
+    if mode in ("both", "h"):
+        outs.append(h); gs.append(g_h)
+    (dz,) = torch.autograd.grad(outs, zd, gs)
+    zr = (z.float() * inv_t).requires_grad_()
+    logsm = torch.log_softmax(zr, -1)
+    y_ok = (y >= 0) & (y < vocab)
+    yc = y.clamp(0, vocab - 1)
+    lp_ref = torch.where(y_ok, logsm.gather(-1, yc[:, None])[:, 0], zr.max(-1).values.detach() - torch.logsumexp(zr, -1))
+    h_ref = -(logsm.exp() * logsm).sum(-1)
+    tot = 0
+    if mode in ("both", "lp"):
+        tot = tot + (lp_ref * g_lp).sum()
+    if mode in ("both", "h"):
+        tot = tot + (h_ref * g_h).sum()
+    (g_ref,) = torch.autograd.grad(tot, zr)
+    g_ref = g_ref * inv_t
+    e_lp = (lp - lp_ref.detach()).abs().max().item()
+    e_h = (h - h_ref.detach()).abs().max().item()
+    scale = g_ref.abs().max().item() + 1e-12
+    err = (dz.float() - g_ref).abs().max().item()
+    rel = 2 ** -7 if dtype != torch.float32 else 3e-5
+    ok = e_lp < 2e-4 and e_h < 2e-4 and err <= rel * scale + 1e-9 and dz.dtype == dtype and dz.shape == z.shape
+    if rows > 2 and mode == "both":
+        ok = ok and not dz[2].any().item()
+    return None if ok else (i, dtype, rows, vocab, pad, inv_t, mode, e_lp, e_h, err, scale)
+
+
+def test_split_sweeps_random_shapes(dev):
+    """Randomised differential test of the split forward and backward (all logits dtypes, vocabularies
+    from 1 to 152064 including sizes that are no multiple of a vector, rows inside a wider buffer,
+    temperature, either gradient alone, rows without gradient, labels outside the vocabulary)."""
+    import random
+    rnd = random.Random(99)
+    failures = [f for f in (_random_split_case(i, rnd) for i in range(80)) if f is not None]
+    assert not failures, failures
