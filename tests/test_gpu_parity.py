@@ -1605,3 +1605,85 @@ def test_split_sweeps_random_shapes(dev):
     rnd = random.Random(99)
     failures = [f for f in (_random_split_case(i, rnd) for i in range(80)) if f is not None]
     assert not failures, failures
+
+
+def _random_loss_case(i, rnd, dev):
+    """One random actor-loss case end to end against the oracle; returns a description of the mismatch or None."""
+    gen = torch.Generator().manual_seed(5000 + i)
+    n_prompts, group = rnd.randint(1, 4), rnd.randint(2, 5)
+    r_lo = rnd.randint(1, 12); r_hi = r_lo + rnd.randint(0, 40)
+    vocab = rnd.choice([64, 1000, 4096])
+    dtype = rnd.choice([torch.float32, torch.bfloat16])
+    align = rnd.choice([1, 2, 8])
+    logits, b, kw, rewards, (ids, labels, mask1d) = _make_batch(gen, n_prompts, group, r_lo, r_hi, vocab, dtype, 2.5, align, prompt_hi=rnd.randint(1, 5))
+    batch = ids.shape[0]
+    if rnd.random() < 0.5:
+        k = rnd.randrange(batch)
+        b["response_length"][k] = 0
+    kind = rnd.choice(["grpo", "dapo_tok", "dapo_seq", "ppo"])
+    fused = rnd.random() < 0.5
+    ent = rnd.choice([0.0, 0.002])
+    layout = rnd.choice(["packed", "padded"])
+    if kind == "grpo":
+        meta = dict(clip_ratio=0.2, kl_coef=0.01, kl_penalty=rnd.choice(["low_var_kl", "kl", "abs", "mse"]), entropy_coeff=ent)
+        f = mrl.LossFuncFactory.get_instance("ray_grpo", "actor")
+        f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.01), "kl_penalty": meta["kl_penalty"], "entropy_coeff": ent})
+        ofn = o_loss.grpo_compute_loss
+    elif kind.startswith("dapo"):
+        tok = kind == "dapo_tok"
+        if not tok:
+            b["response_length"] = torch.clamp(b["response_length"], min=1)     # an all-masked row is NaN in the reference
+        meta = dict(entropy_coeff=ent, token_level_loss=tok, clip_higher_enable=True, clip_ratio_low=0.2, clip_ratio_high=0.28)
+        f = mrl.LossFuncFactory.get_instance("ray_dapo", "actor")
+        f.add_loss_meta_info(dict(meta, clip_ratio=0.2))
+        ofn = o_loss.dapo_compute_loss
+    else:
+        meta = dict(clip_ratio=0.25, entropy_coeff=ent)
+        f = mrl.LossFuncFactory.get_instance("ray_ppo", "actor")
+        f.add_loss_meta_info({"clip_ratio": 0.25, "entropy_coeff": ent, "kl_ctrl": mrl.FixedKLController(0.1)})
+        ofn = o_loss.ppo_compute_loss
+    zo = logits.float().requires_grad_()
+    want, want_stats = ofn(zo, b, meta, **kw)
+    (dz_o,) = torch.autograd.grad(want, zo)
+    bd, kwd = _to_dev(b, dev), _to_dev(kw, dev)
+    if layout == "packed":
+        zd = logits.to(dev).requires_grad_()
+        got, stats = f.compute_loss(zd, bd, fused=fused, **kwd)
+        (dz,) = torch.autograd.grad(got, zd)
+        dz_cmp = dz.float().cpu()
+    else:
+        seqlens, cu = kw["seqlens_in_batch"], kw["cu_seqlens_padded"]
+        width = ids.shape[1]
+        padded = torch.randn(batch, width, vocab, generator=gen).to(dtype)
+        for k in range(batch):
+            padded[k, :seqlens[k]] = logits[0, cu[k]:cu[k] + seqlens[k]]
+        zd = padded.to(dev).requires_grad_()
+        got, stats = f.compute_loss(zd, dict(bd, labels=labels.to(dev)), fused=fused)
+        (dzp,) = torch.autograd.grad(got, zd)
+        dz_cmp = torch.zeros_like(dz_o)
+        for k in range(batch):
+            dz_cmp[0, cu[k]:cu[k] + seqlens[k]] = dzp[k, :seqlens[k]].float().cpu()
+            if dzp[k, seqlens[k]:].any().item():
+                return (i, "padding rows not zero")
+    tol_l = 1e-4 * abs(want.item()) + 1e-7
+    if not abs(got.item() - want.item()) <= tol_l:
+        return (i, kind, fused, layout, "loss", got.item(), want.item())
+    for k in want_stats:
+        if not abs(stats[k] - want_stats[k]) <= 1e-4 * abs(want_stats[k]) + 2e-6:
+            return (i, kind, fused, layout, k, stats[k], want_stats[k])
+    scale = dz_o.abs().max().item()
+    err = (dz_cmp - dz_o).abs().max().item()
+    rel = 2 ** -7 if dtype == torch.bfloat16 else 1e-4
+    if not err <= rel * scale + 1e-9:
+        return (i, kind, fused, layout, dtype, "dlogits", err, scale)
+    return None
+
+
+def test_actor_losses_random_batches(dev):
+    """Randomised end-to-end test against the oracle: GRPO with each KL estimator, DAPO token-level and
+    sequence-mean, PPO; fused sweep and split kernels; packed (alignment 1, 2, 8) and padded layout with
+    noise in the padding rows; fp32 and bf16 logits; empty responses; entropy bonus on and off."""
+    import random
+    rnd = random.Random(7)
+    failures = [f for f in (_random_loss_case(i, rnd, dev) for i in range(80)) if f is not None]
+    assert not failures, failures
