@@ -1687,3 +1687,66 @@ def test_actor_losses_random_batches(dev):
     rnd = random.Random(7)
     failures = [f for f in (_random_loss_case(i, rnd, dev) for i in range(80)) if f is not None]
     assert not failures, failures
+
+
+def _random_index_case(i, rnd, dev):
+    """One random case of the mask / pack / unpack / window maps against the oracle, bit for bit."""
+    gen = torch.Generator().manual_seed(9000 + i)
+    batch = rnd.choice([1, 2, 5, 33, 70])
+    width = rnd.choice([1, 2, 7, 64, 131, 200])
+    align = rnd.choice([1, 2, 4, 8, 16, 64])
+    id_dtype = rnd.choice([torch.int64, torch.int32])
+    lens = torch.randint(0, width + 1, (batch, 1), generator=gen, dtype=torch.int32)
+    if rnd.random() < 0.3:
+        lens[rnd.randrange(batch)] = width
+    if rnd.random() < 0.3:
+        lens[rnd.randrange(batch)] = 0
+    plen = torch.minimum(torch.randint(1, 6, (batch, 1), generator=gen, dtype=torch.int32), torch.clamp(lens, min=1))
+    ids = torch.randint(1, 50000, (batch, width), generator=gen).to(id_dtype)
+    labels = torch.randint(1, 50000, (batch, width), generator=gen).to(id_dtype)
+    mask_o = o_pack.generate_mask(ids, lens)
+    mask = mrl.generate_mask(ids.to(dev), lens.to(dev))
+    if not (mask.dtype == mask_o.dtype and torch.equal(mask.cpu(), mask_o)):
+        return (i, "generate_mask")
+    want = o_pack.preprocess_packed_seqs(ids, labels, mask_o, align)
+    got = mrl.preprocess_packed_seqs(ids.to(dev), labels.to(dev), mask, align)
+    for k, (a, b) in enumerate(zip(got, want)):
+        if not (a.dtype == b.dtype and a.shape == b.shape and torch.equal(a.cpu(), b)):
+            return (i, "preprocess", k, batch, width, align)
+    seqlens, cu = got[3], got[4]
+    total = want[0].shape[1]
+    resp_w = rnd.choice([max(1, int(lens.max())), width, width + 3])
+    for trailing in ((), (3,)):
+        packed = torch.randn((1, total) + trailing, generator=gen)
+        for prompt in (None, plen):
+            seq_len = resp_w if prompt is not None else width
+            w = o_pack.postprocess_packed_seqs(packed, want[3], want[4], seq_len, prompt)
+            g = mrl.postprocess_packed_seqs(packed.to(dev), seqlens, cu, seq_len, None if prompt is None else prompt.to(dev))
+            if not torch.equal(g.cpu(), w):
+                return (i, "postprocess", trailing, prompt is not None, batch, width, align, resp_w)
+    # padded-layout windows
+    rlen = torch.clamp(lens - plen, min=0)
+    window = o_pack.response_window(plen, rlen)
+    responses = torch.zeros(batch, resp_w)
+    x2 = torch.randn(batch, width, generator=gen)
+    x3 = torch.randn(batch, width, 5, generator=gen)
+    w2 = o_pack.truncate_prompt_and_pad(responses, x2, window)
+    g2 = mrl.truncate_prompt_and_pad(responses.to(dev), x2.to(dev), mrl.response_window(plen.to(dev), rlen.to(dev)))
+    if not torch.equal(g2.cpu(), w2):
+        return (i, "truncate_prompt_and_pad", batch, width, resp_w)
+    w3 = o_pack.truncate_middle_and_pad(responses, x3, window)
+    g3 = mrl.truncate_middle_and_pad(responses.to(dev), x3.to(dev), mrl.response_window(plen.to(dev), rlen.to(dev)))
+    if not torch.equal(g3.cpu(), w3):
+        return (i, "truncate_middle_and_pad", batch, width, resp_w)
+    return None
+
+
+def test_index_maps_random_shapes_bit_exact(dev):
+    """Randomised bit-exact test of generate_mask, preprocess_packed_seqs (all five outputs),
+    postprocess_packed_seqs (with and without the prompt shift, with a trailing dimension) and the
+    padded-layout windows: batch 1..70, width 1..200, alignment 1..64, int32 / int64 ids, empty and
+    full-width sequences."""
+    import random
+    rnd = random.Random(3)
+    failures = [f for f in (_random_index_case(i, rnd, dev) for i in range(120)) if f is not None]
+    assert not failures, failures
