@@ -1750,3 +1750,59 @@ def test_index_maps_random_shapes_bit_exact(dev):
     rnd = random.Random(3)
     failures = [f for f in (_random_index_case(i, rnd, dev) for i in range(120)) if f is not None]
     assert not failures, failures
+
+
+def _random_wire_and_gae_case(i, rnd, dev):
+    """One random case of the experience wire format and of the GAE scan against the oracle."""
+    gen = torch.Generator().manual_seed(400 + i)
+    batch = rnd.choice([1, 2, 9, 64, 130])
+    hi = rnd.choice([2, 17, 300])
+    lens_a = torch.randint(0, hi, (batch,), generator=gen, dtype=torch.int32)
+    if int(lens_a.sum()) == 0:
+        lens_a[0] = 1
+    lens_b = torch.randint(1, 9, (batch,), generator=gen, dtype=torch.int32)
+    data = {"responses": torch.randint(0, 1000, (int(lens_a.sum()),), generator=gen),
+            "old_log_prob": torch.randn(int(lens_a.sum()), generator=gen),
+            "position_ids": torch.randint(0, 99, (3, int(lens_b.sum())), generator=gen),
+            "response_length": lens_a.clone()}
+    lens = {"responses": lens_a, "old_log_prob": lens_a, "position_ids": lens_b, "response_length": torch.ones(batch, dtype=torch.int32)}
+    multiple = rnd.choice([1, 2, 8, 16])
+    want = o_pack.unpack_pad_experience(data, lens, -7, multiple)
+    got = mrl.unpack_pad_experience({k: v.to(dev) for k, v in data.items()}, lens, -7, multiple)
+    for k in want:
+        if not (got[k].dtype == want[k].dtype and got[k].shape == want[k].shape and torch.equal(got[k].cpu(), want[k])):
+            return (i, "unpack", k, batch, hi, multiple)
+    width = rnd.choice([1, 5, 40, 257])
+    tensor = torch.randint(0, 500, (batch, width), generator=gen)
+    idx = torch.randint(0, width + 1, (batch, 1), generator=gen)
+    for left in (False, True):
+        w = o_pack.truncate_rows(tensor, idx, left)
+        g = mrl.truncate_rows(tensor.to(dev), idx.to(dev), left)
+        if len(w) != len(g) or not all(a.dtype == b.dtype and torch.equal(a.cpu(), b) for a, b in zip(g, w)):
+            return (i, "truncate_rows", left, batch, width)
+    # GAE + whitening
+    L = rnd.choice([1, 2, 33, 500, 2100])
+    r = torch.randn(batch, L, generator=gen); v = torch.randn(batch, L, generator=gen)
+    ml = torch.randint(0, L + 1, (batch,), generator=gen)
+    ml[0] = L
+    if batch > 1: ml[1] = max(1, L // 2)
+    mask = o_pack.generate_mask(torch.zeros(batch, L), ml)
+    if int(mask.sum()) < 2:
+        return None
+    gamma, lam = rnd.choice([(1.0, 0.95), (0.99, 1.0), (0.9, 0.5)])
+    wa, wr = o_adv.compute_gae_advantage_return(r, v, mask, torch.tensor(gamma), torch.tensor(lam))
+    ga, gr = mrl.compute_gae_advantage_return(r.to(dev), v.to(dev), mask.to(dev), gamma, lam)
+    if not torch.equal(gr.cpu(), wr):
+        return (i, "gae returns", batch, L, gamma, lam, (gr.cpu() - wr).abs().max().item())
+    if not (ga.cpu() - wa).abs().max().item() <= 2e-5 * max(1.0, wa.abs().max().item()):
+        return (i, "gae adv", batch, L, (ga.cpu() - wa).abs().max().item())
+    return None
+
+
+def test_wire_format_and_gae_random_shapes(dev):
+    """Randomised test of unpack_pad_experience and truncate_rows (bit-exact) and of the GAE scan
+    (returns bit-exact, also for rows longer than one staged chunk) against the oracle."""
+    import random
+    rnd = random.Random(11)
+    failures = [f for f in (_random_wire_and_gae_case(i, rnd, dev) for i in range(60)) if f is not None]
+    assert not failures, failures
