@@ -149,7 +149,11 @@ __global__ __launch_bounds__(kThreads, (kTB <= 2 ? 2 : 1)) void lmhead_fwd_kerne
 #pragma unroll
                 for (int i = 0; i < 16; ++i) vmax = fmaxf(vmax, acc[vb][tb][i]);
             grow_max<true>(st[tb], vmax, k_scale);
-            const float mk = st[tb].m * k_scale;
+            // A lane that has seen no valid vocabulary row yet (the first tile of its group is ragged and
+            // ends above its rows) still holds the start value as its maximum: z * k - m * k of the masked
+            // entries would then be the rounding residual of two numbers of magnitude 1e30 instead of
+            // zero.  With an infinite m * k their exponentials are exactly 0.
+            const float mk = st[tb].m > kMaxInit ? st[tb].m * k_scale : __builtin_inff();
 #pragma unroll
             for (int vb = 0; vb < 4; ++vb)
 #pragma unroll
@@ -389,7 +393,8 @@ __global__ __launch_bounds__(kThreads2, 1) void lmhead_fwd_kernel_v2(
 #pragma unroll
                         for (int i = 0; i < 16; ++i) vmax = fmaxf(vmax, acc[vb][tb][i]);
                     grow_max<true>(st[tb], vmax, k_scale);
-                    const float mk = st[tb].m * k_scale;
+                    // no valid vocabulary row seen yet by this lane: see the first-generation kernel
+                    const float mk = st[tb].m > kMaxInit ? st[tb].m * k_scale : __builtin_inff();
 #pragma unroll
                     for (int vb = 0; vb < 4; ++vb)
 #pragma unroll

@@ -1806,3 +1806,51 @@ def test_wire_format_and_gae_random_shapes(dev):
     rnd = random.Random(11)
     failures = [f for f in (_random_wire_and_gae_case(i, rnd, dev) for i in range(60)) if f is not None]
     assert not failures, failures
+
+
+def _random_lmhead_case(i, rnd, dev):
+    """One random case of the fused lm_head forward against an fp32 matmul + log-softmax on the device."""
+    g = torch.Generator(device=dev).manual_seed(70 + i)
+    tokens = rnd.choice([1, 2, 63, 64, 65, 255, 256, 257, 300, 511, 513, 1000])
+    vocab = rnd.choice([8, 16, 248, 256, 264, 2040, 2048, 2056, 4096 + 24, 5000, 12345 // 8 * 8, 40000])
+    hdim = rnd.choice([64, 128, 192, 256, 1024, 3584])
+    inv_t = rnd.choice([1.0, 0.6, 1.5])
+    h = torch.randn(tokens, hdim, generator=g, device=dev).to(torch.bfloat16)
+    w = (torch.randn(vocab, hdim, generator=g, device=dev) * (2.0 / hdim ** 0.5)).to(torch.bfloat16)
+    y = torch.randint(0, vocab, (tokens,), generator=g, device=dev)
+    if tokens > 2:
+        y[1] = -1
+        y[2] = vocab
+    want_ent = rnd.random() < 0.7
+    lp, ent, lse = mrl.lmhead_logprob(h, w, y, inv_temperature=inv_t, want_entropy=want_ent)
+    z = (h.float() @ w.float().t()) * inv_t
+    logsm = torch.log_softmax(z, -1)
+    y_ok = (y >= 0) & (y < vocab)
+    lp_ref = torch.where(y_ok, logsm.gather(-1, y.clamp(0, vocab - 1)[:, None])[:, 0], z.max(-1).values - torch.logsumexp(z, -1))
+    h_ref = -(logsm.exp() * logsm).sum(-1)
+    e1 = (lp - lp_ref).abs().max().item()
+    e2 = (lse - torch.logsumexp(z, -1)).abs().max().item()
+    e3 = (ent - h_ref).abs().max().item() if want_ent else ent.abs().max().item()
+    ok = e1 < 3e-4 and e2 < 2e-4 and e3 < 3e-4
+    return None if ok else (i, tokens, vocab, hdim, inv_t, want_ent, e1, e2, e3)
+
+
+def test_lmhead_forward_random_shapes(dev):
+    """Randomised test of the fused lm_head forward: token counts around the 64- and 256-token tiles,
+    vocabularies whose last 256-row tile holds 8 .. 248 rows and is the only tile of its group (a lane
+    that never sees a valid row must contribute exactly nothing), hidden sizes 64 .. 3584."""
+    import random
+    rnd = random.Random(21)
+    failures = [f for f in (_random_lmhead_case(i, rnd, dev) for i in range(60)) if f is not None]
+    assert not failures, failures
+    # the smallest ragged tiles, alone in their group
+    for tokens, vocab, hdim in [(1, 8, 64), (64, 16, 64), (2, 264, 128), (3, 24, 64), (3, 280, 64), (5, 2056, 64)]:
+        g = torch.Generator(device=dev).manual_seed(vocab)
+        h = torch.randn(tokens, hdim, generator=g, device=dev).to(torch.bfloat16)
+        w = (torch.randn(vocab, hdim, generator=g, device=dev) * 0.2).to(torch.bfloat16)
+        y = torch.randint(0, vocab, (tokens,), generator=g, device=dev)
+        lp, ent, lse = mrl.lmhead_logprob(h, w, y)
+        z = h.float() @ w.float().t()
+        assert (lse - torch.logsumexp(z, -1)).abs().max().item() < 1e-4, (tokens, vocab, hdim)
+        assert (lp - torch.log_softmax(z, -1).gather(-1, y[:, None])[:, 0]).abs().max().item() < 2e-4
+        assert torch.isfinite(ent).all().item()
