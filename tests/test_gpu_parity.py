@@ -1854,3 +1854,65 @@ def test_lmhead_forward_random_shapes(dev):
         assert (lse - torch.logsumexp(z, -1)).abs().max().item() < 1e-4, (tokens, vocab, hdim)
         assert (lp - torch.log_softmax(z, -1).gather(-1, y[:, None])[:, 0]).abs().max().item() < 2e-4
         assert torch.isfinite(ent).all().item()
+
+
+def _random_value_side_case(i, rnd, dev):
+    """One random case of the KL-penalised rewards, the critic value loss, masked whitening and the
+    group advantages against the oracle."""
+    gen = torch.Generator().manual_seed(800 + i)
+    batch = rnd.choice([1, 2, 7, 64, 257])
+    width = rnd.choice([2, 3, 31, 257, 2048, 3000])
+    old = -torch.rand(batch, width, generator=gen) * 5
+    ref = old + torch.randn(batch, width, generator=gen) * 0.3
+    lens = torch.randint(1, width + 1, (batch, 1), generator=gen)
+    scores = torch.randn(batch, generator=gen)
+    penalty = rnd.choice(["kl", "abs", "mse", "low_var_kl"])
+    want, want_kl = o_adv.kl_token_level_rewards(old, ref, lens, scores, 0.05, penalty)
+    got, got_kl = mrl.kl_token_level_rewards(old.to(dev), ref.to(dev), lens.to(dev), scores.to(dev), 0.05, penalty)
+    if not ((got.cpu() - want).abs().max().item() < 1e-6 and abs(got_kl - want_kl) <= 1e-5 * abs(want_kl) + 1e-8):
+        return (i, "kl_rewards", batch, width, penalty)
+    # value loss
+    values = torch.randn(batch, width, generator=gen)
+    vp = values + torch.randn(batch, width, generator=gen) * 0.4
+    returns = values + torch.randn(batch, width, generator=gen)
+    vlens = torch.randint(0, width + 1, (batch, 1), generator=gen)
+    vlens[0] = max(1, width // 2)
+    mask = o_pack.generate_mask(vp, vlens).float()
+    vo = vp.clone().requires_grad_()
+    w_loss, w_frac = o_loss.value_loss(vo, returns, values, mask, 0.2)
+    (g_o,) = torch.autograd.grad(w_loss, vo)
+    vd = vp.to(dev).requires_grad_()
+    g_loss, out = mrl.value_loss(vd, returns.to(dev), values.to(dev), cliprange_value=0.2, response_length=vlens.to(dev))
+    (g,) = torch.autograd.grad(g_loss, vd)
+    if not (abs(g_loss.item() - w_loss.item()) <= 1e-4 * abs(w_loss.item()) + 1e-8 and (g.cpu() - g_o).abs().max().item() < 1e-6
+            and abs(out[2].item() - w_frac.item()) <= 1e-5 * abs(w_frac.item()) + 1e-8):
+        return (i, "value_loss", batch, width, g_loss.item(), w_loss.item())
+    # whitening / variance
+    if int(mask.sum()) >= 2:
+        for shift in (True, False):
+            w = o_loss.masked_whiten(values, mask, shift_mean=shift)
+            gw = mrl.masked_whiten(values.to(dev), mask.to(dev), shift_mean=shift)
+            if not (gw.cpu() - w).abs().max().item() < 2e-5 * max(1.0, w.abs().max().item()):
+                return (i, "whiten", batch, width, shift, (gw.cpu() - w).abs().max().item())
+    # group advantages
+    group = rnd.choice([2, 3, 8, 16])
+    nb = group * rnd.randint(1, 6)
+    L = rnd.choice([1, 5, 300])
+    rewards = torch.randn(nb, 1, generator=gen) if rnd.random() < 0.5 else torch.bernoulli(torch.full((nb, 1), 0.5), generator=gen)
+    alens = torch.randint(0, L + 1, (nb,), generator=gen)
+    amask = o_pack.generate_mask(torch.zeros(nb, L), alens)
+    wa, _ = o_adv.compute_group_norm_advantage_return(rewards, amask, torch.zeros(nb, 1), group)
+    ga, _ = mrl.compute_group_norm_advantage_return(rewards.to(dev), amask.to(dev), torch.zeros(nb, 1), group)
+    if not (ga.cpu() - wa).abs().max().item() < 1e-6 * max(1.0, wa.abs().max().item()):
+        return (i, "advantage", nb, group, L, (ga.cpu() - wa).abs().max().item())
+    return None
+
+
+def test_value_side_random_shapes(dev):
+    """Randomised test of kl_token_level_rewards, value_loss (forward, clip fraction, gradient),
+    masked_whiten and compute_group_norm_advantage_return against the oracle: batch 1..257, width
+    2..3000, every KL estimator, empty rows, gaussian and 0/1 rewards."""
+    import random
+    rnd = random.Random(41)
+    failures = [f for f in (_random_value_side_case(i, rnd, dev) for i in range(60)) if f is not None]
+    assert not failures, failures
