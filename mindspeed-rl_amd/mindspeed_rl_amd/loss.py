@@ -312,14 +312,39 @@ class StandardLogProbComputer(LogProbComputer):
 
 
 class MultimodalLogProbComputer(LogProbComputer):
-    """Reference: ``logprob_computer.py:40-70``: logits are cut to the response window first and
-    scored against ``responses``; entropy is taken over the full output."""
+    """Reference: ``logprob_computer.py:40-70``: the logits of the response window are scored against
+    ``responses`` (not ``labels``); entropy is taken over the full output.
+
+    The reference first copies the window out of the ``[B, S, V]`` logits
+    (``truncate_middle_and_pad``) and scores the zero-padded copy, so positions past a sequence's
+    window come out as ``log_softmax(0)[token] = -log V``.  Here the sweep runs over the window's
+    rows where they lie (the responses are scattered to those rows as labels, every other row is
+    skipped), the per-row results are cut to ``[B, L]`` with ``-log V`` as the pad value, and the
+    gradient flows back through the sweep: no ``[B, L, V]`` copy in either direction."""
 
     def compute(self, output, batch, skip_entropy, **kwargs):
         responses = batch["responses"]
+        if output.dim() != 3:
+            raise ValueError("output must have shape (mbs, seq_len, vocab_size)")
         window = response_window(batch["prompt_length"], batch["response_length"])
-        logits = truncate_middle_and_pad(responses, output, window)
-        log_probs = compute_log_probs(logits, responses)
+        n_seq, seq_len, vocab = output.shape
+        out_len = responses.shape[-1]
+        start = window[:, 0].to(torch.int64).clamp(0, seq_len)
+        end = window[:, 1].to(torch.int64).clamp(0, seq_len)
+        count = (end - start).clamp(0, out_len)
+        j = torch.arange(out_len, device=output.device)
+        valid = j[None, :] < count[:, None]
+        rows = (start[:, None] + j[None, :]).clamp(max=seq_len - 1)
+        labels = torch.zeros((n_seq, seq_len), dtype=torch.int64, device=output.device)
+        active = torch.zeros((n_seq, seq_len), dtype=torch.uint8, device=output.device)
+        seq_idx = torch.arange(n_seq, device=output.device)[:, None].expand_as(rows)
+        labels[seq_idx[valid], rows[valid]] = responses.to(torch.int64)[valid]
+        active[seq_idx[valid], rows[valid]] = 1
+        inv_t = float(kwargs.get("inv_temperature", 1.0))
+        row_logp, _, _ = vocab_logprob_entropy(output, labels, inv_temperature=inv_t, want_entropy=False,
+                                               row_active=active)
+        pad = -float(torch.log(torch.tensor(float(vocab), dtype=torch.float32)))
+        log_probs = truncate_prompt_and_pad(responses, row_logp, window, pad_value=pad)
         entropy = torch.zeros_like(log_probs) if skip_entropy else vocab_parallel_entropy(output)
         return log_probs, entropy
 

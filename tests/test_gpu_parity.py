@@ -1916,3 +1916,37 @@ def test_value_side_random_shapes(dev):
     rnd = random.Random(41)
     failures = [f for f in (_random_value_side_case(i, rnd, dev) for i in range(60)) if f is not None]
     assert not failures, failures
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_multimodal_logprob_computer(dev, dtype):
+    """logprob_computer.py:40-70: the window's logits scored against `responses`; here without the
+    [B, L, V] copy of the reference and with a gradient.  Oracle: the reference's own composition
+    (truncate_middle_and_pad -> compute_log_probs; entropy over the full output)."""
+    gen = torch.Generator().manual_seed(77)
+    n_seq, seq_len, vocab, resp_w = 5, 23, 520, 9
+    plen = torch.tensor([[1], [3], [5], [2], [20]], dtype=torch.int32)
+    rlen = torch.tensor([[9], [4], [0], [7], [9]], dtype=torch.int32)       # the last window runs past seq_len
+    out = (torch.randn(n_seq, seq_len, vocab, generator=gen) * 2).to(dtype)
+    responses = torch.randint(0, vocab, (n_seq, resp_w), generator=gen)
+    b = {"responses": responses, "prompt_length": plen, "response_length": rlen}
+    window = o_pack.response_window(plen, rlen)
+    zo = out.float().requires_grad_()
+    want = o_vocab.compute_log_probs(o_pack.truncate_middle_and_pad(responses, zo, window), responses)
+    want_h = o_vocab.vocab_parallel_entropy(out.float())
+    g_out = torch.randn(n_seq, resp_w, generator=gen)
+    (g_o,) = torch.autograd.grad(want, zo, g_out)
+    comp = mrl.MultimodalLogProbComputer()
+    zd = out.to(dev).requires_grad_()
+    lp, ent = comp.compute(zd, _to_dev(b, dev), skip_entropy=False)
+    assert lp.shape == (n_seq, resp_w) and ent.shape == (n_seq, seq_len)
+    assert (lp.cpu() - want.detach()).abs().max().item() < TOL_LOGP
+    assert (ent.detach().cpu() - want_h).abs().max().item() < TOL_LOGP
+    # positions past a window hold exactly what the reference's zero padding gives
+    assert lp[2].detach().cpu().tolist() == want[2].detach().tolist()
+    (g,) = torch.autograd.grad(lp, zd, g_out.to(dev))
+    assert g.dtype == dtype
+    tol = 1e-5 if dtype == torch.float32 else 2 ** -8 * g_o.abs().max().item()
+    assert (g.float().cpu() - g_o).abs().max().item() <= tol
+    lp2, ent2 = comp.compute(out.to(dev), _to_dev(b, dev), skip_entropy=True)
+    assert torch.equal(lp2, lp.detach()) and not ent2.any().item() and ent2.shape == lp2.shape
