@@ -364,6 +364,11 @@ class BaseLossFunc(ABC):
                      non_loss_data=True, **kwargs) -> Tuple[torch.Tensor, Dict]:
         pass
 
+    def _fused(self, output, kwargs):
+        """The one-pass sweep scores rows against ``labels``: it stands in for the standard log-prob
+        strategy only (a caller that installs another ``logprob_computer`` gets the split path)."""
+        return type(self.logprob_computer) is StandardLogProbComputer and _use_fused(output, kwargs)
+
     @staticmethod
     def _get_compute_log_probs_input(output: torch.Tensor, batch: Dict[str, torch.Tensor]):
         if "responses" not in batch:
@@ -434,7 +439,7 @@ class GRPOActorLossFunc(BaseLossFunc):
         if forward_only:
             log_probs, _ = super().compute_log_probs(output=output, batch=batch, **kwargs)
             return log_probs
-        if _use_fused(output, kwargs):
+        if self._fused(output, kwargs):
             loss, out = fused_logprob_policy_loss(
                 output, batch, ref_log_prob=batch.get("ref_log_prob"), clip_low=self.clip_ratio,
                 clip_high=self.clip_ratio, kl_penalty=self.kl_penalty, kl_coef=self.kl_ctrl.value,
@@ -500,7 +505,7 @@ class DAPOActorLossFunc(BaseLossFunc):
             self.clip_ratio_low = self.clip_ratio
             self.clip_ratio_high = self.clip_ratio
         mask = batch["response_mask"] if "response_mask" in batch else None
-        if _use_fused(output, kwargs):
+        if self._fused(output, kwargs):
             loss, out = fused_logprob_policy_loss(
                 output, batch, mask=mask, clip_low=self.clip_ratio_low, clip_high=self.clip_ratio_high,
                 kl_penalty=None, entropy_coeff=self.entropy_coeff, token_level_loss=self.token_level_loss,
@@ -563,7 +568,7 @@ class PPOActorLossFunc(BaseLossFunc):
         common = dict(clip_low=self.clip_ratio, clip_high=self.clip_ratio, kl_penalty=None,
                       entropy_coeff=self.entropy_coeff, token_level_loss=True,
                       loss_scale=_dynamic_scale(batch, forward_only, kwargs))
-        if _use_fused(output, kwargs):
+        if self._fused(output, kwargs):
             loss, out = fused_logprob_policy_loss(output, batch, **common, **_fused_kwargs(kwargs))
         else:
             log_probs, entropy = super().compute_log_probs(output=output, batch=batch,

@@ -1950,3 +1950,36 @@ def test_multimodal_logprob_computer(dev, dtype):
     assert (g.float().cpu() - g_o).abs().max().item() <= tol
     lp2, ent2 = comp.compute(out.to(dev), _to_dev(b, dev), skip_entropy=True)
     assert torch.equal(lp2, lp.detach()) and not ent2.any().item() and ent2.shape == lp2.shape
+
+
+def test_loss_object_with_multimodal_computer(dev):
+    """A loss object whose log-prob strategy was replaced does not take the fused sweep (which scores
+    against `labels`): GRPO with the multimodal strategy equals the oracle's loss on the log-probs that
+    strategy defines."""
+    gen = torch.Generator().manual_seed(5)
+    n_seq, seq_len, vocab, resp_w = 4, 19, 512, 8
+    plen = torch.tensor([[2], [3], [1], [4]], dtype=torch.int32)
+    rlen = torch.tensor([[8], [5], [8], [2]], dtype=torch.int32)
+    out = torch.randn(n_seq, seq_len, vocab, generator=gen) * 2
+    responses = torch.randint(0, vocab, (n_seq, resp_w), generator=gen)
+    rmask = o_pack.generate_mask(responses, rlen)
+    window = o_pack.response_window(plen, rlen)
+    lp0 = o_vocab.compute_log_probs(o_pack.truncate_middle_and_pad(responses, out, window), responses)
+    b = {"responses": responses, "prompt_length": plen, "response_length": rlen, "labels": torch.zeros(n_seq, seq_len, dtype=torch.int64),
+         "advantages": torch.randn(n_seq, resp_w, generator=gen) * rmask,
+         "old_log_prob": (lp0 + torch.randn(n_seq, resp_w, generator=gen) * 0.05) * rmask,
+         "ref_log_prob": (lp0 + torch.randn(n_seq, resp_w, generator=gen) * 0.05) * rmask}
+    zo = out.clone().requires_grad_()
+    lp_o = o_vocab.compute_log_probs(o_pack.truncate_middle_and_pad(responses, zo, window), responses)
+    want = o_loss.grpo_policy_loss(b["old_log_prob"], lp_o, b["ref_log_prob"], b["advantages"], torch.zeros_like(lp_o),
+                                   rmask, 0.2, 0.01, "low_var_kl", 0.0)[0]
+    (g_o,) = torch.autograd.grad(want, zo)
+    f = mrl.GRPOActorLossFunc()
+    f.logprob_computer = mrl.MultimodalLogProbComputer()
+    f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.01), "kl_penalty": "low_var_kl",
+                          "entropy_coeff": 0.0})
+    zd = out.to(dev).requires_grad_()
+    got, _ = f.compute_loss(zd, _to_dev(b, dev))
+    assert got.item() == pytest.approx(want.item(), rel=TOL_LOSS_REL)
+    (g,) = torch.autograd.grad(got, zd)
+    assert (g.cpu() - g_o).abs().max().item() < 1e-6
