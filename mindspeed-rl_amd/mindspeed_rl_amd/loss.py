@@ -261,6 +261,9 @@ def _use_fused(output, kwargs):
     variable MRL_FUSED=0) selects the split forward / backward kernels."""
     if not kwargs.get("fused", os.environ.get("MRL_FUSED", "1") != "0"):
         return False
+    injected = vocab_ops.get_vocab_parallel()
+    if injected is not None and injected is not vocab_ops.vocab_parallel_cross_entropy:
+        return False            # a caller's own cross entropy must be the one that scores the rows
     return torch.is_grad_enabled() and output.requires_grad and fused_supported(output)
 
 
@@ -292,9 +295,16 @@ class StandardLogProbComputer(LogProbComputer):
     def compute(self, output, batch, skip_entropy, **kwargs):
         labels = batch["labels"]
         inv_t = float(kwargs.get("inv_temperature", 1.0))
-        log_probs, entropy, _ = vocab_logprob_entropy(output, labels, inv_temperature=inv_t,
-                                                      want_entropy=not skip_entropy,
-                                                      grad_inplace=bool(kwargs.get("grad_inplace", False)))
+        injected = vocab_ops.get_vocab_parallel()
+        if injected is not None and injected is not vocab_ops.vocab_parallel_cross_entropy:
+            # a caller's own cross entropy (the reference's hook) scores the rows, as in the reference
+            scaled = output if inv_t == 1.0 else output * inv_t
+            log_probs = compute_log_probs(scaled, labels)
+            entropy = None if skip_entropy else vocab_parallel_entropy(scaled)
+        else:
+            log_probs, entropy, _ = vocab_logprob_entropy(output, labels, inv_temperature=inv_t,
+                                                          want_entropy=not skip_entropy,
+                                                          grad_inplace=bool(kwargs.get("grad_inplace", False)))
         if kwargs.get("use_remove_padding", False):
             seqlens = kwargs.get("seqlens_in_batch", None)
             cu = kwargs.get("cu_seqlens_padded", None)

@@ -1983,3 +1983,38 @@ def test_loss_object_with_multimodal_computer(dev):
     assert got.item() == pytest.approx(want.item(), rel=TOL_LOSS_REL)
     (g,) = torch.autograd.grad(got, zd)
     assert (g.cpu() - g_o).abs().max().item() < 1e-6
+
+
+def test_injected_cross_entropy_reaches_the_loss_objects(dev):
+    """set_vocab_parallel (the reference's hook, utils/compute.py:19-26): a caller's own cross entropy
+    scores the rows of the loss objects too - forward-only log-probs and the training loss - and the
+    fused sweep, which has its own scoring built in, steps aside."""
+    gen = torch.Generator().manual_seed(12)
+    logits, b, kw, _, _ = _make_batch(gen, 2, 3, 4, 12, 256, torch.float32, 2.0, 1)
+    bd, kwd = _to_dev(b, dev), _to_dev(kw, dev)
+    calls = []
+
+    def doubled_ce(vocab_parallel_logits, target):
+        calls.append(tuple(vocab_parallel_logits.shape))
+        return 2.0 * mrl.vocab_parallel_cross_entropy(vocab_parallel_logits, target)
+
+    ref_fn = mrl.LossFuncFactory.get_instance("ray_grpo", "reference")
+    plain = ref_fn.compute_loss(logits.to(dev), bd, forward_only=True, **kwd)
+    f = mrl.LossFuncFactory.get_instance("ray_grpo", "actor")
+    f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.01), "kl_penalty": "low_var_kl",
+                          "entropy_coeff": 0.0})
+    mrl.set_vocab_parallel(doubled_ce)
+    try:
+        got = ref_fn.compute_loss(logits.to(dev), bd, forward_only=True, **kwd)
+        assert calls and torch.allclose(got, 2.0 * plain, atol=1e-6)
+        n_calls = len(calls)
+        zd = logits.to(dev).requires_grad_()
+        loss, _ = f.compute_loss(zd, bd, **kwd)                     # would be the fused sweep by default
+        assert len(calls) > n_calls
+        (dz,) = torch.autograd.grad(loss, zd)
+        assert torch.isfinite(dz).all().item() and dz.abs().max().item() > 0
+    finally:
+        mrl.set_vocab_parallel(None)
+    zd = logits.to(dev).requires_grad_()
+    loss_plain, _ = f.compute_loss(zd, bd, **kwd)
+    assert abs(loss_plain.item() - loss.item()) > 1e-6             # the doubled scoring did change the loss
