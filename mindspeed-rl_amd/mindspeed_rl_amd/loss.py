@@ -292,6 +292,38 @@ class StandardLogProbComputer(LogProbComputer):
         window = response_window(batch["prompt_length"], batch["response_length"])
         return truncate_prompt_and_pad(batch["responses"], logprob, window)
 
+    @staticmethod
+    def _rows_in_windows(output, batch, kwargs):
+        """uint8 flag per logits row: 1 where the row lies in a response window, i.e. where the cut
+        below reads it.  Rows outside every window (prompts, padding) are not swept at all: their
+        log-prob, entropy and gradient are never looked at by the reference either."""
+        dev = output.device
+        width = batch["responses"].shape[-1]
+        prompt = batch["prompt_length"].reshape(-1).to(device=dev, dtype=torch.int64)
+        if kwargs.get("use_remove_padding", False):
+            n_rows = output.shape[-2]
+            n = kwargs["seqlens_in_batch"].reshape(-1).to(device=dev, dtype=torch.int64)
+            start = kwargs["cu_seqlens_padded"].reshape(-1).to(device=dev, dtype=torch.int64)[:-1]
+            cut = (prompt - 1) < n                     # postprocess_packed_seqs: start += P-1, len -= P
+            start = torch.where(cut, start + prompt - 1, start)
+            n = torch.where(cut, n - prompt, n)
+        else:
+            n_seq, padded = output.shape[0], output.shape[1]
+            n_rows = n_seq * padded
+            resp = batch["response_length"].reshape(-1).to(device=dev, dtype=torch.int64)
+            lo = (prompt - 1).clamp(0, padded)
+            hi = (prompt + resp - 1).clamp(0, padded)
+            start = lo + torch.arange(n_seq, device=dev, dtype=torch.int64) * padded
+            n = hi - lo
+        n = n.clamp(0, width)
+        start = start.clamp(0, n_rows)
+        end = (start + n).clamp(max=n_rows)
+        edge = torch.zeros(n_rows + 1, dtype=torch.int32, device=dev)
+        one = torch.ones_like(start, dtype=torch.int32)
+        edge.index_add_(0, start, one)
+        edge.index_add_(0, end, -one)
+        return (torch.cumsum(edge[:-1], 0) > 0).to(torch.uint8)
+
     def compute(self, output, batch, skip_entropy, **kwargs):
         labels = batch["labels"]
         inv_t = float(kwargs.get("inv_temperature", 1.0))
@@ -302,8 +334,9 @@ class StandardLogProbComputer(LogProbComputer):
             log_probs = compute_log_probs(scaled, labels)
             entropy = None if skip_entropy else vocab_parallel_entropy(scaled)
         else:
+            active = self._rows_in_windows(output, batch, kwargs).view(labels.shape)
             log_probs, entropy, _ = vocab_logprob_entropy(output, labels, inv_temperature=inv_t,
-                                                          want_entropy=not skip_entropy,
+                                                          want_entropy=not skip_entropy, row_active=active,
                                                           grad_inplace=bool(kwargs.get("grad_inplace", False)))
         if kwargs.get("use_remove_padding", False):
             seqlens = kwargs.get("seqlens_in_batch", None)

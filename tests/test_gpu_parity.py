@@ -2018,3 +2018,66 @@ def test_injected_cross_entropy_reaches_the_loss_objects(dev):
     zd = logits.to(dev).requires_grad_()
     loss_plain, _ = f.compute_loss(zd, bd, **kwd)
     assert abs(loss_plain.item() - loss.item()) > 1e-6             # the doubled scoring did change the loss
+
+
+@pytest.mark.parametrize("layout", ["padded", "packed"])
+def test_standard_computer_sweeps_only_window_rows(dev, layout):
+    """The split path's log-prob strategy skips the logits rows that the response-window cut never
+    reads (prompt rows, the last row, padding): same [B, L] values bit for bit as a sweep over every
+    row, a gradient of exactly zero outside the windows and the same gradient inside, and rows
+    outside the windows may hold anything (NaN here) without reaching the result."""
+    from mindspeed_rl_amd.packing import preprocess_packed_seqs
+    from mindspeed_rl_amd.vocab_ops import vocab_logprob_entropy
+    gen = torch.Generator().manual_seed(123)
+    n_seq, seq_len, vocab, resp_w = 6, 40, 777, 12
+    plen = torch.tensor([[1], [7], [20], [3], [39], [28]], dtype=torch.int64)
+    rlen = torch.tensor([[12], [5], [0], [12], [1], [12]], dtype=torch.int64)
+    ids = torch.randint(0, vocab, (n_seq, seq_len), generator=gen)
+    attn = (torch.arange(seq_len)[None, :] < (plen + rlen)).to(torch.int64)
+    responses = torch.randint(0, vocab, (n_seq, resp_w), generator=gen)
+    b = _to_dev({"responses": responses, "prompt_length": plen, "response_length": rlen,
+                 "labels": torch.roll(ids, -1, 1)}, dev)
+    kw = {}
+    if layout == "packed":
+        packed_ids, _, packed_labels, seqlens, cu = preprocess_packed_seqs(
+            ids.to(dev), torch.roll(ids, -1, 1).to(dev), attn.to(dev), 1)
+        b["labels"] = packed_labels
+        n_rows = packed_ids.shape[1]
+        kw = dict(use_remove_padding=True, seqlens_in_batch=seqlens, cu_seqlens_padded=cu, seq_len=resp_w)
+        out = torch.randn(1, n_rows, vocab, generator=gen) * 2
+    else:
+        out = torch.randn(n_seq, seq_len, vocab, generator=gen) * 2
+    comp = mrl.StandardLogProbComputer()
+    active = comp._rows_in_windows(out.to(dev), b, kw).view(b["labels"].shape).bool()
+    # the flags are the rows the cut reads: cutting a row-index tensor shows them
+    idx = torch.arange(active.numel(), device=dev, dtype=torch.float32).view(active.shape) + 1
+    if layout == "packed":
+        picked = mrl.postprocess_packed_seqs(idx, seqlens, cu, resp_w, prompt_length=b["prompt_length"])
+    else:
+        picked = mrl.truncate_prompt_and_pad(responses.to(dev), idx, mrl.response_window(b["prompt_length"], b["response_length"]))
+    want_active = torch.zeros(active.numel() + 1, dtype=torch.bool, device=dev)
+    want_active[picked.long().flatten()] = True
+    assert torch.equal(active.flatten(), want_active[1:])
+    assert 0 < active.sum().item() < active.numel()
+
+    zd = out.to(dev).requires_grad_()
+    lp, ent = comp.compute(zd, b, skip_entropy=False, **kw)
+    g_out = torch.randn(n_seq, resp_w, generator=gen).to(dev)
+    (g,) = torch.autograd.grad((lp * g_out).sum() + 0.3 * ent.sum(), zd)
+    # every row swept, then the same cut
+    z2 = out.to(dev).requires_grad_()
+    lp_all, ent_all, _ = vocab_logprob_entropy(z2, b["labels"])
+    if layout == "packed":
+        cut = lambda x: mrl.postprocess_packed_seqs(x, seqlens, cu, resp_w, prompt_length=b["prompt_length"])
+    else:
+        cut = lambda x: comp._get_log_probs_remove_prompt_pad(x, b)
+    lp2, ent2 = cut(lp_all), cut(ent_all)
+    (g2,) = torch.autograd.grad((lp2 * g_out).sum() + 0.3 * ent2.sum(), z2)
+    assert torch.equal(lp, lp2) and torch.equal(ent, ent2)
+    assert torch.equal(g, g2)
+    assert not g.view(-1, vocab)[~active.flatten()].any().item()
+    # rows outside the windows are not read
+    poisoned = out.to(dev).clone()
+    poisoned.view(-1, vocab)[~active.flatten()] = float("nan")
+    lp3, ent3 = comp.compute(poisoned, b, skip_entropy=False, **kw)
+    assert torch.equal(lp3, lp.detach()) and torch.equal(ent3, ent.detach())
