@@ -56,6 +56,8 @@ def parse_args():
                     help="non-zero so that the forward computes entropy and the backward its gradient")
     ap.add_argument("--chunk-rows", type=int, default=32768,
                     help="c3 only: logits rows that exist at a time (chunk of the GEMM -> sweep -> GEMMs loop)")
+    ap.add_argument("--no-compact-rows", action="store_true",
+                    help="c3 only: project every row, also those without a live response token")
     ap.add_argument("--path", default="fused", choices=["fused", "split"],
                     help="fused: one sweep computes log-prob, loss and dlogits (1 read + 1 write of [T,V]); "
                          "split: forward sweep, then the backward sweep from the saved logsumexp (2 reads + 1 write)")
@@ -303,7 +305,8 @@ def run_lmhead_train(args):
         loss, out = mrl.fused_lmhead_policy_loss(h, wt, b, packed=True, seqlens=seqlens_d, cu_seqlens=cu_d,
                                                  ref_log_prob=ref_lp, clip_low=0.2, clip_high=0.2,
                                                  kl_penalty="low_var_kl", kl_coef=0.001,
-                                                 entropy_coeff=args.entropy_coeff, chunk_rows=args.chunk_rows)
+                                                 entropy_coeff=args.entropy_coeff, chunk_rows=args.chunk_rows,
+                                                 compact_rows=not args.no_compact_rows)
         stats = out.cpu().tolist()
         dh, dw = torch.autograd.grad(loss, [h, wt])
         return loss, stats, dh, dw

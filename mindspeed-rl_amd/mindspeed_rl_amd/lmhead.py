@@ -14,10 +14,29 @@ from . import _lib, vocab_ops
 kernel_events = None
 
 
-def lmhead_logprob(hidden, weight, labels, inv_temperature=1.0, want_entropy=True):
+def lmhead_logprob(hidden, weight, labels, inv_temperature=1.0, want_entropy=True, row_active=None):
     """``hidden`` ``[..., H]`` bf16, ``weight`` ``[V, H]`` bf16 (``nn.Linear`` layout), ``labels``
     ``[...]`` int32/int64 -> ``(logp, entropy, lse)`` fp32 shaped like ``labels`` (entropy is zeros
-    if not wanted).  No autograd: use it under ``torch.no_grad()`` for old / reference log-probs."""
+    if not wanted).  No autograd: use it under ``torch.no_grad()`` for old / reference log-probs.
+    ``row_active`` (bool / integer, shaped like ``labels``): only rows with a non-zero flag are
+    projected and scored, the others return 0 in all three outputs (one host synchronisation reads
+    the number of active rows)."""
+    if row_active is not None:
+        if tuple(row_active.shape) != tuple(labels.shape):
+            raise ValueError("row_active must have the shape of labels")
+        dev = _lib.require_device(hidden, weight, labels, row_active)
+        live = torch.nonzero(row_active.reshape(-1) != 0).flatten()
+        n_all = labels.numel()
+        if live.numel() == 0:
+            return tuple(torch.zeros(labels.shape, dtype=torch.float32, device=dev) for _ in range(3))
+        res = lmhead_logprob(hidden.reshape(-1, hidden.shape[-1]).index_select(0, live), weight,
+                             labels.reshape(-1).index_select(0, live), inv_temperature, want_entropy)
+        outs = []
+        for part in res:
+            full = torch.zeros(n_all, dtype=torch.float32, device=dev)
+            full.index_copy_(0, live, part)
+            outs.append(full.view(labels.shape))
+        return tuple(outs)
     dev = _lib.require_device(hidden, weight, labels)
     if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
         raise TypeError("hidden and weight must be bfloat16")
@@ -120,6 +139,23 @@ class _FusedLmHeadLoss(torch.autograd.Function):
                   _lib.ptr(mask_t), mdt, cfg["seq_mean"], _lib.ptr(row_start), _lib.ptr(row_count),
                   _lib.ptr(seq_msum), _lib.ptr(row_ops), stream)
         grad_scale = cfg["loss_scale"] * cfg["expected_upstream"]
+        # Rows whose mask is zero (prompts, padding, masked tokens) add nothing to the loss, to dWeight or
+        # to their own dHidden: when they are more than a twentieth of the rows, the live rows are gathered
+        # and only they go through the GEMMs.  The row count sizes the GEMMs, so it is read back (one
+        # host synchronisation per call; compact_rows=False avoids it).
+        live = None
+        if cfg["compact_rows"] and n_rows > 0:
+            live = torch.nonzero(row_ops.view(n_rows, 8)[:, 3] != 0).flatten()
+            if live.numel() * 20 > n_rows * 19:
+                live = None
+        all_rows, h_all = n_rows, h2d
+        if live is not None:
+            n_rows = live.numel()
+            h2d = h_all.index_select(0, live)
+            lab = lab.index_select(0, live)
+            row_ops = row_ops.view(all_rows, 8).index_select(0, live).reshape(-1)
+            terms_all, row_terms = row_terms, torch.empty(max(n_rows, 1) * 8, dtype=torch.float32, device=dev)
+            ent = torch.empty(max(n_rows, 1), dtype=torch.float32, device=dev) if want_ent else None
         chunk = max(1, min(int(cfg["chunk_rows"]), n_rows))
         logits = torch.empty((chunk, vocab), dtype=h2d.dtype, device=dev)
         d_hidden = torch.empty_like(h2d)
@@ -148,6 +184,12 @@ class _FusedLmHeadLoss(torch.autograd.Function):
                 # the hidden chunk goes in as the transpose of an [H, rows] copy: the library picks a faster
                 # kernel for that operand layout (7.5 against 8.7 ms per chunk), the copy is 59 MB
                 _accumulate_fp32(d_weight32, z.t(), h2d[c0:c1].t().contiguous().t())
+        if live is not None:
+            compact_dh, compact_terms = d_hidden, row_terms
+            d_hidden = torch.zeros_like(h_all)
+            d_hidden.index_copy_(0, live, compact_dh)
+            row_terms = terms_all.zero_()
+            row_terms.view(all_rows, 8).index_copy_(0, live, compact_terms[:n_rows * 8].view(n_rows, 8))
         _lib.call("mrl_fused_loss_reduce", _lib.ptr(row_terms), _lib.ptr(row_start), _lib.ptr(row_count), n_seq, width,
                   _lib.ptr(old), _lib.ptr(ref), _lib.ptr(adv), _lib.ptr(mask_t), mdt, _lib.ptr(resp), rdt,
                   cfg["clip_lo"], cfg["clip_hi"], cfg["kl_penalty"], cfg["kl_coef"], cfg["entropy_coeff"],
@@ -173,14 +215,16 @@ class _FusedLmHeadLoss(torch.autograd.Function):
 def fused_lmhead_policy_loss(hidden, weight, batch, *, packed, seqlens=None, cu_seqlens=None, mask=None,
                              ref_log_prob=None, clip_low, clip_high, kl_penalty=None, kl_coef=0.0, entropy_coeff=0.0,
                              token_level_loss=True, loss_scale=1.0, inv_temperature=1.0, expected_upstream=1.0,
-                             chunk_rows=32768, fp32_dw_gemm=False):
+                             chunk_rows=32768, fp32_dw_gemm=False, compact_rows=True):
     """Policy loss straight from the hidden states: ``hidden`` is packed ``[1, T, H]`` (or padded
     ``[B, S, H]``) bf16, ``weight`` the ``[V, H]`` bf16 lm_head weight; ``batch`` as for
     :func:`mindspeed_rl_amd.fused_logprob_policy_loss` (``labels, responses, response_length,
     prompt_length, advantages``, optional ``old_log_prob``).  Returns ``(loss, out)``; ``backward()``
     yields dHidden and dWeight.  Full ``[T, V]`` logits are never materialised: at most
     ``chunk_rows x V`` exist at a time.  ``hidden_dim`` and ``V`` must make 16-byte rows and
-    ``V <= mrl_fused_max_vocab``."""
+    ``V <= mrl_fused_max_vocab``.  With ``compact_rows`` (default) rows without a live response token
+    skip the GEMMs when they are more than 5 % of all rows; finding them costs one host
+    synchronisation per call."""
     if kl_penalty is None:
         kl_code = _lib.KL_NONE
     elif kl_penalty in _lib.KL_BY_NAME:
@@ -193,5 +237,6 @@ def fused_lmhead_policy_loss(hidden, weight, batch, *, packed, seqlens=None, cu_
                clip_lo=float(1.0 - clip_low), clip_hi=float(1.0 + clip_high), kl_penalty=kl_code,
                kl_coef=float(kl_coef), entropy_coeff=float(entropy_coeff), seq_mean=0 if token_level_loss else 1,
                loss_scale=float(loss_scale), inv_temperature=float(inv_temperature),
-               expected_upstream=float(expected_upstream), chunk_rows=int(chunk_rows), fp32_dw_gemm=bool(fp32_dw_gemm))
+               expected_upstream=float(expected_upstream), chunk_rows=int(chunk_rows), fp32_dw_gemm=bool(fp32_dw_gemm),
+               compact_rows=bool(compact_rows))
     return _FusedLmHeadLoss.apply(hidden, weight, batch["labels"], batch, cfg)

@@ -2081,3 +2081,64 @@ def test_standard_computer_sweeps_only_window_rows(dev, layout):
     poisoned.view(-1, vocab)[~active.flatten()] = float("nan")
     lp3, ent3 = comp.compute(poisoned, b, skip_entropy=False, **kw)
     assert torch.equal(lp3, lp.detach()) and torch.equal(ent3, ent.detach())
+
+
+def test_fused_lmhead_policy_loss_skips_rows_without_response(dev):
+    """With long prompts most rows carry no live response token: the chunked lm_head step gathers the
+    live rows and runs its GEMMs on them alone.  Same loss, statistics, dHidden and dWeight as with
+    every row projected (up to how a GEMM rounds when its row count changes), and dHidden exactly
+    zero on the skipped rows.  A mask that switches off response tokens drops their rows as well."""
+    gen = torch.Generator().manual_seed(31)
+    vocab, hdim = 2048, 128
+    _, b, kw, _, _ = _make_batch(gen, 2, 4, 3, 12, vocab, torch.bfloat16, 1.0, 2, prompt_hi=30)
+    total = b["labels"].shape[1]
+    n_seq, resp_w = b["advantages"].shape
+    h = torch.randn(1, total, hdim, generator=gen).to(torch.bfloat16)
+    w = (torch.randn(vocab, hdim, generator=gen) * (3.0 / hdim ** 0.5)).to(torch.bfloat16)
+    rmask = o_pack.generate_mask(torch.zeros(n_seq, resp_w), b["response_length"])
+    mask = rmask * (torch.rand(n_seq, resp_w, generator=gen) > 0.3)
+    bd, kwd = _to_dev(b, dev), _to_dev(kw, dev)
+    res = {}
+    for compact in (True, False):
+        hd, wd = h.to(dev).requires_grad_(), w.to(dev).requires_grad_()
+        loss, out = mrl.fused_lmhead_policy_loss(hd, wd, bd, packed=True, seqlens=kwd["seqlens_in_batch"],
+                                                 cu_seqlens=kwd["cu_seqlens_padded"], ref_log_prob=bd["ref_log_prob"],
+                                                 mask=mask.to(dev), clip_low=0.2, clip_high=0.2, kl_penalty="low_var_kl",
+                                                 kl_coef=0.01, entropy_coeff=0.002, chunk_rows=16, compact_rows=compact)
+        dh, dw = torch.autograd.grad(loss, [hd, wd])
+        res[compact] = (loss.item(), out.cpu(), dh.float().cpu()[0], dw.float().cpu())
+    (l1, o1, dh1, dw1), (l0, o0, dh0, dw0) = res[True], res[False]
+    assert l1 == pytest.approx(l0, rel=1e-5, abs=1e-8)
+    assert torch.allclose(o1, o0, rtol=1e-5, atol=1e-7)
+    assert (dh1 - dh0).abs().max().item() <= 2 ** -7 * dh0.abs().max().item()
+    assert (dw1 - dw0).abs().max().item() <= 2 ** -7 * dw0.abs().max().item()
+    # rows of the packed stream that hold a live token, from the oracle's own window cut
+    idx = torch.arange(1, total + 1, dtype=torch.float32).view(1, total)
+    picked = o_pack.postprocess_packed_seqs(idx, kw["seqlens_in_batch"], kw["cu_seqlens_padded"], resp_w,
+                                            prompt_length=b["prompt_length"])
+    live = torch.zeros(total + 1, dtype=torch.bool)
+    live[(picked * mask).long().flatten()] = True
+    live = live[1:]
+    assert live.sum().item() * 20 <= total * 19            # the case does take the compacted path
+    assert not dh1[~live].any().item()
+    assert dh1[live].abs().sum(1).min().item() > 0
+
+
+def test_lmhead_logprob_row_active(dev):
+    """Only flagged rows are projected and scored; the others return zeros."""
+    gen = torch.Generator().manual_seed(8)
+    tokens, vocab, hdim = 301, 1000, 128
+    h = torch.randn(tokens, hdim, generator=gen).to(torch.bfloat16).to(dev)
+    w = (torch.randn(vocab, hdim, generator=gen) * (2.0 / hdim ** 0.5)).to(torch.bfloat16).to(dev)
+    y = torch.randint(0, vocab, (tokens,), generator=gen).to(dev)
+    act = (torch.rand(tokens, generator=gen) > 0.6).to(dev)
+    full = mrl.lmhead_logprob(h, w, y)
+    part = mrl.lmhead_logprob(h.view(1, tokens, hdim), w, y.view(1, tokens), row_active=act.view(1, tokens))
+    for a, p in zip(full, part):
+        assert p.shape == (1, tokens)
+        assert not p.view(-1)[~act].any().item()
+        assert (p.view(-1)[act] - a[act]).abs().max().item() < 2e-5
+    none = mrl.lmhead_logprob(h, w, y, row_active=torch.zeros(tokens, dtype=torch.uint8, device=dev))
+    assert all(not t.any().item() and t.shape == (tokens,) for t in none)
+    with pytest.raises(ValueError):
+        mrl.lmhead_logprob(h, w, y, row_active=act[:-1])
