@@ -2142,3 +2142,45 @@ def test_lmhead_logprob_row_active(dev):
     assert all(not t.any().item() and t.shape == (tokens,) for t in none)
     with pytest.raises(ValueError):
         mrl.lmhead_logprob(h, w, y, row_active=act[:-1])
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_loss_on_logits_that_are_views_or_products(dev, fused):
+    """The logits a model hands over are the result of a projection, possibly a transposed or sliced
+    view of it: loss and the gradients that reach hidden states and weight equal the oracle's, with
+    and without the in-place gradient."""
+    gen = torch.Generator().manual_seed(12)
+    n_seq, seq_len, vocab, hdim = 4, 24, 1024, 64
+    plen = torch.tensor([[3], [1], [5], [2]])
+    rlen = torch.tensor([[10], [20], [7], [15]])
+    resp_w = int(rlen.max())
+    ids = torch.randint(0, vocab, (n_seq, seq_len), generator=gen)
+    rmask = o_pack.generate_mask(torch.zeros(n_seq, resp_w), rlen)
+    b = {"labels": torch.roll(ids, -1, 1), "responses": torch.zeros(n_seq, resp_w, dtype=torch.int64),
+         "response_length": rlen, "prompt_length": plen,
+         "advantages": torch.randn(n_seq, resp_w, generator=gen) * rmask,
+         "old_log_prob": -torch.rand(n_seq, resp_w, generator=gen) * rmask * 3,
+         "ref_log_prob": -torch.rand(n_seq, resp_w, generator=gen) * rmask * 3}
+    meta = dict(clip_ratio=0.2, kl_coef=0.01, kl_penalty="low_var_kl", entropy_coeff=0.001)
+    h = torch.randn(n_seq, seq_len, hdim, generator=gen)
+    w = torch.randn(vocab, hdim, generator=gen) * 0.3
+    projections = {
+        "product": lambda hh, ww: hh @ ww.t(),
+        "transposed view": lambda hh, ww: (hh.transpose(0, 1).contiguous() @ ww.t()).transpose(0, 1),
+        "slice of a padded vocabulary": lambda hh, ww: (hh @ torch.cat([ww, torch.zeros(8, hdim, device=ww.device)]).t())[..., :vocab],
+    }
+    bd = _to_dev(b, dev)
+    for name, project in projections.items():
+        ho, wo = h.clone().requires_grad_(), w.clone().requires_grad_()
+        want, _ = o_loss.grpo_compute_loss(project(ho, wo).contiguous(), b, meta)
+        gh_o, gw_o = torch.autograd.grad(want, [ho, wo])
+        for inplace in (False, True):
+            f = mrl.GRPOActorLossFunc()
+            f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.01), "kl_penalty": "low_var_kl",
+                                  "entropy_coeff": 0.001})
+            hd, wd = h.to(dev).requires_grad_(), w.to(dev).requires_grad_()
+            got, _ = f.compute_loss(project(hd, wd), bd, fused=fused, grad_inplace=inplace)
+            gh, gw = torch.autograd.grad(got, [hd, wd])
+            assert got.item() == pytest.approx(want.item(), rel=TOL_LOSS_REL, abs=1e-7), name
+            assert (gh.cpu() - gh_o).abs().max().item() < 1e-6, name
+            assert (gw.cpu() - gw_o).abs().max().item() < 1e-6, name
