@@ -2184,3 +2184,47 @@ def test_loss_on_logits_that_are_views_or_products(dev, fused):
             assert got.item() == pytest.approx(want.item(), rel=TOL_LOSS_REL, abs=1e-7), name
             assert (gh.cpu() - gh_o).abs().max().item() < 1e-6, name
             assert (gw.cpu() - gw_o).abs().max().item() < 1e-6, name
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_one_loss_object_over_interleaved_micro_batches(dev, fused):
+    """A pipeline schedule runs the forward of several micro-batches of different shapes through ONE
+    loss object and their backwards later, in another order: every loss and gradient equals the
+    oracle's for its own micro-batch (nothing is shared between calls)."""
+    def micro_batch(seed, n_seq, seq_len, vocab):
+        g = torch.Generator().manual_seed(seed)
+        plen = torch.randint(1, 5, (n_seq, 1), generator=g)
+        rlen = torch.randint(1, seq_len - 5, (n_seq, 1), generator=g)
+        resp_w = int(rlen.max())
+        ids = torch.randint(0, vocab, (n_seq, seq_len), generator=g)
+        rmask = o_pack.generate_mask(torch.zeros(n_seq, resp_w), rlen)
+        b = {"labels": torch.roll(ids, -1, 1), "responses": torch.zeros(n_seq, resp_w, dtype=torch.int64),
+             "response_length": rlen, "prompt_length": plen,
+             "advantages": torch.randn(n_seq, resp_w, generator=g) * rmask,
+             "old_log_prob": -torch.rand(n_seq, resp_w, generator=g) * rmask * 3,
+             "ref_log_prob": -torch.rand(n_seq, resp_w, generator=g) * rmask * 3}
+        return torch.randn(n_seq, seq_len, vocab, generator=g) * 2, b
+
+    meta = dict(clip_ratio=0.2, kl_coef=0.01, kl_penalty="low_var_kl", entropy_coeff=0.001)
+    items = [micro_batch(1, 4, 30, 512), micro_batch(2, 7, 19, 1032), micro_batch(3, 2, 40, 256)]
+    want = []
+    for z, b in items:
+        zo = z.clone().requires_grad_()
+        loss_o, _ = o_loss.grpo_compute_loss(zo, b, meta)
+        (g_o,) = torch.autograd.grad(loss_o * 0.25, zo)
+        want.append((loss_o.item(), g_o))
+    for extra in ({}, {"grad_inplace": True}, {"expected_grad_scale": 0.25}):
+        f = mrl.GRPOActorLossFunc()
+        f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.01), "kl_penalty": "low_var_kl",
+                              "entropy_coeff": 0.001})
+        leaves, losses = [], []
+        for z, b in items:
+            zd = z.to(dev).requires_grad_()
+            loss, _ = f.compute_loss(zd * 1.0, _to_dev(b, dev), fused=fused, **extra)     # a non-leaf: in-place is legal
+            leaves.append(zd)
+            losses.append(loss)
+        for i in (1, 0, 2):
+            (losses[i] * 0.25).backward()
+        for i in range(3):
+            assert losses[i].item() == pytest.approx(want[i][0], rel=TOL_LOSS_REL, abs=1e-7)
+            assert (leaves[i].grad.cpu() - want[i][1]).abs().max().item() < 1e-6
