@@ -23,8 +23,8 @@ from .wire import (pack_experience_columns, pack_padded_columns, pad_multiple, p
                    remove_padding_and_split_to_list, remove_padding_tensor_dict_to_dict, truncate_rows,
                    unpack_pad_experience)
 from .vocab_ops import (compute_kl_penalty, compute_log_probs, get_parallel_state, get_vocab_parallel,
-                        set_parallel_state, set_vocab_parallel, vocab_logprob_entropy, vocab_parallel_cross_entropy,
-                        vocab_parallel_entropy)
+                        merge_vocab_shard_stats, set_parallel_state, set_vocab_parallel, vocab_logprob_entropy,
+                        vocab_parallel_cross_entropy, vocab_parallel_entropy, vocab_shard_backward, vocab_shard_stats)
 
 __version__ = "0.1.0"
 

@@ -129,6 +129,70 @@ def vocab_logprob_entropy(logits, labels, inv_temperature=1.0, want_entropy=True
     return _VocabLogprobEntropy.apply(logits, labels, inv_temperature, want_entropy, row_active, grad_inplace)
 
 
+# ------------------------------------------------------------------- one rank's share of a sharded vocabulary
+def vocab_shard_stats(logits_shard, labels, vocab_start, inv_temperature=1.0, row_active=None):
+    """One tensor-parallel rank's share of the forward sweep: ``logits_shard`` ``[..., V/tp]`` holds
+    the vocabulary entries ``[vocab_start, vocab_start + V/tp)`` of every row, ``labels`` the global
+    token ids.  Returns fp32 ``[..., 3]`` = (logsumexp over the shard, label logit if the label lies
+    in the shard else 0, softmax-weighted mean logit of the shard): 12 bytes per token, which is all
+    the ranks have to exchange (Megatron's ``vocab_parallel_cross_entropy`` and the reference's
+    ``_VocabParallelEntropy.forward``, ``utils/compute.py:56-73``, all-reduce the row maximum, the
+    predicted logit, the exponential sum and the weighted sum one after the other).  No autograd."""
+    width = logits_shard.shape[-1]
+    local = labels.to(torch.int64) - int(vocab_start)
+    own = (local >= 0) & (local < width)
+    with torch.no_grad():
+        logp, ent, lse = vocab_logprob_entropy(logits_shard.detach(), local, inv_temperature=inv_temperature,
+                                               want_entropy=True, row_active=row_active)
+    label_logit = torch.where(own, logp + lse, torch.zeros_like(logp))
+    if row_active is not None:
+        lse = torch.where(row_active.reshape(lse.shape) != 0, lse, torch.full_like(lse, float("-inf")))
+    return torch.stack([lse, label_logit, lse - ent], dim=-1)
+
+
+def merge_vocab_shard_stats(stats):
+    """``stats`` ``[tp, ..., 3]``: every rank's :func:`vocab_shard_stats` (what an all-gather
+    delivers).  Returns ``(logp, entropy, lse)`` of the full vocabulary, fp32.  Rows that no rank
+    scored (``row_active`` 0 everywhere) return 0."""
+    lse_s, label_s, mean_s = stats.unbind(-1)
+    lse = torch.logsumexp(lse_s, dim=0)
+    dead = torch.isinf(lse) & (lse < 0)
+    lse = torch.where(dead, torch.zeros_like(lse), lse)
+    share = torch.exp(lse_s - lse.unsqueeze(0))                    # each shard's probability mass
+    share = torch.where(dead.unsqueeze(0), torch.zeros_like(share), share)
+    mean_logit = (share * torch.where(share > 0, mean_s, torch.zeros_like(mean_s))).sum(0)
+    logp = torch.where(dead, torch.zeros_like(lse), label_s.sum(0) - lse)
+    return logp, lse - mean_logit, lse
+
+
+def vocab_shard_backward(logits_shard, labels, vocab_start, lse, entropy, g_logp, g_entropy=None, inv_temperature=1.0,
+                         grad_inplace=False):
+    """One rank's share of the backward sweep: dlogits of the shard from the MERGED ``lse`` and
+    ``entropy`` (Megatron's cross-entropy backward and ``_VocabParallelEntropy.backward``,
+    ``utils/compute.py:76-85``, on the rank's vocabulary range).  One read of the shard, one write."""
+    dev = _lib.require_device(logits_shard, labels, lse, entropy, g_logp, g_entropy)
+    width = logits_shard.shape[-1]
+    flat = logits_shard.detach().reshape(-1, width)
+    if flat.stride(-1) != 1 or (flat.shape[0] > 1 and flat.stride(0) < width):
+        flat = flat.contiguous()
+    n_rows = flat.shape[0]
+    row_stride = flat.stride(0) if n_rows > 1 else width
+    local = (labels.to(torch.int64) - int(vocab_start)).reshape(-1).contiguous()
+
+    def f32(t):
+        return None if t is None else t.reshape(-1).to(torch.float32).contiguous()
+
+    lse_f, ent_f, g_lp, g_h = f32(lse), f32(entropy), f32(g_logp), f32(g_entropy)
+    if grad_inplace:
+        dlogits, d_stride = flat, row_stride
+    else:
+        dlogits, d_stride = torch.empty((n_rows, width), dtype=flat.dtype, device=dev), width
+    _timed_call("mrl_vocab_logprob_bwd", n_rows, dev, _lib.ptr(flat), _lib.dtype_code(flat), n_rows, width, row_stride,
+                _lib.ptr(local), _lib.dtype_code(local), float(inv_temperature), _lib.ptr(lse_f), _lib.ptr(ent_f),
+                _lib.ptr(g_lp), _lib.ptr(g_h), _lib.ptr(dlogits), _lib.dtype_code(dlogits), d_stride, _lib.stream(dev))
+    return dlogits.view(logits_shard.shape)
+
+
 def vocab_parallel_cross_entropy(vocab_parallel_logits, target, label_smoothing=0.0):
     """Drop-in for Megatron's ``vocab_parallel_cross_entropy`` at tp = 1 (the function the
     reference injects through ``set_vocab_parallel``, ``workers/base_worker.py:279-284``):

@@ -2228,3 +2228,47 @@ def test_one_loss_object_over_interleaved_micro_batches(dev, fused):
         for i in range(3):
             assert losses[i].item() == pytest.approx(want[i][0], rel=TOL_LOSS_REL, abs=1e-7)
             assert (leaves[i].grad.cpu() - want[i][1]).abs().max().item() < 1e-6
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("bounds", [(0, 2048, 4096), (0, 1024, 2048, 3072, 4096), (0, 520, 528, 3000, 4096)])
+def test_vocabulary_shards_merge_to_the_full_sweep(dev, dtype, bounds):
+    """One tensor-parallel rank's share of the path, run for every rank in turn on one GPU: the
+    per-shard statistics (12 bytes per token) merge to the oracle's full-vocabulary log-prob and
+    entropy, and the shards' gradients, computed from the merged statistics, are the slices of the
+    oracle's gradient.  Labels outside the vocabulary, a skipped row and temperature included."""
+    gen = torch.Generator().manual_seed(len(bounds))
+    rows, vocab, inv_t = 37, bounds[-1], 1.0 / 0.8
+    z = _logits(gen, rows, vocab, dtype)
+    y = torch.randint(0, vocab, (rows,), generator=gen)
+    y[3], y[4] = bounds[1] - 1, bounds[1]                  # either side of a shard boundary
+    active = torch.ones(rows, dtype=torch.uint8)
+    active[5] = 0
+    zo = (z.float() * inv_t).requires_grad_()
+    lp_o = o_vocab.compute_log_probs(zo, y)
+    h_o = o_vocab.vocab_parallel_entropy(zo)
+    g_lp, g_h = torch.randn(rows, generator=gen), torch.randn(rows, generator=gen) * 0.1
+    g_lp[5] = g_h[5] = 0.0
+    (dz_o,) = torch.autograd.grad((lp_o * g_lp).sum() + (h_o * g_h).sum(), zo)
+    dz_o = dz_o * inv_t
+    zd, yd = z.to(dev), y.to(dev)
+    shards = [zd[:, a:b] for a, b in zip(bounds[:-1], bounds[1:])]          # strided views, as a rank's slice
+    stats = torch.stack([mrl.vocab_shard_stats(s, yd, a, inv_temperature=inv_t, row_active=active.to(dev))
+                         for s, a in zip(shards, bounds[:-1])])
+    assert stats.shape == (len(shards), rows, 3)
+    lp, ent, lse = mrl.merge_vocab_shard_stats(stats)
+    live = active.bool()
+    assert (lp.cpu() - lp_o.detach())[live].abs().max().item() < TOL_LOGP
+    assert (ent.cpu() - h_o.detach())[live].abs().max().item() < TOL_LOGP
+    assert lp[5].item() == 0 and ent[5].item() == 0 and lse[5].item() == 0
+    full_lp, full_ent, full_lse = mrl.vocab_logprob_entropy(zd, yd, inv_temperature=inv_t)
+    assert (lp - full_lp)[live.to(dev)].abs().max().item() < 2e-5
+    assert (ent - full_ent)[live.to(dev)].abs().max().item() < 2e-5
+    dz = torch.cat([mrl.vocab_shard_backward(s, yd, a, lse, ent, g_lp.to(dev), g_h.to(dev), inv_temperature=inv_t)
+                    for s, a in zip(shards, bounds[:-1])], dim=1)
+    assert dz.dtype == dtype and dz.shape == (rows, vocab)
+    tol = 1e-5 if dtype == torch.float32 else 2 ** -8 * dz_o.abs().max().item()
+    assert (dz.float().cpu() - dz_o).abs().max().item() <= tol
+    assert not dz[5].any().item()
+    # a label outside every shard: the oracle (Megatron's target mask) scores the row maximum there,
+    # a sharded run scores 0 - documented difference, no rank owns such a label
