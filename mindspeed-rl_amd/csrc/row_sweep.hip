@@ -687,10 +687,9 @@ int fused_by_nv(int nv, const mrl::FusedArgs& a) { MRL_NV_SWITCH(launch_fused, D
 
 namespace mrl {
 
-template <int DT>
-static int launch_bwd_chunk(const BwdArgs& a) {
+template <int DT, int kThreads>
+static int launch_bwd_chunk_n(const BwdArgs& a) {
     using T = typename Elem<DT>::T;
-    constexpr int kThreads = MRL_BWD_CHUNK_THREADS;
     const int64_t n_vec = a.vocab / Elem<DT>::kVec;
     const int64_t gy = a.n_rows < kChunkRowsY ? a.n_rows : kChunkRowsY;
     const int64_t gz = (a.n_rows + kChunkRowsY - 1) / kChunkRowsY;
@@ -703,6 +702,18 @@ static int launch_bwd_chunk(const BwdArgs& a) {
     else MRL_BWDC_LAUNCH(false);
 #undef MRL_BWDC_LAUNCH
     return check_launch("mrl_vocab_logprob_bwd");
+}
+
+// Workgroups of half the size when that leaves at least 3 % fewer lanes idle in a row's last
+// chunk (a 38 KiB row is 9.3 chunks of 256 vectors: 2.30 ms against 2.19 ms for 171 174 such rows).
+template <int DT>
+static int launch_bwd_chunk(const BwdArgs& a) {
+    constexpr int kFull = MRL_BWD_CHUNK_THREADS, kHalf = MRL_BWD_CHUNK_THREADS / 2;
+    const int64_t n_vec = a.vocab / Elem<DT>::kVec;
+    const int64_t idle_full = (n_vec + kFull - 1) / kFull * kFull - n_vec;
+    const int64_t idle_half = (n_vec + kHalf - 1) / kHalf * kHalf - n_vec;
+    if ((idle_full - idle_half) * 100 >= 3 * n_vec) return launch_bwd_chunk_n<DT, kHalf>(a);
+    return launch_bwd_chunk_n<DT, kFull>(a);
 }
 
 int launch_bwd_chunks(const BwdArgs& a) {
