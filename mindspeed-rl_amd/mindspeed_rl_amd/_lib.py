@@ -139,6 +139,10 @@ def require_device(*tensors):
             dev = t.device
         elif t.device != dev:
             raise RuntimeError("tensors on different devices: %s and %s" % (dev, t.device))
+    if dev is not None and dev.index is not None and dev.index != torch.cuda.current_device():
+        # kernels are launched on the current device's context: one process drives one GPU here
+        raise RuntimeError("tensors live on %s but the current device is cuda:%d (call torch.cuda.set_device first)"
+                           % (dev, torch.cuda.current_device()))
     return dev
 
 
