@@ -495,6 +495,16 @@ def main():
         e.record()
         torch.cuda.synchronize()
         ceilings[name] = passes * nbytes * 5 / (s.elapsed_time(e) * 1e-3) / 1e9
+    # the runtime's own device-to-device copy of the same bytes (Tensor.copy_ -> hipMemcpyAsync)
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(2):
+        dst.copy_(src)
+    s.record()
+    for _ in range(5):
+        dst.copy_(src)
+    e.record()
+    torch.cuda.synchronize()
+    ceilings["runtime_d2d_copy_GBps"] = 2 * nbytes * 5 / (s.elapsed_time(e) * 1e-3) / 1e9
     del src, dst
     result["measured_ceiling"] = ceilings
     # a read+write stream of R read bytes and W written bytes cannot beat R/read + W/write on this box
