@@ -419,9 +419,10 @@ def main():
     live_rows = tokens                                    # rows with a non-zero mask / incoming gradient
     dead_rows = total - live_rows
     row_bytes = vocab * ebytes
-    # algorithmic HBM bytes per launch: reads of the rows that are needed + writes of every dlogits row
+    # algorithmic HBM bytes per launch: reads of the rows that are needed (the split path's forward is
+    # handed the rows inside the response windows, like the fused sweep) + writes of every dlogits row
     kernel_bytes = {
-        "mrl_vocab_logprob_fwd": total * row_bytes,
+        "mrl_vocab_logprob_fwd": live_rows * row_bytes,
         "mrl_vocab_logprob_bwd": live_rows * 2 * row_bytes + dead_rows * row_bytes,
         "mrl_fused_logprob_loss": live_rows * 2 * row_bytes + dead_rows * row_bytes,
     }
