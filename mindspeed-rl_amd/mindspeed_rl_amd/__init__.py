@@ -14,7 +14,7 @@ from .loss import (BaseLossFunc, DAPOActorLossFunc, GRPOActorLossFunc, LossFuncF
                    policy_loss)
 from .packing import (generate_mask, pack_index, postprocess_packed_seqs, preprocess_packed_seqs, response_window,
                       truncate_middle_and_pad, truncate_prompt_and_pad)
-from .seqlen_balancing import (get_reverse_idx, get_seqlen_balanced_partitions, heapq_partition,
+from .seqlen_balancing import (balanced_bin_packing, get_reverse_idx, get_seqlen_balanced_partitions, heapq_partition,
                                heapq_partition_with_max, karmarkar_karp, rearrange_micro_batches,
                                split_batches_with_dynamic_bsz)
 from .value_path import (AdaptiveKLController, CriticLossFunc, compute_gae_advantage_return, kl_token_level_rewards,

@@ -6,8 +6,10 @@ Host-side mirror of ``mindspeed_rl/utils/seqlen_balancing.py`` (``karmarkar_karp
 ``BaseTrainingEngine._split_batches_with_dynamic_bsz`` (``models/base/base_training_engine.py:
 160-187``), with the reference's names, arguments, results (including its tie-breaking, so that
 the same lengths give the same micro-batches) and errors.  This is pure host logic on a few
-hundred integers; it decides the row count T of every sweep.  Text-only, one data-parallel rank:
-the multimodal bin-packing branch and the MAX all-reduce of the bin count are not built.
+hundred integers; it decides the row count T of every sweep.  One data-parallel rank: the MAX
+all-reduce of the bin count is not built.  The capacity-bound bin packing the reference uses for
+multimodal batches (``balanced_bin_packing``, ``:191-307``) is selected with ``multimodal=True``
+(the reference reads a global switch).
 """
 import heapq
 from typing import Dict, List, Tuple
@@ -143,11 +145,65 @@ def heapq_partition_with_max(seqlen_list: List[int], k_partitions: int, max_toke
     return closed + [g[3] for g in open_groups]
 
 
+def balanced_bin_packing(seqlen_list: List[int], max_capacity: int):
+    """Reference: ``utils/seqlen_balancing.py:191-307``.  Best fit decreasing under a hard capacity
+    (longest item first into the fullest bin that still takes it, a new bin if none does), then at
+    most three single-item moves from a fuller to an emptier bin that narrow their gap.  Returns
+    the bins as index lists, in the order the balancing pass leaves them (ascending load at its
+    last sort).  ``ValueError`` for an item longer than the capacity."""
+    if not seqlen_list:
+        return []
+    loads: List[int] = []
+    members: List[List[Tuple[int, int]]] = []
+    for length, idx in _longest_first(seqlen_list):
+        if length > max_capacity:
+            raise ValueError(f"Item with seqlen {length} exceeds max_capacity {max_capacity}")
+        room = [max_capacity - load for load in loads]
+        fits = [b for b in range(len(loads)) if room[b] >= length]
+        if fits:
+            target = min(fits, key=lambda b: (room[b], b))
+            loads[target] += length
+            members[target].append((idx, length))
+        else:
+            loads.append(length)
+            members.append([(idx, length)])
+    for _ in range(3 if len(loads) > 1 else 0):
+        order = sorted(range(len(loads)), key=lambda b: loads[b])          # stable, ascending load
+        loads = [loads[b] for b in order]
+        members = [members[b] for b in order]
+        move = _first_narrowing_move(loads, members, max_capacity)
+        if move is None:
+            break
+        heavy, light, slot = move
+        item = members[heavy].pop(slot)
+        members[light].append(item)
+        loads[heavy] -= item[1]
+        loads[light] += item[1]
+    return [[idx for idx, _ in bin_members] for bin_members in members]
+
+
+def _first_narrowing_move(loads, members, max_capacity):
+    """(heavy bin, light bin, position in the heavy bin) of the first item, scanning the fullest
+    bin first against the emptiest first, whose move keeps the capacity and narrows the gap."""
+    for heavy in range(len(loads) - 1, 0, -1):
+        for light in range(heavy):
+            gap = loads[heavy] - loads[light]
+            if gap <= 1:
+                break
+            for slot, (_, length) in enumerate(members[heavy]):
+                if loads[light] + length <= max_capacity and abs(loads[heavy] - loads[light] - 2 * length) < gap:
+                    return heavy, light, slot
+    return None
+
+
 def rearrange_micro_batches(seqlen_list: List[int], max_token_len: int, dynamic_max_batch_size: int = None,
-                            dp_group=None):
+                            dp_group=None, multimodal: bool = False):
     """Micro-batches (index lists) whose token sums are balanced: the bin count comes from the
     capped greedy pass (at least ``ceil(sum / max_token_len)``, and at least
-    ``ceil(n / dynamic_max_batch_size)``), the assignment from the differencing method."""
+    ``ceil(n / dynamic_max_batch_size)``), the assignment from the differencing method.  With
+    ``multimodal`` the capacity-bound bin packing decides both (reference ``:356-359``)."""
+    if multimodal:
+        return balanced_bin_packing(seqlen_list, max_token_len)
     if dp_group is not None:
         raise NotImplementedError("the bin count is not synchronised across ranks on this path (one GPU)")
     floor_bins = (sum(seqlen_list) + max_token_len - 1) // max_token_len

@@ -8,8 +8,10 @@ Restates ``mindspeed_rl/utils/seqlen_balancing.py`` of the reference:
 * ``:127-156``  ``heapq_partition`` (longest first onto the lightest group; equal-size variant)
 * ``:159-188``  ``get_seqlen_balanced_partitions``
 * ``:310-336``  ``heapq_partition_with_max`` (a group that would overflow is closed and replaced)
-* ``:339-380``  ``rearrange_micro_batches`` at data-parallel size 1, text-only (the multimodal bin
-  packing branch and the MAX all-reduce of the bin count are not on this path)
+* ``:191-307``  ``balanced_bin_packing`` / ``_balance_bins`` (best fit decreasing under a capacity, then
+  up to three single-item moves), the branch ``rearrange_micro_batches`` takes for multimodal batches
+* ``:339-380``  ``rearrange_micro_batches`` at data-parallel size 1 (the MAX all-reduce of the bin
+  count is not on this path)
 * ``:383-388``  ``get_reverse_idx``
 
 PARITY UNPINNED against reference-held vectors: the reference has no test or fixture for this
@@ -143,7 +145,63 @@ def heapq_partition_with_max(seqlen_list, k_partitions, max_token_len):
     return partitions
 
 
-def rearrange_micro_batches(seqlen_list, max_token_len, dynamic_max_batch_size=None, dp_group=None):
+def balanced_bin_packing(seqlen_list, max_capacity):
+    """``:191-251``: bins are dicts {'items': [(index, length)], 'used': int}."""
+    if not seqlen_list:
+        return []
+    by_length = sorted(((length, i) for i, length in enumerate(seqlen_list)), reverse=True)
+    bins = []
+    for length, index in by_length:
+        if length > max_capacity:
+            raise ValueError(f"Item with seqlen {length} exceeds max_capacity {max_capacity}")
+        best, best_left = -1, max_capacity + 1
+        for b, info in enumerate(bins):
+            left = max_capacity - info["used"]
+            if left >= length and left < best_left:
+                best, best_left = b, left
+        if best >= 0:
+            bins[best]["items"].append((index, length))
+            bins[best]["used"] += length
+        else:
+            bins.append({"items": [(index, length)], "used": length})
+    _balance_bins(bins, max_capacity)
+    return [[index for index, _ in info["items"]] for info in bins]
+
+
+def _balance_bins(bins, max_capacity):
+    """``:254-307``: three passes at most, one move per pass."""
+    if len(bins) <= 1:
+        return
+    for _ in range(3):
+        moved = False
+        bins.sort(key=lambda info: info["used"])
+        for hi in range(len(bins) - 1, 0, -1):
+            heavy = bins[hi]
+            for lo in range(hi):
+                light = bins[lo]
+                diff = heavy["used"] - light["used"]
+                if diff <= 1:
+                    break
+                for pos, (index, length) in enumerate(heavy["items"]):
+                    new_light = light["used"] + length
+                    new_heavy = heavy["used"] - length
+                    if new_light <= max_capacity and abs(new_heavy - new_light) < diff:
+                        light["items"].append(heavy["items"].pop(pos))
+                        heavy["used"] -= length
+                        light["used"] += length
+                        moved = True
+                        break
+                if moved:
+                    break
+            if moved:
+                break
+        if not moved:
+            break
+
+
+def rearrange_micro_batches(seqlen_list, max_token_len, dynamic_max_batch_size=None, dp_group=None, multimodal=False):
+    if multimodal:                       # ``:356-359`` (the reference reads a global switch)
+        return balanced_bin_packing(seqlen_list, max_token_len)
     total = sum(seqlen_list)
     k_partitions = (total + max_token_len - 1) // max_token_len
     k_partitions = len(heapq_partition_with_max(seqlen_list, k_partitions, max_token_len))

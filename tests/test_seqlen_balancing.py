@@ -122,3 +122,70 @@ def test_split_batches_with_dynamic_bsz():
     order = [i for part in partitions for i in part]
     back = sb.get_reverse_idx(order)
     assert [order[j] for j in back] == list(range(n))
+
+
+def _plain_best_fit_decreasing(lengths, cap):
+    """Textbook best fit decreasing (no balancing pass): bin loads."""
+    loads = []
+    for length in sorted(lengths, reverse=True):
+        fits = [b for b, load in enumerate(loads) if cap - load >= length]
+        if fits:
+            loads[min(fits, key=lambda b: cap - loads[b])] += length
+        else:
+            loads.append(length)
+    return loads
+
+
+def test_oracle_bin_packing_textbook_brute_force_and_invariants():
+    # a worked best-fit-decreasing example: 8 | 4 4 | 2 joins the 8 (tightest fit, first on ties) | 1 1 -> 10 / 10
+    parts = ob.balanced_bin_packing([4, 8, 1, 4, 2, 1], 10)
+    assert _sums([4, 8, 1, 4, 2, 1], parts) == [10, 10] and _is_partition(6, parts)
+    assert ob.balanced_bin_packing([], 10) == []
+    assert ob.balanced_bin_packing([7], 7) == [[0]]
+    with pytest.raises(ValueError):
+        ob.balanced_bin_packing([3, 11], 10)
+    # the balancing pass: best fit alone gives 9 / 2 at capacity 10; moving the 3 leaves 6 / 5
+    assert _sums([6, 3, 2], ob.balanced_bin_packing([6, 3, 2], 10)) == [5, 6]
+    rnd = random.Random(11)
+    for _ in range(300):
+        n = rnd.randint(1, 8)
+        cap = rnd.randint(5, 40)
+        lengths = [rnd.randint(1, cap) for _ in range(n)]
+        parts = ob.balanced_bin_packing(lengths, cap)
+        loads = [sum(lengths[i] for i in p) for p in parts]
+        assert _is_partition(n, parts) and all(p for p in parts) and max(loads) <= cap
+        plain = _plain_best_fit_decreasing(lengths, cap)
+        # the balancing pass keeps the bin count and never widens the range of loads
+        assert len(loads) == len(plain)
+        assert max(loads) <= max(plain) and min(loads) >= min(plain)
+        # bin count against the optimum (all assignments of n items to at most n bins): best fit
+        # decreasing needs at most 11/9 OPT + 6/9 bins
+        if n > 6:
+            continue
+        best = None
+        for assign in itertools.product(range(n), repeat=n):
+            used = {}
+            for length, b in zip(lengths, assign):
+                used[b] = used.get(b, 0) + length
+            if max(used.values()) <= cap and (best is None or len(used) < best):
+                best = len(used)
+            if best == -(-sum(lengths) // cap):
+                break
+        assert len(loads) <= 11 * best / 9 + 6 / 9 + 1e-9
+
+
+def test_bin_packing_matches_oracle():
+    rnd = random.Random(17)
+    for _ in range(400):
+        n = rnd.randint(0, 40)
+        cap = rnd.randint(8, 4096)
+        lengths = [rnd.randint(1, cap) if rnd.random() < 0.3 else rnd.randint(1, max(1, cap // 4)) for _ in range(n)]
+        want = ob.balanced_bin_packing(list(lengths), cap)
+        assert sb.balanced_bin_packing(lengths, cap) == want
+        assert sb.rearrange_micro_batches(lengths, cap, multimodal=True) == want
+        assert ob.rearrange_micro_batches(lengths, cap, multimodal=True) == want
+    # many equal lengths (ties everywhere) and a case the balancing pass changes three times
+    for lengths, cap in (([5] * 13, 12), ([9, 9, 9, 1, 1, 1, 1, 1, 1], 12), ([10, 6, 5, 4, 3, 2, 2, 1], 11)):
+        assert sb.balanced_bin_packing(lengths, cap) == ob.balanced_bin_packing(lengths, cap)
+    with pytest.raises(ValueError, match="exceeds max_capacity"):
+        sb.balanced_bin_packing([3, 11], 10)
