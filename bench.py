@@ -61,6 +61,9 @@ def parse_args():
     ap.add_argument("--path", default="fused", choices=["fused", "split"],
                     help="fused: one sweep computes log-prob, loss and dlogits (1 read + 1 write of [T,V]); "
                          "split: forward sweep, then the backward sweep from the saved logsumexp (2 reads + 1 write)")
+    ap.add_argument("--upstream", type=float, default=1.0,
+                    help="scalar the step multiplies the loss by before backward(), as Megatron's schedule does with "
+                         "1/num_microbatches; the loss object is not told and learns it from the first backward")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=2048, help="rows of the CPU baseline sample")
     ap.add_argument("--seed", type=int, default=0)
@@ -193,12 +196,13 @@ def cpu_baseline(torch, w, rows_target, entropy_coeff, seed, mrl=None, dev=None,
         loss.backward()
         return time.perf_counter() - t0
 
-    one()
-    times = sorted(one() for _ in range(3))
+    for _ in range(3):
+        one()
+    times = sorted(one() for _ in range(5))
     med = times[len(times) // 2]
     out = {
         "value": tokens / med, "unit": "tokens/s", "cores": threads, "kind": "port",
-        "sample": "%d responses, %d packed rows x V=%d (fp32 up-cast), oracle fwd+bwd, median of 3 after 1 warm-up, "
+        "sample": "%d responses, %d packed rows x V=%d (fp32 up-cast), oracle fwd+bwd, median of 5 after 3 warm-ups, "
                   "%.2f s per pass" % (group, total, vocab, med),
     }
     if dev is not None:
@@ -341,17 +345,21 @@ def run_lmhead_train(args):
     print(json.dumps(result), flush=True)
 
 
-# HBM bytes per launch of the dominant kernel from the committed rocprofv3 --pmc summary
-# (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for the copy probe); only
-# the default workload has been profiled that way, every other run reports null.
-PROFILED_TRAFFIC_BYTES = {("c1", "fused", "mrl_fused_logprob_loss"): 104.05e9,
-                          ("c1", "split", "mrl_vocab_logprob_bwd"): 104.06e9}
+# HBM bytes per launch of the dominant kernel.  Not measured by this run: the figure comes from the
+# committed rocprofv3 --pmc summaries (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter
+# reads for the copy probe).  Only the default workload has been profiled that way; any other
+# workload, another library build (MRL_LIB_PATH) or a tuning switch (MRL_*) reports null.
+PROFILED_TRAFFIC = {
+    ("c1", "fused", "mrl_fused_logprob_loss"): (104.05e9, "profiles/fused_sweep_persistent_kernel__c1_qwen25_grpo.md"),
+    ("c1", "split", "mrl_vocab_logprob_bwd"): (104.06e9, "profiles/vocab_fwd_kernel_and_bwd_chunk_kernel__c1_split_path.md"),
+}
 
 
 def _profiled_traffic(args, w, dominant):
-    if args.entropy_coeff != 0.001:
-        return None
-    return PROFILED_TRAFFIC_BYTES.get((args.workload, args.path, dominant))
+    """(bytes or None, where the figure comes from)."""
+    if args.entropy_coeff != 0.001 or any(k.startswith("MRL_") for k in os.environ):
+        return None, None
+    return PROFILED_TRAFFIC.get((args.workload, args.path, dominant), (None, None))
 
 
 def main():
@@ -394,12 +402,14 @@ def main():
     def step():
         z = logits.detach().requires_grad_()
         loss, stats = f.compute_loss(z, b, fused=(args.path == "fused"), **kw)
-        (dz,) = torch.autograd.grad(loss, z)
+        (dz,) = torch.autograd.grad(loss if args.upstream == 1.0 else loss * args.upstream, z)
         return loss, stats, dz
 
+    rescales = f.grad_scale_state(dev).rescales
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    rescales_before = int(rescales.item())
     vocab_ops.kernel_events = []
     dz = None
     t0 = time.perf_counter()
@@ -426,8 +436,13 @@ def main():
         "mrl_vocab_logprob_bwd": live_rows * 2 * row_bytes + dead_rows * row_bytes,
         "mrl_fused_logprob_loss": live_rows * 2 * row_bytes + dead_rows * row_bytes,
     }
-    kernel_symbol = {"mrl_vocab_logprob_fwd": "vocab_fwd_kernel", "mrl_vocab_logprob_bwd": "bwd_chunk_kernel",
-                     "mrl_fused_logprob_loss": "fused_sweep_persistent_kernel"}
+    # the kernel each entry point dispatches to for this shape (csrc/row_sweep.hip, csrc/vocab_logprob.hip)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    persistent = os.environ.get("MRL_SWEEP_PERSISTENT", "1") != "0" and total > 2 * cus
+    chunked = os.environ.get("MRL_BWD_CHUNK", "1") != "0" and row_bytes >= 16384 and row_bytes % 16 == 0
+    kernel_symbol = {"mrl_vocab_logprob_fwd": "vocab_fwd_kernel",
+                     "mrl_vocab_logprob_bwd": "bwd_chunk_kernel" if chunked else "vocab_bwd_kernel",
+                     "mrl_fused_logprob_loss": "fused_sweep_persistent_kernel" if persistent else "fused_sweep_kernel"}
     kernels = {}
     for name, nbytes in kernel_bytes.items():
         ms = avg_ms(name)
@@ -442,6 +457,7 @@ def main():
     # path needs only 2 of them, so the same step is also quoted against that 3-pass byte count
     three_pass_bytes = total * row_bytes + live_rows * 2 * row_bytes + dead_rows * row_bytes
     three_pass_gbps = three_pass_bytes / (ms_per_step * 1e-3) / 1e9
+    traffic, traffic_source = _profiled_traffic(args, w, dominant)
 
     result = {
         "metric": "tokens/sec for logprob+GRPO loss fwd+bwd; achieved HBM GB/s as % of peak",
@@ -461,17 +477,22 @@ def main():
             "packed_rows": total, "response_tokens": tokens,
             "vocab": vocab, "accumulate": "f32", "loss_kind": w.get("loss", "grpo: clip 0.2, low_var_kl 0.001"),
             "entropy_coeff": args.entropy_coeff, "loss": "token-mean", "path": args.path,
+            # the scalar the step multiplies the loss by before backward(); the loss object is not told
+            "upstream": args.upstream,
         },
         "roofline": {
             "kernel": "%s (%s)" % (kernels[dominant]["symbol"], dominant), "bound": "hbm",
             "achieved": kernels[dominant]["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": kernels[dominant]["frac"], "traffic": _profiled_traffic(args, w, dominant),
+            "frac": kernels[dominant]["frac"], "traffic": traffic,
+            "traffic_source": {"measured_this_run": False, "from_committed_profile": traffic_source},
             "bytes_per_launch": kernels[dominant]["bytes_per_launch"], "avg_ms": kernels[dominant]["avg_ms"],
         },
         "kernels": kernels,
-        "step_hbm": {"GBps": step_gbps, "frac": step_gbps / HBM_PEAK_GBPS, "algorithmic_bytes_per_step": step_bytes,
-                     "three_pass_equivalent_GBps": three_pass_gbps,
-                     "three_pass_equivalent_frac": three_pass_gbps / HBM_PEAK_GBPS},
+        "step_hbm": {"GBps": step_gbps, "frac": step_gbps / HBM_PEAK_GBPS, "algorithmic_bytes_per_step": step_bytes},
+        # NOT a roofline fraction: the step's time applied to the bytes a 3-pass (read, read, write)
+        # implementation would move, so that the fused and the split path can be compared on one denominator
+        "comparison_on_three_pass_bytes": {"bytes": three_pass_bytes, "equivalent_GBps": three_pass_gbps},
+        "rescale_passes_in_timed_steps": int(rescales.item()) - rescales_before if args.path == "fused" else None,
         "stats": {k: float(v) for k, v in stats.items()},
         "loss": float(loss.detach()),
     }

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define MRL_VERSION 100
+#define MRL_VERSION 200
 
 enum mrl_status {
     MRL_OK = 0,
@@ -299,21 +299,28 @@ int mrl_fused_loss_prepare(int layout, int64_t batch, int64_t width, int64_t n_r
 
 /* Step 2.  The sweep.  Per row with a non-zero mask: logp, entropy (if `entropy` is given) as in
  * mrl_vocab_logprob_fwd; the token's loss terms as in mrl_policy_loss_fwd; then
- *   dlogits = grad_scale * d(loss)/d(logits)   (grad_scale = loss_scale * the upstream gradient
- *   the caller expects, normally 1)
- * written in the logits dtype.  Rows with mask 0 get zero dlogits and are not read.  dlogits may
+ *   dlogits = grad_scale * (*grad_scale_dev) * d(loss)/d(logits)
+ * written in the logits dtype.  grad_scale carries what the host knows (loss_scale, and the upstream
+ * gradient if the caller was told it); grad_scale_dev (nullable, NULL = 1) is a DEVICE scalar read by
+ * the kernel, typically the upstream gradient that mrl_grad_scale_note recorded at the previous
+ * backward - Megatron's 1/num_microbatches and loss scale reach the loss function only through
+ * autograd (models/base/base_training_engine.py:238-270), so the host never knows them in time.  Rows with mask 0 get zero dlogits and are not read.  dlogits may
  * alias logits exactly (in-place).  row_terms float [n_rows * 8] receives {pg, clipped, old-lp,
  * kl, entropy, 1} * mask per row for step 3.  logp / entropy: nullable [n_rows] outputs.
- * has_old = 0 means old_log_prob = log_prob.detach() (ratio 1).  Needs 16-byte aligned rows,
- * vocab % (16/elem) == 0 and vocab <= mrl_fused_max_vocab(dtype), else MRL_ERR_UNSUPPORTED (use
- * the split fwd/bwd entry points then). */
+ * has_old = 0 means old_log_prob = log_prob.detach() (ratio 1).  row_ticket (nullable): 4 bytes of
+ * device memory owned by the caller, the counter from which the persistent workgroups take their
+ * next row (reset by this call on `stream`; it must not be shared by sweeps that can be in flight at
+ * the same time, and a captured graph keeps using the address it was captured with).  NULL: rows are
+ * walked with a fixed stride, about a twentieth slower on large batches.  Needs 16-byte aligned
+ * rows, vocab % (16/elem) == 0 and vocab <= mrl_fused_max_vocab(dtype), else MRL_ERR_UNSUPPORTED
+ * (use the split fwd/bwd entry points then). */
 int mrl_fused_logprob_loss(const void* logits, int logits_dtype, int64_t n_rows, int64_t vocab,
                            int64_t row_stride, const void* labels, int labels_dtype,
                            float inv_temperature, const float* row_ops, int has_old,
                            float clip_lo, float clip_hi, int kl_penalty, float kl_coef,
-                           float entropy_coeff, float grad_scale, void* dlogits,
-                           int64_t dlogits_row_stride, float* logp, float* entropy,
-                           float* row_terms, void* stream);
+                           float entropy_coeff, float grad_scale, const float* grad_scale_dev,
+                           void* dlogits, int64_t dlogits_row_stride, float* logp, float* entropy,
+                           float* row_terms, uint32_t* row_ticket, void* stream);
 
 /* Step 3.  Sums row_terms per sequence (tokens with a non-zero mask but no logits row enter with
  * log_prob = entropy = 0, as in the split path) and finalizes out[8] / row_sums exactly like
@@ -327,11 +334,22 @@ int mrl_fused_loss_reduce(const float* row_terms, const int64_t* row_start,
                           int seq_mean, float loss_scale, float* row_sums, float* out,
                           void* stream);
 
-/* x[r, :] *= (*upstream / assumed) in place, unless that ratio is exactly 1 (then the kernel
- * exits without touching memory).  Lets the eager gradient honour whatever scalar autograd
- * delivers (Megatron's 1/num_microbatches and loss scale) without a host synchronisation. */
+/* x[r, :] *= (*upstream / *applied) in place, unless that ratio is exactly 1 (then the kernel
+ * exits without touching memory).  upstream and applied are DEVICE scalars: the gradient autograd
+ * delivers and the scale x already carries.  Lets the eager gradient honour whatever scalar arrives
+ * (Megatron's 1/num_microbatches and loss scale) without a host synchronisation.  Neither scalar is
+ * written; follow the last mrl_scale_rows of a backward with mrl_grad_scale_note. */
 int mrl_scale_rows(void* x, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
-                   const float* upstream, float assumed, void* stream);
+                   const float* upstream, const float* applied, void* stream);
+
+/* Book-keeping after the mrl_scale_rows calls of one backward (no counterpart in the reference,
+ * where autograd multiplies by the upstream gradient as part of every backward op): *applied =
+ * *upstream, so a second backward over the same buffers rescales by the ratio of the two upstream
+ * values only; *learned (nullable) = *upstream if that is finite and non-zero - the scalar the next
+ * mrl_fused_logprob_loss reads through grad_scale_dev; *rescales (nullable) is incremented when
+ * upstream differed from applied, i.e. when the rescale moved memory.  All DEVICE pointers. */
+int mrl_grad_scale_note(const float* upstream, float* applied, float* learned, uint32_t* rescales,
+                        void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Fused lm_head + log-prob, forward (no counterpart in the reference, which always materialises

@@ -20,6 +20,8 @@ struct FusedArgs {
     const void* labels; int labels_dtype; float inv_t;
     const float* row_ops; int has_old;
     float clip_lo, clip_hi; int kl_penalty; float kl_coef, entropy_coeff, grad_scale;
+    const float* grad_scale_dev;    // nullable device scalar that multiplies grad_scale
+    unsigned int* row_ticket;       // nullable: the caller's row counter of the persistent sweep
     void* dlogits; int64_t d_stride;
     float* logp; float* entropy; float* row_terms;
     bool with_entropy;

@@ -16,8 +16,6 @@
 // has to stay on chip): a plain stream of one vector per thread.
 #include <stdlib.h>
 
-#include <atomic>
-
 #include "mrl_internal.h"
 #include "policy_terms.h"
 #include "row_sweep.h"
@@ -301,13 +299,14 @@ template <int DT, int NV, bool kEntropy>
 __global__ __launch_bounds__(kBlock) void fused_sweep_kernel(
     const typename Elem<DT>::T* logits, int64_t row_stride, int vocab, const void* __restrict__ labels,
     int labels_dtype, float inv_t, const float* __restrict__ row_ops, int has_old, Params p, float grad_scale,
-    typename Elem<DT>::T* dlogits, int64_t d_stride, float* __restrict__ logp, float* __restrict__ entropy,
-    float* __restrict__ row_terms) {
+    const float* __restrict__ grad_scale_dev, typename Elem<DT>::T* dlogits, int64_t d_stride,
+    float* __restrict__ logp, float* __restrict__ entropy, float* __restrict__ row_terms) {
     using E = Elem<DT>;
     using T = typename E::T;
     constexpr int kVec = E::kVec;
     __shared__ Stats lds[kWaves + 1];
 
+    if (grad_scale_dev) grad_scale *= *grad_scale_dev;
     const int64_t r = blockIdx.x;
     const int tid = threadIdx.x;
     const int n_vec = vocab / kVec;
@@ -358,14 +357,10 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_kernel(
 // the next unclaimed one.  With a fixed stride (row r, r + grid, ...) the workgroups drift apart and
 // the rows in flight spread over a wide stretch of memory; with tickets the rows in flight are always
 // the most recent `grid` consecutive ones, which the HBM system serves about a tenth faster.
-// The counters live in device memory of the library (one array per GPU); a launch takes the next
-// slot round-robin and resets it with ticket_reset_kernel on the same stream, so launches that are
-// in flight together on different streams do not share a counter (up to kTicketSlots of them).
-constexpr int kTicketSlots = 256;
-__device__ unsigned int g_row_ticket[kTicketSlots];
-
-__global__ void ticket_reset_kernel(int slot, unsigned int first) {
-    if (threadIdx.x == 0) g_row_ticket[slot] = first;
+// The counter is four bytes of device memory that the caller owns (one per sweep that can be in
+// flight at a time); the launch resets it with ticket_reset_kernel on the same stream.
+__global__ void ticket_reset_kernel(unsigned int* counter, unsigned int first) {
+    if (threadIdx.x == 0) *counter = first;
 }
 
 // Thread 0 passes its ticket to the workgroup through LDS.  The fences order LDS accesses only and
@@ -392,8 +387,9 @@ template <int DT, int NV, bool kEntropy, bool kTicket>
 __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
     const typename Elem<DT>::T* logits, int64_t row_stride, int vocab, int64_t n_rows,
     const void* __restrict__ labels, int labels_dtype, float inv_t, const float* __restrict__ row_ops, int has_old,
-    Params p, float grad_scale, typename Elem<DT>::T* dlogits, int64_t d_stride, float* __restrict__ logp,
-    float* __restrict__ entropy, float* __restrict__ row_terms, int ticket_slot) {
+    Params p, float grad_scale, const float* __restrict__ grad_scale_dev, typename Elem<DT>::T* dlogits,
+    int64_t d_stride, float* __restrict__ logp, float* __restrict__ entropy, float* __restrict__ row_terms,
+    unsigned int* row_ticket) {
     using E = Elem<DT>;
     using T = typename E::T;
     constexpr int kVec = E::kVec;
@@ -407,8 +403,9 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
     const uint32_t row_bytes = (uint32_t)vocab * (uint32_t)sizeof(T);
     const float k = inv_t * kLog2e;
     const int64_t step = gridDim.x;
+    if (grad_scale_dev) grad_scale *= *grad_scale_dev;
     // the counter as a 4-byte buffer: only the lane with offset 0 (thread 0) is inside it
-    const mrl::rsrc_t ticket = mrl::make_rsrc(&g_row_ticket[ticket_slot], 4u);
+    const mrl::rsrc_t ticket = mrl::make_rsrc(kTicket ? (const void*)row_ticket : (const void*)dlogits, kTicket ? 4u : 0u);
 
     // What a workgroup needs to know of the row it fetches next.  A row that is not a response token
     // is never read: its descriptor gets zero bytes, so the (unconditional) loads return zeros
@@ -570,15 +567,15 @@ __global__ __launch_bounds__(kThreads) void bwd_chunk_kernel(
     }
 }
 
-// Conditional in-place rescale: multiplies every row by upstream/assumed unless that ratio is 1
+// Conditional in-place rescale: multiplies every row by upstream/applied unless that ratio is 1
 // (then every workgroup exits at once; the grid is kept small so that this costs microseconds).
 template <int DT>
 __global__ __launch_bounds__(256) void scale_rows_kernel(typename Elem<DT>::T* x, int64_t row_stride, int vocab,
                                                          int64_t n_rows, const float* __restrict__ upstream,
-                                                         float assumed) {
+                                                         const float* __restrict__ applied) {
     using E = Elem<DT>;
     constexpr int kVec = E::kVec;
-    const float ratio = *upstream / assumed;
+    const float ratio = *upstream / *applied;
     if (ratio == 1.f) return;
     const int n_vec = vocab / kVec;
     for (int64_t r = blockIdx.x; r < n_rows; r += gridDim.x) {
@@ -591,6 +588,18 @@ __global__ __launch_bounds__(256) void scale_rows_kernel(typename Elem<DT>::T* x
             vec[idx] = E::pack(z);
         }
     }
+}
+
+// Book-keeping behind one or more scale_rows_kernel launches: the buffers now carry `upstream`.
+__global__ void grad_scale_note_kernel(const float* __restrict__ upstream, float* applied, float* learned,
+                                       uint32_t* rescales) {
+    if (threadIdx.x != 0) return;
+    const float u = *upstream;
+    const float was = *applied;
+    if (rescales && u / was != 1.f) *rescales += 1u;
+    *applied = u;
+    // a scale that the next sweep can start from: finite and non-zero
+    if (learned && u != 0.f && __builtin_isfinite(u)) *learned = u;
 }
 
 // ----------------------------------------------------------------------------- host dispatch
@@ -621,24 +630,6 @@ bool persistent_enabled() {
     return on;
 }
 
-// MRL_SWEEP_TICKET=0 walks rows with a fixed stride instead of tickets (a tuning switch).
-bool ticket_enabled() {
-    static const bool on = [] {
-        const char* e = getenv("MRL_SWEEP_TICKET");
-        return !(e && e[0] == '0');
-    }();
-    return on;
-}
-
-// Next counter slot, reset on the launch stream to the first row that is not handed out by
-// blockIdx (the workgroups start on rows 0 .. grid-1).
-int take_ticket_slot(unsigned first_ticket, hipStream_t stream) {
-    static std::atomic<unsigned> next{0};
-    const int slot = (int)(next.fetch_add(1u) % (unsigned)kTicketSlots);
-    hipLaunchKernelGGL(ticket_reset_kernel, dim3(1), dim3(64), 0, stream, slot, first_ticket);
-    return slot;
-}
-
 template <int DT, int NV>
 int launch_fused(const mrl::FusedArgs& a) {
     using T = typename Elem<DT>::T;
@@ -650,9 +641,11 @@ int launch_fused(const mrl::FusedArgs& a) {
 #define MRL_FUSEDP_LAUNCH(ENT, TK)                                                                                \
     hipLaunchKernelGGL((fused_sweep_persistent_kernel<DT, NV, ENT, TK>), pgrid, block, 0, a.stream, (const T*)a.logits, \
                        a.row_stride, (int)a.vocab, a.n_rows, a.labels, a.labels_dtype, a.inv_t, a.row_ops,         \
-                       a.has_old, p, a.grad_scale, (T*)a.dlogits, a.d_stride, a.logp, a.entropy, a.row_terms, slot)
-        const bool tk = ticket_enabled();
-        const int slot = tk ? take_ticket_slot((unsigned)cus, a.stream) : 0;
+                       a.has_old, p, a.grad_scale, a.grad_scale_dev, (T*)a.dlogits, a.d_stride, a.logp, a.entropy,     \
+                       a.row_terms, a.row_ticket)
+        // the workgroups start on rows 0 .. grid-1; the counter hands out the rows behind them
+        const bool tk = a.row_ticket != nullptr;
+        if (tk) hipLaunchKernelGGL(ticket_reset_kernel, dim3(1), dim3(64), 0, a.stream, a.row_ticket, (unsigned)cus);
         if (a.with_entropy && tk) MRL_FUSEDP_LAUNCH(true, true);
         else if (a.with_entropy) MRL_FUSEDP_LAUNCH(true, false);
         else if (tk) MRL_FUSEDP_LAUNCH(false, true);
@@ -664,7 +657,7 @@ int launch_fused(const mrl::FusedArgs& a) {
 #define MRL_FUSED_LAUNCH(ENT)                                                                                  \
     hipLaunchKernelGGL((fused_sweep_kernel<DT, NV, ENT>), grid, block, 0, a.stream, (const T*)a.logits,        \
                        a.row_stride, (int)a.vocab, a.labels, a.labels_dtype, a.inv_t, a.row_ops, a.has_old, p, \
-                       a.grad_scale, (T*)a.dlogits, a.d_stride, a.logp, a.entropy, a.row_terms)
+                       a.grad_scale, a.grad_scale_dev, (T*)a.dlogits, a.d_stride, a.logp, a.entropy, a.row_terms)
     if (a.with_entropy) MRL_FUSED_LAUNCH(true);
     else MRL_FUSED_LAUNCH(false);
 #undef MRL_FUSED_LAUNCH
@@ -762,8 +755,9 @@ extern "C" int mrl_fused_logprob_loss(const void* logits, int logits_dtype, int6
                                       int64_t row_stride, const void* labels, int labels_dtype,
                                       float inv_temperature, const float* row_ops, int has_old, float clip_lo,
                                       float clip_hi, int kl_penalty, float kl_coef, float entropy_coeff,
-                                      float grad_scale, void* dlogits, int64_t dlogits_row_stride, float* logp,
-                                      float* entropy, float* row_terms, void* stream) {
+                                      float grad_scale, const float* grad_scale_dev, void* dlogits,
+                                      int64_t dlogits_row_stride, float* logp, float* entropy, float* row_terms,
+                                      uint32_t* row_ticket, void* stream) {
     const char* fn = "mrl_fused_logprob_loss";
     MRL_REQUIRE(n_rows >= 0 && vocab > 0 && n_rows <= 0x7fffffffLL, MRL_ERR_INVALID_ARG, "%s: n_rows=%lld vocab=%lld",
                 fn, (long long)n_rows, (long long)vocab);
@@ -779,6 +773,8 @@ extern "C" int mrl_fused_logprob_loss(const void* logits, int logits_dtype, int6
                 "%s: inv_temperature=%g must be in (0, 1e6)", fn, (double)inv_temperature);
     if (n_rows == 0) return MRL_OK;
     MRL_REQUIRE(logits && labels && row_ops && dlogits && row_terms, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+    MRL_REQUIRE(mrl::aligned(row_ticket, 4) && mrl::aligned(grad_scale_dev, 4), MRL_ERR_MISALIGNED,
+                "%s: row_ticket and grad_scale_dev must be 4-byte aligned", fn);
     MRL_REQUIRE(mrl::row_sweep_supported(logits_dtype, vocab, logits, row_stride, dlogits, dlogits_row_stride, n_rows),
                 MRL_ERR_UNSUPPORTED,
                 "%s: needs 16-byte aligned rows, vocab %% %d == 0 and vocab <= %lld for this dtype (got vocab=%lld)", fn,
@@ -795,7 +791,8 @@ extern "C" int mrl_fused_logprob_loss(const void* logits, int logits_dtype, int6
     a.logits = logits; a.dtype = logits_dtype; a.n_rows = n_rows; a.vocab = vocab; a.row_stride = row_stride;
     a.labels = labels; a.labels_dtype = labels_dtype; a.inv_t = inv_temperature; a.row_ops = row_ops;
     a.has_old = has_old; a.clip_lo = clip_lo; a.clip_hi = clip_hi; a.kl_penalty = kl_penalty; a.kl_coef = kl_coef;
-    a.entropy_coeff = entropy_coeff; a.grad_scale = grad_scale; a.dlogits = dlogits; a.d_stride = dlogits_row_stride;
+    a.entropy_coeff = entropy_coeff; a.grad_scale = grad_scale; a.grad_scale_dev = grad_scale_dev;
+    a.row_ticket = row_ticket; a.dlogits = dlogits; a.d_stride = dlogits_row_stride;
     a.logp = logp; a.entropy = entropy; a.row_terms = row_terms; a.with_entropy = (entropy != nullptr);
     a.stream = mrl::as_stream(stream);
     const int nv = pick_nv(vocab / (16 / eb));
@@ -807,16 +804,17 @@ extern "C" int mrl_fused_logprob_loss(const void* logits, int logits_dtype, int6
 }
 
 extern "C" int mrl_scale_rows(void* x, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
-                              const float* upstream, float assumed, void* stream) {
+                              const float* upstream, const float* applied, void* stream) {
     const char* fn = "mrl_scale_rows";
     const int eb = mrl::float_dtype_bytes(dtype);
     MRL_REQUIRE(eb != 0, MRL_ERR_UNSUPPORTED, "%s: dtype %d (want F32, BF16 or F16)", fn, dtype);
     MRL_REQUIRE(n_rows >= 0 && n_rows <= 0x7fffffffLL && vocab > 0 && row_stride >= vocab, MRL_ERR_INVALID_ARG,
                 "%s: n_rows=%lld vocab=%lld row_stride=%lld", fn, (long long)n_rows, (long long)vocab,
                 (long long)row_stride);
-    MRL_REQUIRE(assumed != 0.f, MRL_ERR_INVALID_ARG, "%s: assumed scale is zero", fn);
     if (n_rows == 0) return MRL_OK;
-    MRL_REQUIRE(x && upstream, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+    MRL_REQUIRE(x && upstream && applied, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+    MRL_REQUIRE(mrl::aligned(upstream, 4) && mrl::aligned(applied, 4), MRL_ERR_MISALIGNED,
+                "%s: upstream and applied must be 4-byte aligned", fn);
     MRL_REQUIRE(vocab % (16 / eb) == 0 && mrl::aligned(x, 16) && (n_rows == 1 || (row_stride * eb) % 16 == 0),
                 MRL_ERR_UNSUPPORTED, "%s: needs 16-byte aligned rows", fn);
     hipStream_t s = mrl::as_stream(stream);
@@ -824,16 +822,28 @@ extern "C" int mrl_scale_rows(void* x, int dtype, int64_t n_rows, int64_t vocab,
     switch (dtype) {
         case MRL_F32:
             hipLaunchKernelGGL(scale_rows_kernel<MRL_F32>, grid, block, 0, s, (float*)x, row_stride, (int)vocab,
-                               n_rows, upstream, assumed);
+                               n_rows, upstream, applied);
             break;
         case MRL_BF16:
             hipLaunchKernelGGL(scale_rows_kernel<MRL_BF16>, grid, block, 0, s, (uint16_t*)x, row_stride, (int)vocab,
-                               n_rows, upstream, assumed);
+                               n_rows, upstream, applied);
             break;
         default:
             hipLaunchKernelGGL(scale_rows_kernel<MRL_F16>, grid, block, 0, s, (uint16_t*)x, row_stride, (int)vocab,
-                               n_rows, upstream, assumed);
+                               n_rows, upstream, applied);
             break;
     }
+    return mrl::check_launch(fn);
+}
+
+extern "C" int mrl_grad_scale_note(const float* upstream, float* applied, float* learned, uint32_t* rescales,
+                                   void* stream) {
+    const char* fn = "mrl_grad_scale_note";
+    MRL_REQUIRE(upstream && applied, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+    MRL_REQUIRE(mrl::aligned(upstream, 4) && mrl::aligned(applied, 4) && mrl::aligned(learned, 4) &&
+                    mrl::aligned(rescales, 4),
+                MRL_ERR_MISALIGNED, "%s: pointers must be 4-byte aligned", fn);
+    hipLaunchKernelGGL(grad_scale_note_kernel, dim3(1), dim3(64), 0, mrl::as_stream(stream), upstream, applied, learned,
+                       rescales);
     return mrl::check_launch(fn);
 }

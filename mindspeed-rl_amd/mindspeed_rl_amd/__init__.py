@@ -9,9 +9,9 @@ from .advantage import (FixedKLController, compute_group_norm_advantage_return, 
                         dynamic_sampling_keep_mask)
 from .functional import clip_by_value, masked_mean, masked_sum
 from .lmhead import fused_lmhead_policy_loss, lmhead_logprob
-from .loss import (BaseLossFunc, DAPOActorLossFunc, GRPOActorLossFunc, LossFuncFactory, LossRegister,
-                   MultimodalLogProbComputer, PPOActorLossFunc, ReferenceLossFunc, RewardLossFunc, StandardLogProbComputer, fused_logprob_policy_loss, fused_supported,
-                   policy_loss)
+from .loss import (BaseLossFunc, DAPOActorLossFunc, GradScaleState, GRPOActorLossFunc, LossFuncFactory, LossRegister,
+                   MultimodalLogProbComputer, PPOActorLossFunc, ReferenceLossFunc, RewardLossFunc,
+                   StandardLogProbComputer, fused_logprob_policy_loss, fused_supported, policy_loss)
 from .packing import (generate_mask, pack_index, postprocess_packed_seqs, preprocess_packed_seqs, response_window,
                       truncate_middle_and_pad, truncate_prompt_and_pad)
 from .seqlen_balancing import (balanced_bin_packing, get_reverse_idx, get_seqlen_balanced_partitions, heapq_partition,

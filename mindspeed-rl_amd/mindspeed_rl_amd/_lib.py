@@ -52,10 +52,11 @@ SIGNATURES = {
     "mrl_fused_loss_prepare": [_int, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _int, _vp, _int, _vp, _vp, _vp, _vp, _int,
                                _int, _vp, _vp, _vp, _vp, _vp],
     "mrl_fused_logprob_loss": [_vp, _int, _i64, _i64, _i64, _vp, _int, _f32, _vp, _int, _f32, _f32, _int, _f32, _f32,
-                               _f32, _vp, _i64, _vp, _vp, _vp, _vp],
+                               _f32, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp],
     "mrl_fused_loss_reduce": [_vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _int, _vp, _int, _f32, _f32, _int, _f32,
                               _f32, _int, _f32, _vp, _vp, _vp],
-    "mrl_scale_rows": [_vp, _int, _i64, _i64, _i64, _vp, _f32, _vp],
+    "mrl_scale_rows": [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp],
+    "mrl_grad_scale_note": [_vp, _vp, _vp, _vp, _vp],
     "mrl_lmhead_workspace_bytes": [_i64, _i64],
     "mrl_lmhead_logprob_fwd": [_vp, _vp, _i64, _i64, _i64, _vp, _int, _f32, _vp, _vp, _vp, _vp, _i64, _vp],
     "mrl_group_standardize": [_vp, _int, _i64, _i64, ctypes.c_double, _vp, _vp],

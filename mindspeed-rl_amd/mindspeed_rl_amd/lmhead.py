@@ -92,7 +92,7 @@ class _FusedLmHeadLoss(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, hidden, weight, labels, batch, cfg):
-        from .loss import _mask_args
+        from .loss import _expected_scale, _mask_args, _row_ticket
         dev = _lib.require_device(hidden, weight, labels)
         hdim = hidden.shape[-1]
         h2d = hidden.detach().reshape(-1, hdim).contiguous()
@@ -138,7 +138,8 @@ class _FusedLmHeadLoss(torch.autograd.Function):
                   _lib.ptr(prompt), pdt, _lib.ptr(resp), rdt, _lib.ptr(old), _lib.ptr(ref), _lib.ptr(adv),
                   _lib.ptr(mask_t), mdt, cfg["seq_mean"], _lib.ptr(row_start), _lib.ptr(row_count),
                   _lib.ptr(seq_msum), _lib.ptr(row_ops), stream)
-        grad_scale = cfg["loss_scale"] * cfg["expected_upstream"]
+        grad_scale, scale_dev, applied = _expected_scale(cfg, dev)
+        ticket = _row_ticket(dev)
         # Rows whose mask is zero (prompts, padding, masked tokens) add nothing to the loss, to dWeight or
         # to their own dHidden: when they are more than a twentieth of the rows, the live rows are gathered
         # and only they go through the GEMMs.  The row count sizes the GEMMs, so it is read back (one
@@ -173,8 +174,9 @@ class _FusedLmHeadLoss(torch.autograd.Function):
                 "mrl_fused_logprob_loss", rows, dev, _lib.ptr(z), _lib.dtype_code(z), rows, vocab, vocab,
                 lab.data_ptr() + c0 * lab.element_size(), _lib.dtype_code(lab), cfg["inv_temperature"],
                 row_ops.data_ptr() + c0 * 32, 0 if old is None else 1, cfg["clip_lo"], cfg["clip_hi"], cfg["kl_penalty"],
-                cfg["kl_coef"], cfg["entropy_coeff"], grad_scale, _lib.ptr(z), vocab, None,
-                (ent.data_ptr() + c0 * 4) if want_ent else None, row_terms.data_ptr() + c0 * 32, stream)
+                cfg["kl_coef"], cfg["entropy_coeff"], grad_scale, _lib.ptr(scale_dev), _lib.ptr(z), vocab, None,
+                (ent.data_ptr() + c0 * 4) if want_ent else None, row_terms.data_ptr() + c0 * 32, _lib.ptr(ticket),
+                stream)
             torch.mm(z, w if w_hv is None else w_hv.t(), out=d_hidden[c0:c1])    # dHidden_c = dlogits_c @ W
             # dW += dlogits_c^T @ hidden_c, accumulated in fp32 by the GEMM itself (no separate add pass,
             # no rounding of the chunk's product to bf16)
@@ -195,27 +197,25 @@ class _FusedLmHeadLoss(torch.autograd.Function):
                   cfg["clip_lo"], cfg["clip_hi"], cfg["kl_penalty"], cfg["kl_coef"], cfg["entropy_coeff"],
                   cfg["seq_mean"], cfg["loss_scale"], _lib.ptr(row_sums), _lib.ptr(out), stream)
         d_weight = d_weight32.to(w.dtype)
-        ctx.save_for_backward(d_hidden, d_weight)
-        ctx.meta = (tuple(hidden.shape), cfg["expected_upstream"])
+        ctx.save_for_backward(d_hidden, d_weight, applied)
+        ctx.meta = (tuple(hidden.shape), cfg.get("scale_state"))
+        ctx.handed_out = False
         ctx.mark_non_differentiable(out)
         return out[0].clone(), out
 
     @staticmethod
     def backward(ctx, g_loss, _g_out):
-        d_hidden, d_weight = ctx.saved_tensors
-        shape, expected = ctx.meta
-        dev = d_hidden.device
-        upstream = g_loss.to(torch.float32).reshape(1).contiguous()
-        for t in (d_hidden, d_weight):
-            _lib.call("mrl_scale_rows", _lib.ptr(t), _lib.dtype_code(t), t.shape[0], t.shape[1], t.shape[1],
-                      _lib.ptr(upstream), float(expected), _lib.stream(dev))
+        from .loss import _deliver_eager_grads
+        d_hidden, d_weight, applied = ctx.saved_tensors
+        shape, state = ctx.meta
+        d_hidden, d_weight = _deliver_eager_grads(ctx, (d_hidden, d_weight), applied, state, g_loss)
         return d_hidden.view(shape), d_weight, None, None, None
 
 
 def fused_lmhead_policy_loss(hidden, weight, batch, *, packed, seqlens=None, cu_seqlens=None, mask=None,
                              ref_log_prob=None, clip_low, clip_high, kl_penalty=None, kl_coef=0.0, entropy_coeff=0.0,
-                             token_level_loss=True, loss_scale=1.0, inv_temperature=1.0, expected_upstream=1.0,
-                             chunk_rows=32768, fp32_dw_gemm=False, compact_rows=True):
+                             token_level_loss=True, loss_scale=1.0, inv_temperature=1.0, expected_upstream=None,
+                             scale_state=None, chunk_rows=32768, fp32_dw_gemm=False, compact_rows=True):
     """Policy loss straight from the hidden states: ``hidden`` is packed ``[1, T, H]`` (or padded
     ``[B, S, H]``) bf16, ``weight`` the ``[V, H]`` bf16 lm_head weight; ``batch`` as for
     :func:`mindspeed_rl_amd.fused_logprob_policy_loss` (``labels, responses, response_length,
@@ -237,6 +237,7 @@ def fused_lmhead_policy_loss(hidden, weight, batch, *, packed, seqlens=None, cu_
                clip_lo=float(1.0 - clip_low), clip_hi=float(1.0 + clip_high), kl_penalty=kl_code,
                kl_coef=float(kl_coef), entropy_coeff=float(entropy_coeff), seq_mean=0 if token_level_loss else 1,
                loss_scale=float(loss_scale), inv_temperature=float(inv_temperature),
-               expected_upstream=float(expected_upstream), chunk_rows=int(chunk_rows), fp32_dw_gemm=bool(fp32_dw_gemm),
+               expected_upstream=None if expected_upstream is None else float(expected_upstream),
+               scale_state=scale_state, chunk_rows=int(chunk_rows), fp32_dw_gemm=bool(fp32_dw_gemm),
                compact_rows=bool(compact_rows))
     return _FusedLmHeadLoss.apply(hidden, weight, batch["labels"], batch, cfg)

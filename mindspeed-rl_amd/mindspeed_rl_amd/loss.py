@@ -150,10 +150,74 @@ def fused_supported(output):
     return output.is_contiguous() and output.data_ptr() % 16 == 0
 
 
+class GradScaleState:
+    """What a loss object remembers, in device memory, about the scalar that autograd multiplies its
+    loss by: Megatron divides the loss by ``num_microbatches`` (and applies the loss scale) AFTER
+    the loss function has returned, and the reference's caller does not tell the loss function
+    (``models/base/base_training_engine.py:238-270``).  ``learned`` is the upstream gradient of the
+    most recent backward; the next fused sweep reads it on the device and writes its dlogits with
+    that scale already applied, so the backward finds nothing to rescale.  Everything is ordered
+    by the stream: no host synchronisation, and a wrong guess only costs one rescale pass.
+    ``rescales`` counts the backwards that had to move memory."""
+
+    def __init__(self, device):
+        self.learned = torch.ones(1, dtype=torch.float32, device=device)
+        self.rescales = torch.zeros(1, dtype=torch.int32, device=device)
+
+
+def _row_ticket(dev):
+    """The persistent sweep's row counter: four bytes per call from torch's allocator (a sweep in
+    flight never shares its counter).  MRL_SWEEP_TICKET=0 makes the sweep walk rows with a fixed
+    stride instead (a tuning switch)."""
+    if os.environ.get("MRL_SWEEP_TICKET", "1") == "0":
+        return None
+    return torch.empty(1, dtype=torch.int32, device=dev)
+
+
+def _note_upstream(upstream, applied, state, stream):
+    _lib.call("mrl_grad_scale_note", _lib.ptr(upstream), _lib.ptr(applied),
+              _lib.ptr(state.learned) if state is not None else None,
+              _lib.ptr(state.rescales) if state is not None else None, stream)
+
+
+def _expected_scale(cfg, dev):
+    """(host factor, device scalar or None, applied): the scale the sweep writes into its gradients.
+    An explicit ``expected_upstream`` wins; else the loss object's learned scale is read on the
+    device; else 1."""
+    state, explicit = cfg.get("scale_state"), cfg.get("expected_upstream")
+    if explicit is None and state is not None:
+        applied = state.learned.clone()
+        return cfg["loss_scale"], applied, applied
+    expected = 1.0 if explicit is None else float(explicit)
+    return cfg["loss_scale"] * expected, None, torch.full((1,), expected, dtype=torch.float32, device=dev)
+
+
+def _deliver_eager_grads(ctx, buffers, applied, state, g_loss):
+    """Backward of an eager-gradient op: ``buffers`` hold the gradients at scale ``applied`` (a
+    device scalar); returns them at the scale of ``g_loss``.  The first backward rescales the stored
+    buffers in place and hands them out; a later backward over a retained graph must not touch what
+    the first one handed out, so it scales copies."""
+    dev = buffers[0].device
+    stream = _lib.stream(dev)
+    upstream = g_loss.to(torch.float32).reshape(1).contiguous()
+    first = not ctx.handed_out
+    ctx.handed_out = True
+    if not first:
+        buffers = tuple(t.clone() for t in buffers)
+    for t in buffers:
+        flat = t.view(-1, t.shape[-1])
+        _lib.call("mrl_scale_rows", _lib.ptr(flat), _lib.dtype_code(flat), flat.shape[0], flat.shape[1],
+                  flat.shape[1], _lib.ptr(upstream), _lib.ptr(applied), stream)
+    # the stored buffers now carry `upstream` (first backward) or still what they carried (copies)
+    _note_upstream(upstream, applied if first else applied.clone(), state, stream)
+    return buffers
+
+
 class _FusedLogprobLoss(torch.autograd.Function):
     """logits -> (loss, out[8]) with dlogits produced in the same sweep (one read, one write of
     the [T, V] tensor for forward + backward).  The backward only rescales the stored dlogits if
-    the upstream gradient differs from the scale assumed in the forward."""
+    the upstream gradient differs from the scale they already carry (kept in a device scalar, so
+    a second backward over a retained graph rescales by the ratio of the two upstream values)."""
 
     @staticmethod
     def forward(ctx, output, labels, batch, cfg):
@@ -204,44 +268,45 @@ class _FusedLogprobLoss(torch.autograd.Function):
                   _lib.ptr(prompt), pdt, _lib.ptr(resp), rdt, _lib.ptr(old), _lib.ptr(ref), _lib.ptr(adv),
                   _lib.ptr(mask_t), mdt, cfg["seq_mean"], _lib.ptr(row_start), _lib.ptr(row_count),
                   _lib.ptr(seq_msum), _lib.ptr(row_ops), stream)
-        grad_scale = cfg["loss_scale"] * cfg["expected_upstream"]
+        grad_scale, scale_dev, applied = _expected_scale(cfg, dev)
+        ticket = _row_ticket(dev)
         vocab_ops._timed_call("mrl_fused_logprob_loss", n_rows, dev, _lib.ptr(flat), _lib.dtype_code(flat), n_rows,
                               vocab, vocab, _lib.ptr(lab), _lib.dtype_code(lab), cfg["inv_temperature"],
                               _lib.ptr(row_ops), 0 if old is None else 1, cfg["clip_lo"], cfg["clip_hi"],
-                              cfg["kl_penalty"], cfg["kl_coef"], cfg["entropy_coeff"], grad_scale, _lib.ptr(dlogits),
-                              vocab, None, _lib.ptr(ent), _lib.ptr(row_terms), stream)
+                              cfg["kl_penalty"], cfg["kl_coef"], cfg["entropy_coeff"], grad_scale,
+                              _lib.ptr(scale_dev), _lib.ptr(dlogits), vocab, None, _lib.ptr(ent), _lib.ptr(row_terms),
+                              _lib.ptr(ticket), stream)
         _lib.call("mrl_fused_loss_reduce", _lib.ptr(row_terms), _lib.ptr(row_start), _lib.ptr(row_count), n_seq, width,
                   _lib.ptr(old), _lib.ptr(ref), _lib.ptr(adv), _lib.ptr(mask_t), mdt, _lib.ptr(resp), rdt,
                   cfg["clip_lo"], cfg["clip_hi"], cfg["kl_penalty"], cfg["kl_coef"], cfg["entropy_coeff"],
                   cfg["seq_mean"], cfg["loss_scale"], _lib.ptr(row_sums), _lib.ptr(out), stream)
-        ctx.save_for_backward(dlogits)
-        ctx.meta = (tuple(output.shape), cfg["expected_upstream"])
+        ctx.save_for_backward(dlogits, applied)
+        ctx.meta = (tuple(output.shape), cfg.get("scale_state"))
+        ctx.handed_out = False
         ctx.mark_non_differentiable(out)
         return out[0].clone(), out
 
     @staticmethod
     def backward(ctx, g_loss, _g_out):
-        (dlogits,) = ctx.saved_tensors
-        shape, expected = ctx.meta
-        dev = dlogits.device
-        n_rows, vocab = dlogits.shape
-        upstream = g_loss.to(torch.float32).reshape(1).contiguous()
-        _lib.call("mrl_scale_rows", _lib.ptr(dlogits), _lib.dtype_code(dlogits), n_rows, vocab, vocab,
-                  _lib.ptr(upstream), float(expected), _lib.stream(dev))
-        return dlogits.view(shape), None, None, None
+        dlogits, applied = ctx.saved_tensors
+        shape, state = ctx.meta
+        (grad,) = _deliver_eager_grads(ctx, (dlogits,), applied, state, g_loss)
+        return grad.view(shape), None, None, None
 
 
 def fused_logprob_policy_loss(output, batch, *, packed, seqlens=None, cu_seqlens=None, mask=None, ref_log_prob=None,
                               clip_low, clip_high, kl_penalty=None, kl_coef=0.0, entropy_coeff=0.0,
                               token_level_loss=True, loss_scale=1.0, inv_temperature=1.0, grad_inplace=False,
-                              expected_upstream=1.0):
+                              expected_upstream=None, scale_state=None):
     """Log-prob, entropy, policy loss AND dlogits in one sweep over the logits.
 
     ``output`` is the packed ``[1, T, V]`` (``packed=True``, with ``seqlens`` / ``cu_seqlens``) or
     padded ``[B, S, V]`` logits; ``batch`` holds ``labels, responses, response_length,
     prompt_length, advantages`` and optionally ``old_log_prob``.  Returns ``(loss, out)`` like
-    :func:`policy_loss`.  ``expected_upstream`` is the scalar the caller will multiply the loss by
-    before ``backward()`` (1 unless known otherwise); any other value is honoured by a rescale."""
+    :func:`policy_loss`.  The gradients are written with the scale the caller is expected to
+    multiply the loss by before ``backward()``: ``expected_upstream`` if given, else what
+    ``scale_state`` (a :class:`GradScaleState`) learned from the previous backward, else 1; any
+    other upstream value is honoured by one rescale pass in the backward."""
     if kl_penalty is None:
         kl_code = _lib.KL_NONE
     elif kl_penalty in _lib.KL_BY_NAME:
@@ -252,7 +317,8 @@ def fused_logprob_policy_loss(output, batch, *, packed, seqlens=None, cu_seqlens
                clip_lo=float(1.0 - clip_low), clip_hi=float(1.0 + clip_high), kl_penalty=kl_code,
                kl_coef=float(kl_coef), entropy_coeff=float(entropy_coeff), seq_mean=0 if token_level_loss else 1,
                loss_scale=float(loss_scale), inv_temperature=float(inv_temperature), grad_inplace=bool(grad_inplace),
-               expected_upstream=float(expected_upstream))
+               expected_upstream=None if expected_upstream is None else float(expected_upstream),
+               scale_state=scale_state)
     return _FusedLogprobLoss.apply(output, batch["labels"], batch, cfg)
 
 
@@ -267,11 +333,11 @@ def _use_fused(output, kwargs):
     return torch.is_grad_enabled() and output.requires_grad and fused_supported(output)
 
 
-def _fused_kwargs(kwargs):
+def _fused_kwargs(kwargs, scale_state=None):
     return dict(packed=kwargs.get("use_remove_padding", False), seqlens=kwargs.get("seqlens_in_batch"),
                 cu_seqlens=kwargs.get("cu_seqlens_padded"), inv_temperature=float(kwargs.get("inv_temperature", 1.0)),
                 grad_inplace=bool(kwargs.get("grad_inplace", False)),
-                expected_upstream=float(kwargs.get("expected_grad_scale", 1.0)))
+                expected_upstream=kwargs.get("expected_grad_scale"), scale_state=scale_state)
 
 
 # ------------------------------------------------------------------------------------ log-prob strategy
@@ -398,9 +464,17 @@ class BaseLossFunc(ABC):
 
     def __init__(self):
         self.logprob_computer = StandardLogProbComputer()
+        self._grad_scale_states = {}
 
     def add_loss_meta_info(self, meta_info: Dict):
         pass
+
+    def grad_scale_state(self, device) -> GradScaleState:
+        """This object's learned upstream gradient scale on ``device`` (created on first use)."""
+        key = torch.device(device)
+        if key not in self._grad_scale_states:
+            self._grad_scale_states[key] = GradScaleState(key)
+        return self._grad_scale_states[key]
 
     @abstractmethod
     def compute_loss(self, output: torch.Tensor, batch: Dict[str, torch.Tensor], forward_only=False,
@@ -487,7 +561,8 @@ class GRPOActorLossFunc(BaseLossFunc):
                 output, batch, ref_log_prob=batch.get("ref_log_prob"), clip_low=self.clip_ratio,
                 clip_high=self.clip_ratio, kl_penalty=self.kl_penalty, kl_coef=self.kl_ctrl.value,
                 entropy_coeff=self.entropy_coeff, token_level_loss=True,
-                loss_scale=_dynamic_scale(batch, forward_only, kwargs), **_fused_kwargs(kwargs))
+                loss_scale=_dynamic_scale(batch, forward_only, kwargs),
+                **_fused_kwargs(kwargs, self.grad_scale_state(output.device)))
             return _finish(loss, out)
         log_probs, entropy = super().compute_log_probs(output=output, batch=batch,
                                                        skip_entropy=(self.entropy_coeff == 0), **kwargs)
@@ -552,7 +627,8 @@ class DAPOActorLossFunc(BaseLossFunc):
             loss, out = fused_logprob_policy_loss(
                 output, batch, mask=mask, clip_low=self.clip_ratio_low, clip_high=self.clip_ratio_high,
                 kl_penalty=None, entropy_coeff=self.entropy_coeff, token_level_loss=self.token_level_loss,
-                loss_scale=_dynamic_scale(batch, forward_only, kwargs), **_fused_kwargs(kwargs))
+                loss_scale=_dynamic_scale(batch, forward_only, kwargs),
+                **_fused_kwargs(kwargs, self.grad_scale_state(output.device)))
             return _finish(loss, out)
         log_probs, entropy = super().compute_log_probs(output=output, batch=batch,
                                                        skip_entropy=(self.entropy_coeff == 0), **kwargs)
@@ -612,7 +688,8 @@ class PPOActorLossFunc(BaseLossFunc):
                       entropy_coeff=self.entropy_coeff, token_level_loss=True,
                       loss_scale=_dynamic_scale(batch, forward_only, kwargs))
         if self._fused(output, kwargs):
-            loss, out = fused_logprob_policy_loss(output, batch, **common, **_fused_kwargs(kwargs))
+            loss, out = fused_logprob_policy_loss(output, batch, **common,
+                                                  **_fused_kwargs(kwargs, self.grad_scale_state(output.device)))
         else:
             log_probs, entropy = super().compute_log_probs(output=output, batch=batch,
                                                            skip_entropy=(self.entropy_coeff == 0), **kwargs)

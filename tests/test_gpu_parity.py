@@ -1320,11 +1320,11 @@ def test_bandwidth_probes_touch_exactly_their_range(dev):
         assert (sink == 7).all().item()
 
 
-def _raw_fused_sweep(z, y, row_ops, dz, ent, terms, stream):
+def _raw_fused_sweep(z, y, row_ops, dz, ent, terms, stream, ticket=None, scale_dev=None):
     rows, vocab = z.shape
     _lib.call("mrl_fused_logprob_loss", z.data_ptr(), _lib.dtype_code(z), rows, vocab, vocab, y.data_ptr(), _lib.I64,
-              1.0, row_ops.data_ptr(), 1, 0.8, 1.2, 3, 0.01, 0.002, 1.0, dz.data_ptr(), vocab, None, ent.data_ptr(),
-              terms.data_ptr(), stream)
+              1.0, row_ops.data_ptr(), 1, 0.8, 1.2, 3, 0.01, 0.002, 1.0, _lib.ptr(scale_dev), dz.data_ptr(), vocab,
+              None, ent.data_ptr(), terms.data_ptr(), _lib.ptr(ticket), stream)
 
 
 def _raw_fused_case(dev, seed, rows, vocab):
@@ -1342,33 +1342,46 @@ def _raw_fused_case(dev, seed, rows, vocab):
 
 
 def test_fused_sweep_on_two_streams_and_in_a_graph(dev):
-    """The persistent sweep hands out rows through a counter that a launch resets on its own stream:
-    two sweeps in flight on two streams (different counters) and a captured sweep replayed several
-    times (the reset is a kernel, so it is part of the graph) give the results of a lone eager call,
-    bit for bit - every row's result is independent of the order in which rows are taken."""
+    """The persistent sweep hands out rows through a counter that the caller owns and that a launch
+    resets on its own stream: two sweeps in flight on two streams (a counter each), a sweep without a
+    counter (fixed row stride) and a captured sweep replayed several times next to eager sweeps (the
+    reset is a kernel, so it is part of the graph, and the graph keeps its own counter) give the
+    results of a lone eager call, bit for bit - every row's result is independent of the order in
+    which rows are taken."""
     rows, vocab = 1500, 8200
     cases = [_raw_fused_case(dev, 50 + i, rows, vocab) for i in range(2)]
+    tickets = [torch.full((1,), 12345, dtype=torch.int32, device=dev) for _ in range(3)]
     want = []
     for z, y, ops in cases:
         dz, ent, terms = torch.empty_like(z), torch.empty(rows, device=dev), torch.empty(rows, 8, device=dev)
-        _raw_fused_sweep(z, y, ops, dz, ent, terms, _lib.stream(dev))
+        _raw_fused_sweep(z, y, ops, dz, ent, terms, _lib.stream(dev), tickets[0])
         torch.cuda.synchronize()
         want.append((dz, ent, terms))
         assert dz.float().abs().max().item() > 0 and not dz[ops[:, 3] == 0].any().item()
+        # every row was handed out exactly once: the counter ends at rows + workgroups
+        cus = torch.cuda.get_device_properties(dev).multi_processor_count
+        assert int(tickets[0].item()) == rows + cus
+    # no counter: rows are walked with a fixed stride
+    z, y, ops = cases[0]
+    plain = (torch.empty_like(z), torch.empty(rows, device=dev), torch.empty(rows, 8, device=dev))
+    _raw_fused_sweep(z, y, ops, *plain, _lib.stream(dev), None)
+    torch.cuda.synchronize()
+    for a, b in zip(plain, want[0]):
+        assert torch.equal(a, b)
     # two streams at once, several rounds
     streams = [torch.cuda.Stream(device=dev) for _ in cases]
     outs = [(torch.empty_like(c[0]), torch.empty(rows, device=dev), torch.empty(rows, 8, device=dev)) for c in cases]
     torch.cuda.synchronize()
     for _ in range(4):
-        for (z, y, ops), (dz, ent, terms), s in zip(cases, outs, streams):
-            _raw_fused_sweep(z, y, ops, dz, ent, terms, s.cuda_stream)
+        for (z, y, ops), (dz, ent, terms), s, t in zip(cases, outs, streams, tickets):
+            _raw_fused_sweep(z, y, ops, dz, ent, terms, s.cuda_stream, t)
     torch.cuda.synchronize()
     for got, ref in zip(outs, want):
         for a, b in zip(got, ref):
             assert torch.equal(a, b)
-    # more launches than the library has counters: the slots are reused round-robin
+    # many launches in a row on one stream may share one counter (each resets it behind the previous sweep)
     for _ in range(300):
-        _raw_fused_sweep(cases[0][0], cases[0][1], cases[0][2], *outs[0], _lib.stream(dev))
+        _raw_fused_sweep(cases[0][0], cases[0][1], cases[0][2], *outs[0], _lib.stream(dev), tickets[0])
     torch.cuda.synchronize()
     for a, b in zip(outs[0], want[0]):
         assert torch.equal(a, b)
@@ -1377,14 +1390,17 @@ def test_fused_sweep_on_two_streams_and_in_a_graph(dev):
     dz, ent, terms = torch.zeros_like(z), torch.zeros(rows, device=dev), torch.zeros(rows, 8, device=dev)
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        _raw_fused_sweep(z, y, ops, dz, ent, terms, _lib.stream(dev))
+        _raw_fused_sweep(z, y, ops, dz, ent, terms, _lib.stream(dev), tickets[2])
+    side = torch.cuda.Stream(device=dev)
     for i in range(3):
         dz.zero_()
         ent.zero_()
         terms.zero_()
         other = torch.empty_like(cases[1][0])
-        _raw_fused_sweep(cases[1][0], cases[1][1], cases[1][2], other, torch.empty(rows, device=dev),
-                         torch.empty(rows, 8, device=dev), _lib.stream(dev))      # eager sweep between replays
+        o_ent, o_terms = torch.empty(rows, device=dev), torch.empty(rows, 8, device=dev)
+        torch.cuda.synchronize()
+        # an eager sweep on another stream runs next to the replay, with a counter of its own
+        _raw_fused_sweep(cases[1][0], cases[1][1], cases[1][2], other, o_ent, o_terms, side.cuda_stream, tickets[1])
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(dz, want[0][0]) and torch.equal(ent, want[0][1]) and torch.equal(terms, want[0][2]), i
@@ -1500,10 +1516,12 @@ def _random_fused_case(i, rnd):
     ent = torch.zeros(rows, device=dev)
     lp = torch.zeros(rows, device=dev)
     terms = torch.zeros(rows, 8, device=dev)
+    ticket = torch.zeros(1, dtype=torch.int32, device=dev)         # every other case walks rows with a fixed stride
     clip_lo, clip_hi, kl_kind, kl_coef = 0.8, 1.25, 4, 0.01
     _lib.call("mrl_fused_logprob_loss", z.data_ptr(), _lib.dtype_code(z), rows, vocab, vocab, y.data_ptr(), _lib.I64,
-              inv_t, ops.data_ptr(), 1, clip_lo, clip_hi, kl_kind, kl_coef, ent_c, 1.0, dz.data_ptr(), vocab,
-              lp.data_ptr(), ent.data_ptr() if ent_c != 0 else None, terms.data_ptr(), _lib.stream(dev))
+              inv_t, ops.data_ptr(), 1, clip_lo, clip_hi, kl_kind, kl_coef, ent_c, 1.0, None, dz.data_ptr(), vocab,
+              lp.data_ptr(), ent.data_ptr() if ent_c != 0 else None, terms.data_ptr(),
+              ticket.data_ptr() if i % 2 == 0 else None, _lib.stream(dev))
     zr = (z.float() * inv_t).requires_grad_()
     logsm = torch.log_softmax(zr, -1)
     y_ok = (y >= 0) & (y < vocab)
@@ -2191,20 +2209,7 @@ def test_one_loss_object_over_interleaved_micro_batches(dev, fused):
     """A pipeline schedule runs the forward of several micro-batches of different shapes through ONE
     loss object and their backwards later, in another order: every loss and gradient equals the
     oracle's for its own micro-batch (nothing is shared between calls)."""
-    def micro_batch(seed, n_seq, seq_len, vocab):
-        g = torch.Generator().manual_seed(seed)
-        plen = torch.randint(1, 5, (n_seq, 1), generator=g)
-        rlen = torch.randint(1, seq_len - 5, (n_seq, 1), generator=g)
-        resp_w = int(rlen.max())
-        ids = torch.randint(0, vocab, (n_seq, seq_len), generator=g)
-        rmask = o_pack.generate_mask(torch.zeros(n_seq, resp_w), rlen)
-        b = {"labels": torch.roll(ids, -1, 1), "responses": torch.zeros(n_seq, resp_w, dtype=torch.int64),
-             "response_length": rlen, "prompt_length": plen,
-             "advantages": torch.randn(n_seq, resp_w, generator=g) * rmask,
-             "old_log_prob": -torch.rand(n_seq, resp_w, generator=g) * rmask * 3,
-             "ref_log_prob": -torch.rand(n_seq, resp_w, generator=g) * rmask * 3}
-        return torch.randn(n_seq, seq_len, vocab, generator=g) * 2, b
-
+    micro_batch = _small_padded_micro_batch
     meta = dict(clip_ratio=0.2, kl_coef=0.01, kl_penalty="low_var_kl", entropy_coeff=0.001)
     items = [micro_batch(1, 4, 30, 512), micro_batch(2, 7, 19, 1032), micro_batch(3, 2, 40, 256)]
     want = []
@@ -2228,6 +2233,115 @@ def test_one_loss_object_over_interleaved_micro_batches(dev, fused):
         for i in range(3):
             assert losses[i].item() == pytest.approx(want[i][0], rel=TOL_LOSS_REL, abs=1e-7)
             assert (leaves[i].grad.cpu() - want[i][1]).abs().max().item() < 1e-6
+
+
+def _small_padded_micro_batch(seed, n_seq, seq_len, vocab):
+    g = torch.Generator().manual_seed(seed)
+    plen = torch.randint(1, 5, (n_seq, 1), generator=g)
+    rlen = torch.randint(1, seq_len - 5, (n_seq, 1), generator=g)
+    resp_w = int(rlen.max())
+    ids = torch.randint(0, vocab, (n_seq, seq_len), generator=g)
+    rmask = o_pack.generate_mask(torch.zeros(n_seq, resp_w), rlen)
+    b = {"labels": torch.roll(ids, -1, 1), "responses": torch.zeros(n_seq, resp_w, dtype=torch.int64),
+         "response_length": rlen, "prompt_length": plen,
+         "advantages": torch.randn(n_seq, resp_w, generator=g) * rmask,
+         "old_log_prob": -torch.rand(n_seq, resp_w, generator=g) * rmask * 3,
+         "ref_log_prob": -torch.rand(n_seq, resp_w, generator=g) * rmask * 3}
+    return torch.randn(n_seq, seq_len, vocab, generator=g) * 2, b
+
+
+def test_upstream_scale_is_learned_across_micro_batches(dev):
+    """What the reference's caller does (models/base/base_training_engine.py:238-270): one loss object,
+    n micro-batches, and the schedule back-propagates loss / n without telling the loss function.
+    The fused sweep writes its gradients with the scale of the previous backward, so only the first
+    micro-batch pays a rescale pass; every gradient equals the oracle's.  A change of the scale (a
+    new number of micro-batches, a new loss scale) costs one more rescale, never a wrong gradient."""
+    meta = dict(clip_ratio=0.2, kl_coef=0.01, kl_penalty="low_var_kl", entropy_coeff=0.001)
+    f = mrl.GRPOActorLossFunc()
+    f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.01), "kl_penalty": "low_var_kl",
+                          "entropy_coeff": 0.001})
+    state = f.grad_scale_state(dev)
+    assert state is f.grad_scale_state(dev) and state.learned.item() == 1.0 and state.rescales.item() == 0
+    plan = [(0.25, 4), (0.5, 2), (1.0 / 3.0, 3)]                # (upstream, micro-batches); 1/3 is not a power of two
+    expected_rescales, seed = 0, 100
+    for upstream, n_micro in plan:
+        expected_rescales += 1
+        for _ in range(n_micro):
+            seed += 1
+            z, b = _small_padded_micro_batch(seed, 3 + seed % 3, 24, 520)
+            zo = z.clone().requires_grad_()
+            loss_o, _ = o_loss.grpo_compute_loss(zo, b, meta)
+            (g_o,) = torch.autograd.grad(loss_o * upstream, zo)
+            zd = z.to(dev).requires_grad_()
+            loss, _ = f.compute_loss(zd, _to_dev(b, dev), fused=True)
+            (loss * upstream).backward()
+            assert loss.item() == pytest.approx(loss_o.item(), rel=TOL_LOSS_REL, abs=1e-7)
+            assert (zd.grad.cpu() - g_o).abs().max().item() < 1e-6
+            assert state.rescales.item() == expected_rescales
+            assert state.learned.item() == torch.tensor(upstream, dtype=torch.float32).item()
+    # an upstream gradient that cannot be a scale (0, inf, NaN) is honoured but not learned
+    z, b = _small_padded_micro_batch(7, 3, 24, 520)
+    zd = z.to(dev).requires_grad_()
+    loss, _ = f.compute_loss(zd, _to_dev(b, dev), fused=True)
+    (loss * 0.0).backward()
+    assert not zd.grad.any().item() and state.learned.item() == torch.tensor(1.0 / 3.0).item()
+    # an explicit expected_grad_scale bypasses the learned one
+    zd = z.to(dev).requires_grad_()
+    before = state.rescales.item()
+    loss, _ = f.compute_loss(zd, _to_dev(b, dev), fused=True, expected_grad_scale=0.125)
+    (loss * 0.125).backward()
+    assert state.rescales.item() == before
+    zo = z.clone().requires_grad_()
+    (g_o,) = torch.autograd.grad(o_loss.grpo_compute_loss(zo, b, meta)[0] * 0.125, zo)
+    assert (zd.grad.cpu() - g_o).abs().max().item() < 1e-6
+
+
+@pytest.mark.parametrize("kind", ["logits", "lmhead"])
+def test_two_backwards_over_one_retained_graph(dev, kind):
+    """retain_graph=True: the second backward must not multiply the stored gradient by its upstream
+    ratio a second time, and must leave the tensor the first backward handed out untouched."""
+    meta = dict(clip_ratio=0.2, kl_coef=0.01, kl_penalty="low_var_kl", entropy_coeff=0.001)
+    z, b = _small_padded_micro_batch(11, 4, 24, 520)
+    bd = _to_dev(b, dev)
+    if kind == "logits":
+        # the oracle's cross entropy works in place like Megatron's and cannot be back-propagated twice:
+        # one fresh graph per upstream value
+        want = []
+        for u in (0.5, 0.3, 0.5):
+            zo = z.clone().requires_grad_()
+            want.append(torch.autograd.grad(o_loss.grpo_compute_loss(zo, b, meta)[0] * u, zo))
+        f = mrl.GRPOActorLossFunc()
+        f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.01), "kl_penalty": "low_var_kl",
+                              "entropy_coeff": 0.001})
+        leaves = (z.to(dev).requires_grad_(),)
+        loss, _ = f.compute_loss(leaves[0], bd, fused=True)
+        tol = 1e-6
+    else:
+        g = torch.Generator().manual_seed(5)
+        hdim = 64
+        h = torch.randn(z.shape[0], z.shape[1], hdim, generator=g).to(torch.bfloat16)
+        w = (torch.randn(520, hdim, generator=g) * 0.3).to(torch.bfloat16)
+        want = []
+        for u in (0.5, 0.3, 0.5):
+            ho, wo = h.float().requires_grad_(), w.float().requires_grad_()
+            loss_o, _ = o_loss.grpo_compute_loss(torch.nn.functional.linear(ho, wo).to(torch.bfloat16).float(), b, meta)
+            want.append(torch.autograd.grad(loss_o * u, [ho, wo]))
+        leaves = (h.to(dev).requires_grad_(), w.to(dev).requires_grad_())
+        loss, _ = mrl.fused_lmhead_policy_loss(leaves[0], leaves[1], bd, packed=False, ref_log_prob=bd["ref_log_prob"],
+                                               clip_low=0.2, clip_high=0.2, kl_penalty="low_var_kl", kl_coef=0.01,
+                                               entropy_coeff=0.001)
+        tol = None
+    got = []
+    for i, u in enumerate((0.5, 0.3, 0.5)):
+        got.append(torch.autograd.grad(loss * u, leaves, retain_graph=(i < 2)))
+    torch.cuda.synchronize()
+    for grads, refs in zip(got, want):
+        for a, r in zip(grads, refs):
+            bound = tol if tol is not None else 2e-2 * r.abs().max().item()
+            assert (a.float().cpu() - r).abs().max().item() <= bound
+    # the first and the third backward had the same upstream value: identical results, separate storage
+    for a, c in zip(got[0], got[2]):
+        assert a.data_ptr() != c.data_ptr() and torch.equal(a, c)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

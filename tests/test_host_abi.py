@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), "libmrl_hip.so lacks %s" % name
     # and the ctypes table binds exactly the declared set
     assert sorted(_lib.SIGNATURES) == declared
-    assert lib.mrl_version() == 100
+    assert lib.mrl_version() == 200
     assert lib.mrl_last_error() == b""
     assert os.path.dirname(_lib.library_path()).startswith(ROOT), "the library must live in-tree"
 
@@ -103,11 +103,15 @@ def test_argument_validation_launches_nothing():
     assert lib.mrl_fused_max_vocab(_lib.BF16) == 155648 and lib.mrl_fused_max_vocab(_lib.I64) == 0
     for vocab in (155656, 1003):
         rc = lib.mrl_fused_logprob_loss(p, _lib.BF16, 2, vocab, vocab, p, _lib.I64, 1.0, p, 1, 0.8, 1.2, 4, 0.0, 0.0,
-                                        1.0, p, vocab, None, None, p, None)
+                                        1.0, None, p, vocab, None, None, p, None, None)
         assert rc == -2, vocab
     assert lib.mrl_fused_logprob_loss(p, _lib.BF16, 2, 64, 64, p, _lib.I64, 1.0, None, 1, 0.8, 1.2, 4, 0.0, 0.0, 1.0,
-                                      p, 64, None, None, p, None) == -1                   # no row operands
-    assert lib.mrl_scale_rows(p, _lib.I32, 2, 64, 64, p, 1.0, None) == -2
+                                      None, p, 64, None, None, p, None, None) == -1       # no row operands
+    assert lib.mrl_fused_logprob_loss(p, _lib.BF16, 2, 64, 64, p, _lib.I64, 1.0, p, 1, 0.8, 1.2, 4, 0.0, 0.0, 1.0,
+                                      None, p, 64, None, None, p, p + 2, None) == -3      # misaligned row counter
+    assert lib.mrl_scale_rows(p, _lib.I32, 2, 64, 64, p, p, None) == -2
+    assert lib.mrl_scale_rows(p, _lib.BF16, 2, 64, 64, p, None, None) == -1                # no applied scale
+    assert lib.mrl_grad_scale_note(p, None, None, None, None) == -1
     # fused lm_head: hidden size must be a multiple of the K tile, workspace must be large enough
     assert lib.mrl_lmhead_workspace_bytes(100, 1000) > 0
     assert lib.mrl_lmhead_logprob_fwd(p, p, 4, 1000, 100, p, _lib.I64, 1.0, p, None, None, p, 1 << 20, None) != 0
