@@ -372,6 +372,22 @@ int mrl_lmhead_logprob_fwd(const void* hidden, const void* weight, int64_t n_tok
                            float inv_temperature, float* logp, float* entropy, float* lse,
                            void* workspace, int64_t workspace_bytes, void* stream);
 
+/* mrl_lmhead_logprob_fwd for callers that cannot allocate device memory or pass a workspace (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in
+ * the reference.  Same arguments, kernels and results as mrl_lmhead_logprob_fwd, but the partial
+ * statistics live in a static device array of the library (8 MiB per GPU that runs it, looked up
+ * once per device with hipGetSymbolAddress and held until the process ends), so at most
+ * mrl_lmhead_static_max_tokens() = 65536 tokens per call: more is rejected with
+ * MRL_ERR_UNSUPPORTED (slice the tokens).  Calls nothing that allocates or frees.  Every call on a
+ * GPU shares that GPU's array: calls that overlap in time on one GPU (two streams, two threads)
+ * race and give wrong results - serialise them.  The array needs no clearing between calls: every
+ * entry a call reads was written by that call. */
+int64_t mrl_lmhead_static_max_tokens(void);
+int mrl_lmhead_logprob_fwd_static(const void* hidden, const void* weight, int64_t n_tokens,
+                                  int64_t vocab, int64_t hidden_dim, const void* labels,
+                                  int labels_dtype, float inv_temperature, float* logp,
+                                  float* entropy, float* lse, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * PPO's value side (the "next" row after the actor path): rewards with the KL penalty, GAE,
  * whitening and the critic's clipped value loss.  All tensors [batch, width] fp32, contiguous.

@@ -17,8 +17,16 @@
 // second kernel merges, together with the label logit (one fp32 dot product per token).
 #include <stdlib.h>
 
+#include <atomic>
+
 #include "mrl_internal.h"
 #include "vocab_common.h"
+
+// Partial statistics of mrl_lmhead_logprob_fwd_static: device memory that belongs to the library,
+// one copy per GPU that runs it, held until the process ends.  In host code this name is only a
+// handle for hipGetSymbolAddress; kernels get the address that call returns.
+#define MRL_LMHEAD_STATIC_MAX_TOKENS 65536
+static __device__ __align__(256) float scratch[(size_t)MRL_LMHEAD_GROUPS * MRL_LMHEAD_STATIC_MAX_TOKENS * 4];
 
 namespace {
 
@@ -497,33 +505,14 @@ extern "C" int64_t mrl_lmhead_workspace_bytes(int64_t n_tokens, int64_t vocab) {
     return (int64_t)MRL_LMHEAD_GROUPS * n_tokens * 4 * (int64_t)sizeof(float);
 }
 
-extern "C" int mrl_lmhead_logprob_fwd(const void* hidden, const void* weight, int64_t n_tokens, int64_t vocab,
-                                      int64_t hidden_dim, const void* labels, int labels_dtype,
-                                      float inv_temperature, float* logp, float* entropy, float* lse,
-                                      void* workspace, int64_t workspace_bytes, void* stream) {
-    const char* fn = "mrl_lmhead_logprob_fwd";
-    MRL_REQUIRE(n_tokens >= 0 && vocab > 0 && hidden_dim > 0, MRL_ERR_INVALID_ARG,
-                "%s: n_tokens=%lld vocab=%lld hidden_dim=%lld", fn, (long long)n_tokens, (long long)vocab,
-                (long long)hidden_dim);
-    MRL_REQUIRE(hidden_dim % BK == 0, MRL_ERR_UNSUPPORTED, "%s: hidden_dim=%lld must be a multiple of %d", fn,
-                (long long)hidden_dim, BK);
-    MRL_REQUIRE(vocab <= (1LL << 30) && hidden_dim <= (1LL << 20), MRL_ERR_UNSUPPORTED, "%s: size out of range", fn);
-    MRL_REQUIRE(mrl::int_dtype_bytes(labels_dtype) != 0, MRL_ERR_UNSUPPORTED, "%s: labels dtype %d (want I32 or I64)",
-                fn, labels_dtype);
-    MRL_REQUIRE(inv_temperature > 0.f && inv_temperature < 1.0e6f, MRL_ERR_INVALID_ARG,
-                "%s: inv_temperature=%g must be in (0, 1e6)", fn, (double)inv_temperature);
-    if (n_tokens == 0) return MRL_OK;
-    MRL_REQUIRE(hidden && weight && labels && logp && workspace, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
-    MRL_REQUIRE(mrl::aligned(hidden, 16) && mrl::aligned(weight, 16) && mrl::aligned(workspace, 16), MRL_ERR_MISALIGNED,
-                "%s: hidden, weight and workspace must be 16-byte aligned", fn);
-    MRL_REQUIRE(workspace_bytes >= mrl_lmhead_workspace_bytes(n_tokens, vocab), MRL_ERR_INVALID_ARG,
-                "%s: workspace of %lld bytes, need %lld", fn, (long long)workspace_bytes,
-                (long long)mrl_lmhead_workspace_bytes(n_tokens, vocab));
+// Checks and launches shared by the two forward entry points; `partial` holds
+// mrl_lmhead_workspace_bytes(n_tokens, vocab) bytes.
+static int lmhead_forward(const char* fn, const void* hidden, const void* weight, int64_t n_tokens, int64_t vocab,
+                          int64_t hidden_dim, const void* labels, int labels_dtype, float inv_temperature, float* logp,
+                          float* entropy, float* lse, float* partial, hipStream_t s) {
     const int n_groups = MRL_LMHEAD_GROUPS;
     const int n_vtiles = (int)((vocab + BV - 1) / BV);
     const int tiles_per_group = (n_vtiles + n_groups - 1) / n_groups;
-    hipStream_t s = mrl::as_stream(stream);
-    float* partial = (float*)workspace;
     // a group without tiles (tiny vocabularies) still writes its neutral partials
     // the second-generation loop addresses the weights with 32-bit byte offsets
     if (lmhead_v2_enabled() && vocab * hidden_dim * 2 < (1LL << 32)) {
@@ -561,4 +550,77 @@ extern "C" int mrl_lmhead_logprob_fwd(const void* hidden, const void* weight, in
                            (int)hidden_dim, n_groups, inv_temperature, logp, entropy, lse);
     }
     return mrl::check_launch(fn);
+}
+
+#define MRL_LMHEAD_CHECK_ARGS(fn)                                                                                      \
+    MRL_REQUIRE(n_tokens >= 0 && vocab > 0 && hidden_dim > 0, MRL_ERR_INVALID_ARG,                                     \
+                "%s: n_tokens=%lld vocab=%lld hidden_dim=%lld", fn, (long long)n_tokens, (long long)vocab,             \
+                (long long)hidden_dim);                                                                                \
+    MRL_REQUIRE(hidden_dim % BK == 0, MRL_ERR_UNSUPPORTED, "%s: hidden_dim=%lld must be a multiple of %d", fn,         \
+                (long long)hidden_dim, BK);                                                                            \
+    MRL_REQUIRE(vocab <= (1LL << 30) && hidden_dim <= (1LL << 20), MRL_ERR_UNSUPPORTED, "%s: size out of range", fn);  \
+    MRL_REQUIRE(mrl::int_dtype_bytes(labels_dtype) != 0, MRL_ERR_UNSUPPORTED, "%s: labels dtype %d (want I32 or I64)", \
+                fn, labels_dtype);                                                                                     \
+    MRL_REQUIRE(inv_temperature > 0.f && inv_temperature < 1.0e6f, MRL_ERR_INVALID_ARG,                                \
+                "%s: inv_temperature=%g must be in (0, 1e6)", fn, (double)inv_temperature)
+
+extern "C" int mrl_lmhead_logprob_fwd(const void* hidden, const void* weight, int64_t n_tokens, int64_t vocab,
+                                      int64_t hidden_dim, const void* labels, int labels_dtype,
+                                      float inv_temperature, float* logp, float* entropy, float* lse,
+                                      void* workspace, int64_t workspace_bytes, void* stream) {
+    const char* fn = "mrl_lmhead_logprob_fwd";
+    MRL_LMHEAD_CHECK_ARGS(fn);
+    if (n_tokens == 0) return MRL_OK;
+    MRL_REQUIRE(hidden && weight && labels && logp && workspace, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+    MRL_REQUIRE(mrl::aligned(hidden, 16) && mrl::aligned(weight, 16) && mrl::aligned(workspace, 16), MRL_ERR_MISALIGNED,
+                "%s: hidden, weight and workspace must be 16-byte aligned", fn);
+    MRL_REQUIRE(workspace_bytes >= mrl_lmhead_workspace_bytes(n_tokens, vocab), MRL_ERR_INVALID_ARG,
+                "%s: workspace of %lld bytes, need %lld", fn, (long long)workspace_bytes,
+                (long long)mrl_lmhead_workspace_bytes(n_tokens, vocab));
+    return lmhead_forward(fn, hidden, weight, n_tokens, vocab, hidden_dim, labels, labels_dtype, inv_temperature, logp,
+                          entropy, lse, (float*)workspace, mrl::as_stream(stream));
+}
+
+// Address of `scratch` on the current device, looked up once per device (each GPU holds its own
+// copy of the array at its own address).  NULL and an error message if the lookup fails.
+static float* static_scratch(const char* fn) {
+    constexpr int kMaxDevices = 64;
+    static std::atomic<float*> known[kMaxDevices];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        mrl::fail(MRL_ERR_LAUNCH, "%s: no current device (hipGetDevice gave %d)", fn, dev);
+        return nullptr;
+    }
+    float* p = known[dev].load(std::memory_order_acquire);
+    if (p) return p;
+    void* addr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || addr == nullptr) {
+        mrl::fail(MRL_ERR_LAUNCH, "%s: hipGetSymbolAddress(scratch) on device %d: %s", fn, dev, hipGetErrorString(e));
+        return nullptr;
+    }
+    known[dev].store((float*)addr, std::memory_order_release);
+    return (float*)addr;
+}
+
+extern "C" int64_t mrl_lmhead_static_max_tokens(void) { return MRL_LMHEAD_STATIC_MAX_TOKENS; }
+
+extern "C" int mrl_lmhead_logprob_fwd_static(const void* hidden, const void* weight, int64_t n_tokens, int64_t vocab,
+                                             int64_t hidden_dim, const void* labels, int labels_dtype,
+                                             float inv_temperature, float* logp, float* entropy, float* lse,
+                                             void* stream) {
+    const char* fn = "mrl_lmhead_logprob_fwd_static";
+    MRL_LMHEAD_CHECK_ARGS(fn);
+    MRL_REQUIRE(n_tokens <= MRL_LMHEAD_STATIC_MAX_TOKENS, MRL_ERR_UNSUPPORTED,
+                "%s: n_tokens=%lld exceeds the %d tokens the library's own scratch memory holds; call it on slices of "
+                "at most that many tokens, or use mrl_lmhead_logprob_fwd with a workspace",
+                fn, (long long)n_tokens, MRL_LMHEAD_STATIC_MAX_TOKENS);
+    if (n_tokens == 0) return MRL_OK;
+    MRL_REQUIRE(hidden && weight && labels && logp, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+    MRL_REQUIRE(mrl::aligned(hidden, 16) && mrl::aligned(weight, 16), MRL_ERR_MISALIGNED,
+                "%s: hidden and weight must be 16-byte aligned", fn);
+    float* partial = static_scratch(fn);
+    if (!partial) return MRL_ERR_LAUNCH;
+    return lmhead_forward(fn, hidden, weight, n_tokens, vocab, hidden_dim, labels, labels_dtype, inv_temperature, logp,
+                          entropy, lse, partial, mrl::as_stream(stream));
 }
