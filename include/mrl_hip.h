@@ -405,11 +405,13 @@ int mrl_kl_token_rewards(const float* old_log_prob, const float* ref_log_prob,
 
 /* mrl_gae_scan: the reverse scan of compute_gae_advantage_return (compute_utils.py:134-145), before
  * its whitening: delta_t = rewards[t] + gamma * values[t+1] - values[t] (values[width] = 0),
- * lastgaelam = delta_t + (gamma * lam) * lastgaelam, advantages[t] = lastgaelam, returns =
- * advantages + values.  fp32 with the reference's operation order and roundings: bit-identical to
- * the torch loop.  Outputs must not alias the inputs. */
+ * lastgaelam = delta_t + gamma_lam * lastgaelam, advantages[t] = lastgaelam, returns =
+ * advantages + values.  gamma_lam is the product gamma * lam formed in DOUBLE and rounded to fp32
+ * once (python evaluates `gamma * lam` first, torch then rounds the scalar); gamma is rounded on its
+ * own.  fp32 with the reference's operation order and roundings: bit-identical to the torch loop.
+ * Outputs must not alias the inputs. */
 int mrl_gae_scan(const float* rewards, const float* values, int64_t batch, int64_t width, float gamma,
-                 float lam, float* advantages, float* returns, void* stream);
+                 float gamma_lam, float* advantages, float* returns, void* stream);
 
 /* mrl_masked_whiten: masked_whiten / masked_var / masked_mean (mindspeed_rl/utils/
  * torch_functional.py:46-106) over n entries: mean = sum(x*mask)/(sum(mask)+1e-8), var the same of

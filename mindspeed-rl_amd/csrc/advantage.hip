@@ -1,7 +1,8 @@
 // Group-relative advantage normalisation and the DAPO group filter for gfx950.
 //
 // Both are O(batch) scalar work plus one [batch, width] broadcast store; they exist as kernels so
-// that the rewards never leave the device between rollout scoring and the loss.  fp64 is used
+// that the rewards never leave the device between rollout scoring and the loss.  The advantages are
+// a segmented reduction: one wavefront reduces each group of consecutive rewards with shuffles.  fp64 is used
 // where the reference uses it; the filter follows numpy's summation order exactly because its
 // result is compared with zero.
 #include "mrl_internal.h"
@@ -24,53 +25,74 @@ __device__ __forceinline__ double reward_at(const void* p, int dtype, int64_t i)
                             : (double) reinterpret_cast<const float*>(p)[i];
 }
 
-// One workgroup per row: lane 0 normalises the row's reward inside its group (two passes in
-// fp64, unbiased variance), then the workgroup writes score * mask across the row.
+// Segmented reduction over one group of `group` consecutive rewards by ONE wavefront, in fp64 and in a
+// fixed order (lane l adds rewards l, l + 64, ... in sequence, then a butterfly of shuffles in which
+// both partners form the same sum): mean and unbiased standard deviation, identical in every lane.
+// All 64 lanes of the wavefront must call it.
+struct GroupMoments {
+    double mean, sd;
+};
+
+__device__ __forceinline__ double wave_sum_f64(double x) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) x += __shfl_xor(x, off, 64);
+    return x;
+}
+
+__device__ __forceinline__ GroupMoments group_moments(const void* rewards, int rdtype, int64_t g0, int64_t group) {
+    const int lane = threadIdx.x & 63;
+    double part = 0.0;
+    for (int64_t q = lane; q < group; q += 64) part += reward_at(rewards, rdtype, g0 + q);
+    GroupMoments m;
+    m.mean = wave_sum_f64(part) / (double)group;
+    part = 0.0;
+    for (int64_t q = lane; q < group; q += 64) {
+        const double d = reward_at(rewards, rdtype, g0 + q) - m.mean;
+        part += d * d;
+    }
+    m.sd = sqrt(wave_sum_f64(part) / (double)(group - 1));   // group == 1: 0/0 = NaN, like torch.std
+    return m;
+}
+
+// One workgroup per GROUP: its first wavefront reduces the group's rewards (above), then the four
+// wavefronts share the group's rows and write score * mask across each of them.
 __global__ __launch_bounds__(kBlock) void group_advantage_kernel(const void* __restrict__ rewards, int rdtype,
                                                                  int64_t group, const void* __restrict__ mask,
                                                                  int mdtype, int64_t width,
                                                                  float* __restrict__ adv, float* __restrict__ ret) {
-    __shared__ float score_s;
-    const int64_t i = blockIdx.x;
-    if (threadIdx.x == 0) {
-        const int64_t g0 = (i / group) * group;
-        double sum = 0.0;
-        for (int64_t q = 0; q < group; ++q) sum += reward_at(rewards, rdtype, g0 + q);
-        const double mean = sum / (double)group;
-        double ss = 0.0;
-        for (int64_t q = 0; q < group; ++q) {
-            const double d = reward_at(rewards, rdtype, g0 + q) - mean;
-            ss += d * d;
+    __shared__ double moments_s[2];
+    const int64_t g0 = (int64_t)blockIdx.x * group;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (wave == 0) {
+        const GroupMoments m = group_moments(rewards, rdtype, g0, group);
+        if (lane == 0) {
+            moments_s[0] = m.mean;
+            moments_s[1] = m.sd;
         }
-        const double sd = sqrt(ss / (double)(group - 1));   // group == 1: 0/0 = NaN, like torch.std
-        score_s = (float)((reward_at(rewards, rdtype, i) - mean) / (sd + 1e-6));
     }
     __syncthreads();
-    const float score = score_s;
-    for (int64_t j = threadIdx.x; j < width; j += kBlock) {
-        const float v = score * mask_as_float(mask, mdtype, i * width + j);
-        adv[i * width + j] = v;
-        if (ret) ret[i * width + j] = v;
+    const double mean = moments_s[0], sd = moments_s[1];
+    for (int64_t q = wave; q < group; q += kBlock / 64) {
+        const int64_t i = g0 + q;
+        const float score = (float)((reward_at(rewards, rdtype, i) - mean) / (sd + 1e-6));
+        for (int64_t j = lane; j < width; j += 64) {
+            const float v = score * mask_as_float(mask, mdtype, i * width + j);
+            adv[i * width + j] = v;
+            if (ret) ret[i * width + j] = v;
+        }
     }
 }
 
-// One thread per reward: (r - mean) / (unbiased std + eps) inside its group, fp64 internally.
+// One wavefront per group (four groups per workgroup): (r - mean) / (unbiased std + eps), fp64 internally.
 __global__ __launch_bounds__(kBlock) void group_standardize_kernel(const void* __restrict__ rewards, int rdtype,
-                                                                   int64_t n, int64_t group, double eps,
+                                                                   int64_t n_groups, int64_t group, double eps,
                                                                    float* __restrict__ out) {
-    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (i >= n) return;
-    const int64_t g0 = (i / group) * group;
-    double sum = 0.0;
-    for (int64_t q = 0; q < group; ++q) sum += reward_at(rewards, rdtype, g0 + q);
-    const double mean = sum / (double)group;
-    double ss = 0.0;
-    for (int64_t q = 0; q < group; ++q) {
-        const double d = reward_at(rewards, rdtype, g0 + q) - mean;
-        ss += d * d;
-    }
-    const double sd = sqrt(ss / (double)(group - 1));
-    out[i] = (float)((reward_at(rewards, rdtype, i) - mean) / (sd + eps));
+    const int64_t g = (int64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+    if (g >= n_groups) return;                              // whole wavefronts leave together
+    const int64_t g0 = g * group;
+    const GroupMoments m = group_moments(rewards, rdtype, g0, group);
+    for (int64_t q = threadIdx.x & 63; q < group; q += 64)
+        out[g0 + q] = (float)((reward_at(rewards, rdtype, g0 + q) - m.mean) / (m.sd + eps));
 }
 
 // numpy's arithmetic, one correctly rounded operation at a time (no FMA contraction)
@@ -159,8 +181,8 @@ extern "C" int mrl_group_advantage(const void* rewards, int rewards_dtype, int64
                     mrl::aligned(returns, 4),
                 MRL_ERR_MISALIGNED, "%s: misaligned buffer", fn);
     if (width == 0) return MRL_OK;
-    hipLaunchKernelGGL(group_advantage_kernel, dim3((unsigned)batch), dim3(kBlock), 0, mrl::as_stream(stream), rewards,
-                       rewards_dtype, group, mask, mask_dtype, width, advantages, returns);
+    hipLaunchKernelGGL(group_advantage_kernel, dim3((unsigned)(batch / group)), dim3(kBlock), 0, mrl::as_stream(stream),
+                       rewards, rewards_dtype, group, mask, mask_dtype, width, advantages, returns);
     return mrl::check_launch(fn);
 }
 
@@ -196,8 +218,10 @@ extern "C" int mrl_group_standardize(const void* rewards, int rewards_dtype, int
                 (long long)group);
     if (n == 0) return MRL_OK;
     MRL_REQUIRE(rewards && out, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
-    const unsigned blocks = (unsigned)((n + kBlock - 1) / kBlock);
+    const int64_t n_groups = n / group;
+    MRL_REQUIRE(n_groups <= 0x7fffffffLL, MRL_ERR_UNSUPPORTED, "%s: too many groups", fn);
+    const unsigned blocks = (unsigned)((n_groups + kBlock / 64 - 1) / (kBlock / 64));
     hipLaunchKernelGGL(group_standardize_kernel, dim3(blocks), dim3(kBlock), 0, mrl::as_stream(stream), rewards,
-                       rewards_dtype, n, group, eps, out);
+                       rewards_dtype, n_groups, group, eps, out);
     return mrl::check_launch(fn);
 }

@@ -76,17 +76,17 @@ __global__ __launch_bounds__(256) void kl_rewards_kernel(const float* __restrict
 // One workgroup per sample.  The recurrence lastgaelam = delta_t + (gamma*lam) * lastgaelam is
 // evaluated by ONE thread in the reference's order and with its roundings (separate multiply and
 // add, no contraction), so advantages and returns are bit-identical to the torch loop; the other
-// threads stage the row through LDS in coalesced chunks and write the results.
+// threads stage the row through LDS in coalesced chunks and write the results.  gl is gamma*lam as
+// the host formed it: python multiplies the two in double and torch rounds the product to fp32 once.
 __global__ __launch_bounds__(kScanBlock) void gae_scan_kernel(const float* __restrict__ rewards,
                                                               const float* __restrict__ values, int64_t width,
-                                                              float gamma, float lam, float* __restrict__ adv,
+                                                              float gamma, float gl, float* __restrict__ adv,
                                                               float* __restrict__ ret) {
     __shared__ float r_s[kScanChunk];
     __shared__ float v_s[kScanChunk + 1];
     __shared__ float a_s[kScanChunk];
     __shared__ float carry;
     const int64_t base = (int64_t)blockIdx.x * width;
-    const float gl = mrl::mul_rn(gamma, lam);
     if (threadIdx.x == 0) carry = 0.f;
     for (int64_t hi = width; hi > 0; hi -= kScanChunk) {
         const int64_t lo = hi > kScanChunk ? hi - kScanChunk : 0;
@@ -264,7 +264,7 @@ extern "C" int mrl_kl_token_rewards(const float* old_log_prob, const float* ref_
 }
 
 extern "C" int mrl_gae_scan(const float* rewards, const float* values, int64_t batch, int64_t width, float gamma,
-                            float lam, float* advantages, float* returns, void* stream) {
+                            float gamma_lam, float* advantages, float* returns, void* stream) {
     const char* fn = "mrl_gae_scan";
     MRL_REQUIRE(batch >= 0 && width > 0 && batch <= 0x7fffffffLL, MRL_ERR_INVALID_ARG, "%s: batch=%lld width=%lld", fn,
                 (long long)batch, (long long)width);
@@ -274,7 +274,7 @@ extern "C" int mrl_gae_scan(const float* rewards, const float* values, int64_t b
                     advantages != returns,
                 MRL_ERR_INVALID_ARG, "%s: outputs must not alias the inputs or each other", fn);
     hipLaunchKernelGGL(gae_scan_kernel, dim3((unsigned)batch), dim3(kScanBlock), 0, mrl::as_stream(stream), rewards,
-                       values, width, gamma, lam, advantages, returns);
+                       values, width, gamma, gamma_lam, advantages, returns);
     return mrl::check_launch(fn);
 }
 

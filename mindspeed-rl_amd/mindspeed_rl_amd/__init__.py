@@ -7,7 +7,7 @@ or eager fallback.  Build the library with ``python -m mindspeed_rl_amd._build``
 from . import _lib
 from .advantage import (FixedKLController, compute_group_norm_advantage_return, dynamic_sampling_keep, get_last_reward,
                         dynamic_sampling_keep_mask)
-from .functional import clip_by_value, masked_mean, masked_sum
+from .functional import clip_by_value, is_multimodal, masked_mean, masked_sum
 from .lmhead import fused_lmhead_policy_loss, lmhead_logprob
 from .loss import (BaseLossFunc, DAPOActorLossFunc, GradScaleState, GRPOActorLossFunc, LossFuncFactory, LossRegister,
                    MultimodalLogProbComputer, PPOActorLossFunc, ReferenceLossFunc, RewardLossFunc,

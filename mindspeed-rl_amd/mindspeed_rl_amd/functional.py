@@ -1,10 +1,21 @@
-"""Masked reductions with the reference's semantics.
+"""Masked reductions with the reference's semantics, and the multimodal switch.
 
 Host-side mirror of ``masked_sum`` / ``masked_mean`` of
 ``mindspeed_rl/utils/torch_functional.py:38-59`` for callers that use them stand-alone; the
 fused policy-loss kernel has the same reductions built in and does not go through these.
 """
+import ast
+import os
+
 import torch
+
+
+def is_multimodal():
+    """Reference: ``utils/utils.py:719-720``: the process-wide switch is the environment variable
+    IS_MULTIMODAL, read as a python literal at every call (``"True"`` / ``"False"``, default False).
+    The loss objects choose their log-prob strategy by it when they are constructed and
+    ``rearrange_micro_batches`` its partitioner when it is called, as in the reference."""
+    return ast.literal_eval(os.getenv("IS_MULTIMODAL", "False"))
 
 
 def masked_sum(values, mask, axis=None):

@@ -15,6 +15,7 @@ from typing import Dict, Tuple
 import torch
 
 from . import _lib, vocab_ops
+from .functional import is_multimodal
 from .packing import (generate_mask, postprocess_packed_seqs, response_window, truncate_middle_and_pad,
                       truncate_prompt_and_pad)
 from .vocab_ops import compute_log_probs, vocab_logprob_entropy, vocab_parallel_entropy
@@ -463,7 +464,8 @@ class BaseLossFunc(ABC):
     """Reference: ``base_loss_func.py:13-57``."""
 
     def __init__(self):
-        self.logprob_computer = StandardLogProbComputer()
+        # base_loss_func.py:15
+        self.logprob_computer = MultimodalLogProbComputer() if is_multimodal() else StandardLogProbComputer()
         self._grad_scale_states = {}
 
     def add_loss_meta_info(self, meta_info: Dict):

@@ -8,13 +8,16 @@ Host-side mirror of ``mindspeed_rl/utils/seqlen_balancing.py`` (``karmarkar_karp
 the same lengths give the same micro-batches) and errors.  This is pure host logic on a few
 hundred integers; it decides the row count T of every sweep.  One data-parallel rank: the MAX
 all-reduce of the bin count is not built.  The capacity-bound bin packing the reference uses for
-multimodal batches (``balanced_bin_packing``, ``:191-307``) is selected with ``multimodal=True``
-(the reference reads a global switch).
+multimodal batches (``balanced_bin_packing``, ``:191-307``) is selected by the reference's
+process-wide switch (``is_multimodal()``, the environment variable IS_MULTIMODAL) or explicitly
+with ``multimodal=True`` / ``False``.
 """
 import heapq
 from typing import Dict, List, Tuple
 
 import torch
+
+from .functional import is_multimodal
 
 
 class _Reversed:
@@ -197,11 +200,13 @@ def _first_narrowing_move(loads, members, max_capacity):
 
 
 def rearrange_micro_batches(seqlen_list: List[int], max_token_len: int, dynamic_max_batch_size: int = None,
-                            dp_group=None, multimodal: bool = False):
+                            dp_group=None, multimodal: bool = None):
     """Micro-batches (index lists) whose token sums are balanced: the bin count comes from the
     capped greedy pass (at least ``ceil(sum / max_token_len)``, and at least
     ``ceil(n / dynamic_max_batch_size)``), the assignment from the differencing method.  With
     ``multimodal`` the capacity-bound bin packing decides both (reference ``:356-359``)."""
+    if multimodal is None:
+        multimodal = is_multimodal()
     if multimodal:
         return balanced_bin_packing(seqlen_list, max_token_len)
     if dp_group is not None:

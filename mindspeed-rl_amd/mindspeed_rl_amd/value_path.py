@@ -105,8 +105,10 @@ def compute_gae_advantage_return(token_level_rewards, values, eos_mask, gamma, l
     batch, width = rewards.shape
     adv = torch.empty_like(rewards)
     ret = torch.empty_like(rewards)
-    _lib.call("mrl_gae_scan", _lib.ptr(rewards), _lib.ptr(vals), batch, width, float(gamma), float(lam), _lib.ptr(adv),
-              _lib.ptr(ret), _lib.stream(dev))
+    # `gamma * lam` as python evaluates it inside the reference's `gamma * lam * lastgaelam`: in double
+    # for python floats (the config's values), in the tensors' own precision for 0-dim tensors
+    _lib.call("mrl_gae_scan", _lib.ptr(rewards), _lib.ptr(vals), batch, width, float(gamma), float(gamma * lam),
+              _lib.ptr(adv), _lib.ptr(ret), _lib.stream(dev))
     return masked_whiten(adv, eos_mask), ret
 
 

@@ -6,6 +6,7 @@ assignment bit-exact; logp / entropy / advantages 1e-3 abs; loss 1e-4 rel; dlogi
 The observed errors are far smaller; tighter bounds are asserted where the arithmetic allows.
 """
 import math
+import os
 
 import numpy as np
 import pytest
@@ -549,6 +550,13 @@ def test_gae_and_whitening_parity(dev, batch, width):
         assert torch.equal(ret.cpu(), want_ret)
         scale = max(1.0, want_adv.abs().max().item())
         assert (adv.cpu() - want_adv).abs().max().item() < 1e-5 * scale
+    # python floats, as the trainer passes them from its config: gamma * lam is formed in double and
+    # rounded to fp32 once (for 0.9 * 0.95, 0.95 * 0.96 and 0.98 * 0.92 that differs from the product of
+    # the two fp32-rounded factors by one unit in the last place)
+    for gamma, lam in ((0.99, 0.95), (0.9, 0.95), (0.95, 0.96), (0.98, 0.92)):
+        _, want_ret = o_adv.compute_gae_advantage_return(r, v, mask, gamma, lam)
+        _, ret = mrl.compute_gae_advantage_return(r.to(dev), v.to(dev), mask.to(dev), gamma, lam)
+        assert torch.equal(ret.cpu(), want_ret), (gamma, lam)
     # masked_var stand-alone, both estimators, float and bool masks
     for unbiased in (True, False):
         want = o_loss.masked_var(r, mask.float(), unbiased)
@@ -645,7 +653,8 @@ def test_group_advantage_parity(dev, reference_vectors):
     assert torch.allclose(ret.cpu(), torch.tensor(v["returns"]), atol=1e-4)
     assert adv.data_ptr() != ret.data_ptr()
     gen = torch.Generator().manual_seed(31)
-    for batch, group, width in [(128, 8, 2048), (16, 4, 256), (128, 16, 333), (6, 1, 4), (64, 64, 7)]:
+    for batch, group, width in [(128, 8, 2048), (16, 4, 256), (128, 16, 333), (6, 1, 4), (64, 64, 7), (192, 96, 9),
+                                (400, 200, 5), (130, 65, 70)]:
         rewards = torch.bernoulli(torch.rand(batch // group, 1, generator=gen).repeat(1, group), generator=gen)
         rewards = rewards.reshape(batch, 1)
         rewards[:group] = 1.0                          # an all-equal group: exactly zero
@@ -666,12 +675,17 @@ def test_group_advantage_parity(dev, reference_vectors):
             assert torch.equal(got[:group].cpu(), torch.zeros(group, width))
             # group assignment is row // G exactly: the sign pattern of each row follows its own group
             assert torch.equal((got.cpu() != 0), (want != 0))
-    # gaussian rewards in fp64
-    rewards = torch.randn(48, 1, generator=gen, dtype=torch.float64)
-    mask = torch.ones(48, 3)
-    want, _ = o_adv.compute_group_norm_advantage_return(rewards, mask, torch.zeros(48, 1), 6)
-    got, _ = mrl.compute_group_norm_advantage_return(rewards.to(dev), mask.to(dev), torch.zeros(48, 1), 6)
-    assert (got.cpu() - want).abs().max().item() < 1e-6
+    # gaussian rewards in fp64 and fp32, groups below, at and above the 64 lanes of the reducing wavefront
+    for n, group, dtype in ((48, 6, torch.float64), (256, 64, torch.float32), (300, 100, torch.float64),
+                            (63 * 3, 63, torch.float32)):
+        rewards = torch.randn(n, 1, generator=gen, dtype=dtype) * 3 + 1
+        mask = torch.ones(n, 3)
+        want, _ = o_adv.compute_group_norm_advantage_return(rewards, mask, torch.zeros(n, 1), group)
+        got, _ = mrl.compute_group_norm_advantage_return(rewards.to(dev), mask.to(dev), torch.zeros(n, 1), group)
+        assert (got.cpu() - want).abs().max().item() < 1e-6
+        want_last = o_adv.get_last_reward(rewards.float(), group)
+        got_last = mrl.get_last_reward(rewards.float().to(dev), group)
+        assert got_last.shape == rewards.shape and (got_last.cpu() - want_last).abs().max().item() < 1e-5
 
 
 def test_dynamic_sampling_keep_bit_exact(dev):
@@ -2235,6 +2249,126 @@ def test_one_loss_object_over_interleaved_micro_batches(dev, fused):
             assert (leaves[i].grad.cpu() - want[i][1]).abs().max().item() < 1e-6
 
 
+def _pack_sequence_logits(seq_logits, seqlens, cu, total):
+    """The stand-in for the model of the dynamic-batching test: row cu[i] + j of the packed
+    [1, T, V] logits is what the model emits for position j of sequence i; alignment rows are 0."""
+    out = torch.zeros(1, total, seq_logits.shape[-1], dtype=seq_logits.dtype, device=seq_logits.device)
+    for i, n in enumerate(seqlens.tolist()):
+        start = int(cu[i])
+        out[0, start:start + n] = seq_logits[i, :n]
+    return out
+
+
+@pytest.mark.parametrize("algo", ["grpo", "dapo"])
+def test_dynamic_micro_batches_end_to_end(dev, algo):
+    """How the reference chunks an update when use_dynamic_bsz is on (utils/seqlen_balancing.py:339-380,
+    models/base/base_training_engine.py:160-187, 238-270): 80 ragged sequences on the device are cut
+    into token-budget micro-batches, each is packed, scored and back-propagated with loss / n_micro
+    through ONE loss object with use_dynamic_bsz / actual_micro_batch_size.  The partitions, every
+    micro-batch's loss and statistics, the summed loss and every sequence's dlogits equal the
+    oracle's run over the oracle's own partitions, fused and split.  The DAPO variant applies the
+    dynamic-sampling filter first (workers/dynamic_sampling.py:81-86): groups whose rewards are all
+    equal never reach the loss."""
+    from mindspeed_rl_amd import seqlen_balancing as bal
+    from oracle import balancing as o_bal
+    gen = torch.Generator().manual_seed(77 if algo == "grpo" else 78)
+    n_prompts, group, vocab, align = 10, 8, 1032, 2
+    n_all = n_prompts * group
+    rlen = torch.randint(4, 61, (n_all, 1), generator=gen, dtype=torch.int32)
+    plen = torch.randint(1, 7, (n_all, 1), generator=gen, dtype=torch.int32)
+    width, resp_w = int((plen + rlen).max()), int(rlen.max())
+    ids = torch.randint(0, vocab, (n_all, width), generator=gen)
+    ids = ids * o_pack.generate_mask(ids, plen + rlen)
+    seq_logits = torch.randn(n_all, width, vocab, generator=gen) * 2
+    p = torch.rand(n_prompts, 1, generator=gen)
+    p[1], p[4], p[7] = 0.0, 1.0, 0.0                       # three groups with all-equal rewards
+    rewards = torch.bernoulli(p.repeat(1, group).reshape(n_all, 1), generator=gen)
+    rmask = o_pack.generate_mask(torch.zeros(n_all, resp_w), rlen)
+    adv, _ = o_adv.compute_group_norm_advantage_return(rewards, rmask, rlen, group)
+    labels_pad = torch.cat([ids[:, 1:], torch.zeros(n_all, 1, dtype=ids.dtype)], 1)
+    full = {"input_ids": ids, "responses": torch.zeros(n_all, resp_w, dtype=torch.int64), "response_length": rlen,
+            "prompt_length": plen, "advantages": adv}
+    lp0 = o_loss.logprob_computer(seq_logits, dict(full, labels=labels_pad), True)[0]
+    full["old_log_prob"] = (lp0 + torch.randn(lp0.shape, generator=gen) * 0.05) * rmask
+    full["ref_log_prob"] = (lp0 + torch.randn(lp0.shape, generator=gen) * 0.05) * rmask
+    if algo == "dapo":
+        keep_o = o_adv.dynamic_sampling_keep(rewards.flatten().numpy(), group)
+        keep = mrl.dynamic_sampling_keep(rewards.flatten().to(dev), group)
+        assert keep == keep_o and 0 < len(keep) <= n_all - 3 * group
+        full = {k: v[keep] for k, v in full.items()}
+        seq_logits = seq_logits[keep]
+        meta_o = dict(clip_ratio=0.2, clip_higher_enable=True, clip_ratio_low=0.2, clip_ratio_high=0.28,
+                      token_level_loss=True, entropy_coeff=0.001)
+        meta_d = dict(meta_o)
+        oracle_loss, make = o_loss.dapo_compute_loss, mrl.DAPOActorLossFunc
+    else:
+        meta_o = dict(clip_ratio=0.2, kl_coef=0.01, kl_penalty="low_var_kl", entropy_coeff=0.001)
+        meta_d = {"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.01), "kl_penalty": "low_var_kl",
+                  "entropy_coeff": 0.001}
+        oracle_loss, make = o_loss.grpo_compute_loss, mrl.GRPOActorLossFunc
+    n_seq = full["input_ids"].shape[0]
+    max_tokens, max_bsz = 300, 12
+
+    # ---- the oracle: its own partitions, CPU packing, CPU loss
+    lengths = (full["prompt_length"] + full["response_length"]).flatten().tolist()
+    parts_o = o_bal.rearrange_micro_batches(lengths, max_tokens, dynamic_max_batch_size=max_bsz)
+    n_micro = len(parts_o)
+    assert n_micro >= 5 and sorted(i for part in parts_o for i in part) == list(range(n_seq))
+    want_grads, want_losses, want_stats = {}, [], []
+    for part in parts_o:
+        mb = {k: v[part] for k, v in full.items()}
+        lab = torch.cat([mb["input_ids"][:, 1:], torch.zeros(len(part), 1, dtype=ids.dtype)], 1)
+        mask1d = o_pack.generate_mask(mb["input_ids"], mb["prompt_length"] + mb["response_length"])
+        _, _, p_lab, seqlens, cu = o_pack.preprocess_packed_seqs(mb["input_ids"], lab, mask1d, align)
+        z = _pack_sequence_logits(seq_logits[part], seqlens, cu, p_lab.shape[1]).requires_grad_()
+        mb["labels"] = p_lab
+        loss, stats = oracle_loss(z, mb, meta_o, use_remove_padding=True, seqlens_in_batch=seqlens,
+                                  cu_seqlens_padded=cu, seq_len=width, use_dynamic_bsz=True,
+                                  actual_micro_batch_size=n_seq / n_micro)
+        (loss / n_micro).backward()
+        want_losses.append(loss.item())
+        want_stats.append(stats)
+        for i, s in enumerate(part):
+            want_grads[s] = z.grad[0, int(cu[i]):int(cu[i]) + int(seqlens[i])].clone()
+
+    # ---- the device path: split on the device batch, pack with the index-map kernels, one loss object
+    full_d = _to_dev(full, dev)
+    logits_d = seq_logits.to(dev)
+    for fused in (True, False):
+        f = make()
+        f.add_loss_meta_info(meta_d)
+        batches, parts = bal.split_batches_with_dynamic_bsz(full_d, max_tokens, max_bsz)
+        assert parts == parts_o
+        total_loss = 0.0
+        for k, (mb, part) in enumerate(zip(batches, parts)):
+            lab = torch.cat([mb["input_ids"][:, 1:], torch.zeros(len(part), 1, dtype=ids.dtype, device=dev)], 1)
+            mask1d = mrl.generate_mask(mb["input_ids"], mb["prompt_length"] + mb["response_length"])
+            _, _, p_lab, seqlens, cu = mrl.preprocess_packed_seqs(mb["input_ids"], lab, mask1d, align)
+            zd = _pack_sequence_logits(logits_d[part], seqlens.cpu(), cu.cpu(), p_lab.shape[1]).requires_grad_()
+            mb["labels"] = p_lab
+            loss, stats = f.compute_loss(zd, mb, fused=fused, use_remove_padding=True, seqlens_in_batch=seqlens,
+                                         cu_seqlens_padded=cu, seq_len=width, use_dynamic_bsz=True,
+                                         actual_micro_batch_size=n_seq / n_micro, index=None)
+            (loss / n_micro).backward()
+            assert loss.item() == pytest.approx(want_losses[k], rel=TOL_LOSS_REL, abs=1e-7)
+            for name, v in want_stats[k].items():
+                assert stats[name] == pytest.approx(v, rel=TOL_LOSS_REL, abs=1e-6), (k, name)
+            total_loss += loss.item() / n_micro
+            cu_h, len_h = cu.cpu(), seqlens.cpu()
+            for i, s in enumerate(part):
+                got = zd.grad[0, int(cu_h[i]):int(cu_h[i]) + int(len_h[i])].cpu()
+                assert (got - want_grads[s]).abs().max().item() < 1e-6, (k, s)
+            if align > 1 and int(cu_h[-1]) > int(len_h.sum()):
+                pad_rows = torch.ones(int(cu_h[-1]), dtype=torch.bool)
+                for i in range(len(part)):
+                    pad_rows[int(cu_h[i]):int(cu_h[i]) + int(len_h[i])] = False
+                assert not zd.grad[0][pad_rows.to(dev)].any().item()      # alignment rows get no gradient
+        assert total_loss == pytest.approx(sum(want_losses) / n_micro, rel=TOL_LOSS_REL, abs=1e-7)
+        if fused:
+            # upstream 1/n_micro is learned from the first backward: one rescale pass, not n_micro
+            assert f.grad_scale_state(dev).rescales.item() == 1
+
+
 def _small_padded_micro_batch(seed, n_seq, seq_len, vocab):
     g = torch.Generator().manual_seed(seed)
     plen = torch.randint(1, 5, (n_seq, 1), generator=g)
@@ -2386,3 +2520,31 @@ def test_vocabulary_shards_merge_to_the_full_sweep(dev, dtype, bounds):
     assert not dz[5].any().item()
     # a label outside every shard: the oracle (Megatron's target mask) scores the row maximum there,
     # a sharded run scores 0 - documented difference, no rank owns such a label
+
+
+@pytest.mark.parametrize("switches,subset", [
+    ({"MRL_SWEEP_PERSISTENT": "0", "MRL_BWD_CHUNK": "0"},
+     "test_persistent_row_sweeps or test_fused_sweep_persistent or test_backward_fp32_full_vocab or "
+     "test_fused_sweep_random_shapes or test_split_sweeps_random_shapes or test_vocab_forward_backward_parity"),
+    ({"MRL_LMHEAD_V2": "0", "MRL_SWEEP_TICKET": "0"},
+     "test_lmhead_logprob_forward or test_lmhead_forward_random_shapes or test_fused_lmhead_policy_loss or "
+     "test_fused_sweep_persistent or test_persistent_row_sweeps"),
+], ids=["per_row_sweep_and_loop_backward", "first_lmhead_loop_and_fixed_stride"])
+def test_library_switches_in_child_processes(dev, switches, subset):
+    """The library reads its tuning switches once per process, so the kernels behind them (one workgroup
+    per row instead of persistent workgroups, the loop backward for every row length, the first
+    lm_head tile loop, the fixed row stride) cannot be reached from this process: a child process per
+    switch set runs the parity tests that cover those kernels at the sizes where the switch matters."""
+    import subprocess
+    import sys
+    env = dict(os.environ, **switches)
+    here = os.path.abspath(__file__)
+    assert "MRL_CHILD_OF_SWITCH_TEST" not in os.environ, "a child process must not start children of its own"
+    env["MRL_CHILD_OF_SWITCH_TEST"] = "1"
+    subset = "(%s) and not child_processes" % subset
+    proc = subprocess.run([sys.executable, "-m", "pytest", here, "-x", "-q", "-m", "gpu", "-k", subset,
+                           "-p", "no:cacheprovider"],
+                          env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=280)
+    tail = "\n".join(proc.stdout.splitlines()[-15:])
+    assert proc.returncode == 0, tail
+    assert " passed" in tail and "failed" not in tail, tail

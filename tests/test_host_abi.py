@@ -226,3 +226,23 @@ def test_host_side_error_contracts():
     assert mrl.masked_mean(torch.tensor([1.0, 2.0, 3.0]), torch.tensor([1.0, 0.0, 1.0]), epsilon=0) == 2.0
     assert mrl.compute_kl_penalty(torch.tensor([[0.5, 1.0]]), torch.tensor([[1.0, 0.5]])).tolist() == \
         [[0.14872121810913086, 0.10653066635131836]]
+
+
+def test_multimodal_switch_selects_strategy_and_partitioner(monkeypatch):
+    """The reference's process-wide switch (utils/utils.py:719-720, read in base_loss_func.py:15 and
+    utils/seqlen_balancing.py:358): the environment variable IS_MULTIMODAL as a python literal."""
+    from mindspeed_rl_amd import seqlen_balancing as sb
+    monkeypatch.delenv("IS_MULTIMODAL", raising=False)
+    assert mrl.is_multimodal() is False
+    assert type(mrl.GRPOActorLossFunc().logprob_computer) is mrl.StandardLogProbComputer
+    lengths = [90, 80, 70, 30, 20, 10]
+    plain = sb.rearrange_micro_batches(lengths, 100)
+    monkeypatch.setenv("IS_MULTIMODAL", "True")
+    assert mrl.is_multimodal() is True
+    for klass in (mrl.GRPOActorLossFunc, mrl.DAPOActorLossFunc, mrl.PPOActorLossFunc, mrl.ReferenceLossFunc):
+        assert type(klass().logprob_computer) is mrl.MultimodalLogProbComputer
+    packed = sb.rearrange_micro_batches(lengths, 100)
+    assert packed == sb.balanced_bin_packing(lengths, 100)
+    assert sb.rearrange_micro_batches(lengths, 100, multimodal=False) == plain
+    monkeypatch.setenv("IS_MULTIMODAL", "False")
+    assert type(mrl.GRPOActorLossFunc().logprob_computer) is mrl.StandardLogProbComputer
