@@ -1421,21 +1421,43 @@ def test_fused_sweep_on_two_streams_and_in_a_graph(dev):
         assert torch.equal(other, want[1][0])
 
 
-@pytest.mark.parametrize("workload", ["c1", "c4chunk"])
+@pytest.mark.parametrize("workload", ["c1", "c4chunk", "c2"])
 def test_full_size_properties(dev, workload):
     """configs[1] at its full size (128 responses, about 171 k packed rows x 152064 bf16 = 52 GB of
-    logits) and one 64 k-row chunk of configs[4] (DAPO clip-higher, no KL, V = 129280), where the
-    oracle cannot follow: the fused sweep and the split kernels (independent code) agree on loss,
-    statistics and dlogits; every dlogits row sums to zero (the softmax gradient is orthogonal to the
-    constant vector); rows without a response token are exactly zero; and a random sample of rows
-    matches the oracle's closed forms."""
+    logits), the same batch as configs[2]'s padded [128, S, 152064] logits (79 GB, with a group of empty
+    responses and a group of all-equal rewards) and one 64 k-row chunk of configs[4] (DAPO clip-higher,
+    no KL, V = 129280), where the oracle cannot follow: the fused sweep and the split kernels
+    (independent code) agree on loss, statistics and dlogits; every dlogits row sums to zero (the
+    softmax gradient is orthogonal to the constant vector); rows without a response token (prompt
+    rows, padding) are exactly zero; and a random sample of rows matches the oracle's closed forms.
+    The split leg writes its gradient over the logits (grad_inplace) so that the padded case fits."""
     import bench
+    import gc
     w = bench.WORKLOADS[workload]
+    gc.collect()
+    torch.cuda.empty_cache()                    # blocks cached by earlier tests count as used otherwise
     free, _ = torch.cuda.mem_get_info(dev)
-    if free < (190 if workload == "c1" else 70) * 2 ** 30:
+    if free < {"c1": 190, "c2": 230, "c4chunk": 70}[workload] * 2 ** 30:
         pytest.skip("needs more free HBM")
     plen, rlen, rewards = bench.make_lengths(torch, w, 0)
     logits, b, kw, total = bench.build_device_batch(torch, mrl, w, plen, rlen, rewards, dev, 0)
+    vocab = logits.shape[-1]
+    flat = logits.view(-1, vocab)
+    flat_labels = b["labels"].reshape(-1)
+    assert flat.shape[0] == total
+    # rows that carry a response token (prompt length 1 everywhere: the first R_i rows of each sequence)
+    live = torch.zeros(total, dtype=torch.bool)
+    if w.get("layout") == "padded":
+        width = logits.shape[1]
+        assert logits.shape[0] == 128 and total == 128 * width
+        for i, r in enumerate(rlen.flatten().tolist()):
+            live[i * width:i * width + r] = True
+        assert (rlen.reshape(-1, w["group"]) == 0).all(1).any().item()          # the group of empty responses
+    else:
+        cu = kw["cu_seqlens_padded"].cpu().tolist()
+        for i, r in enumerate(rlen.flatten().tolist()):
+            live[cu[i]:cu[i] + r] = True
+    live_d = live.to(dev)
     if w.get("loss") == "dapo":
         f = mrl.LossFuncFactory.get_instance("ray_dapo", "actor")
         f.add_loss_meta_info({"clip_ratio": 0.2, "clip_higher_enable": True, "clip_ratio_low": 0.2,
@@ -1444,12 +1466,32 @@ def test_full_size_properties(dev, workload):
         f = mrl.LossFuncFactory.get_instance("ray_grpo", "actor")
         f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.001), "kl_penalty": "low_var_kl",
                               "entropy_coeff": 0.001})
+    # a sample of rows against the oracle: log-prob and entropy (taken first: the split leg below
+    # overwrites the logits)
+    gen = torch.Generator().manual_seed(5)
+    live_idx = torch.nonzero(live).flatten()
+    pick = torch.cat([live_idx[torch.randint(0, live_idx.numel(), (40,), generator=gen)],
+                      torch.randint(0, total, (8,), generator=gen)])
+    pick_d = pick.to(dev)
+    zs = flat[pick_d].float().cpu()
+    ys = flat_labels[pick_d].cpu()
+    lp, h, lse = mrl.vocab_logprob_entropy(flat, flat_labels)
+    want_lp = o_vocab.compute_log_probs(zs, ys)
+    want_h = o_vocab.vocab_parallel_entropy(zs)
+    assert (lp[pick_d].cpu() - want_lp).abs().max().item() < TOL_LOGP
+    assert (h[pick_d].cpu() - want_h).abs().max().item() < TOL_LOGP
+    del lp, h, lse
+
     z1 = logits.detach().requires_grad_()
     loss_f, stats_f = f.compute_loss(z1, b, fused=True, **kw)
     (dz_f,) = torch.autograd.grad(loss_f, z1)
+    dz_f = dz_f.view(-1, vocab)
+    got = dz_f[pick_d].float().cpu()
     z2 = logits.detach().requires_grad_()
-    loss_s, stats_s = f.compute_loss(z2, b, fused=False, **kw)
+    loss_s, stats_s = f.compute_loss(z2, b, fused=False, grad_inplace=True, **kw)
     (dz_s,) = torch.autograd.grad(loss_s, z2)
+    dz_s = dz_s.view(-1, vocab)
+    assert dz_s.data_ptr() == logits.data_ptr()
     assert loss_s.item() == pytest.approx(loss_f.item(), rel=TOL_LOSS_REL)
     for k in stats_f:
         # ppo_kl is a mean of 171 k differences of about +-0.05 that nearly cancels (5e-6): the absolute
@@ -1458,44 +1500,86 @@ def test_full_size_properties(dev, workload):
     rows_per = 8192
     scale, worst_sum, worst_diff = 0.0, 0.0, 0.0
     for lo in range(0, total, rows_per):
-        a = dz_f[0, lo:lo + rows_per].float()
+        a = dz_f[lo:lo + rows_per].float()
+        c = dz_s[lo:lo + rows_per].float()
         scale = max(scale, a.abs().max().item())
-        worst_diff = max(worst_diff, (a - dz_s[0, lo:lo + rows_per].float()).abs().max().item())
+        worst_diff = max(worst_diff, (a - c).abs().max().item())
         worst_sum = max(worst_sum, a.sum(-1).abs().max().item())
-        del a
+        # rows that are no response token get exactly zero from both paths
+        dead = ~live_d[lo:lo + rows_per]
+        assert a.abs().amax(-1)[dead].max().item() == 0 if dead.any().item() else True
+        assert c.abs().amax(-1)[dead].max().item() == 0 if dead.any().item() else True
+        del a, c
     assert scale > 0
     assert worst_diff <= 2 ** -7 * scale
     assert worst_sum <= 0.02 * scale                    # 152 k bf16 roundings against a one-hot entry of `scale`
-    # rows that are no response token (the last row of every sequence here: prompt length 1)
-    cu = kw["cu_seqlens_padded"].cpu()
-    last = (cu[1:] - 1).long().to(dev)
-    assert not dz_f[0, last].any().item() and not dz_s[0, last].any().item()
-    del dz_s, z2
-    # a sample of rows against the oracle: log-prob, entropy, and the gradient implied by them
-    gen = torch.Generator().manual_seed(5)
-    pick = torch.randint(0, total, (48,), generator=gen)
-    zs = logits[0, pick.to(dev)].float().cpu()
-    ys = b["labels"][0, pick.to(dev)].cpu()
-    lp, h, lse = mrl.vocab_logprob_entropy(logits[0], b["labels"][0])
-    want_lp = o_vocab.compute_log_probs(zs, ys)
-    want_h = o_vocab.vocab_parallel_entropy(zs)
-    assert (lp[pick.to(dev)].cpu() - want_lp).abs().max().item() < TOL_LOGP
-    assert (h[pick.to(dev)].cpu() - want_h).abs().max().item() < TOL_LOGP
+    assert (~live).sum().item() >= rlen.numel()
     # dlogits of a live row is c0 * (onehot - p) - c1 * p * (z - E z): recover c0 from the label entry and
     # check the rest of the row against the oracle's softmax with it (entropy coefficient folded into c1)
     p = torch.softmax(zs, -1)
-    got = dz_f[0, pick.to(dev)].float().cpu()
     ent_term = p * (zs - (p * zs).sum(-1, keepdim=True))
     onehot = torch.zeros_like(p)
     onehot[torch.arange(len(ys)), ys] = 1.0
     basis0, basis1 = onehot - p, -ent_term
+    checked = 0
     for i in range(len(pick)):
+        assert bool(got[i].any()) == bool(live[pick[i]]) or not live[pick[i]]
         if not got[i].any():
             continue
         a = torch.stack([basis0[i], basis1[i]], 1).double()
         coef = torch.linalg.lstsq(a, got[i].double().unsqueeze(1)).solution
         resid = (a @ coef).squeeze(1) - got[i].double()
         assert resid.abs().max().item() <= 2 ** -8 * got[i].abs().max().item() + 1e-12, i
+        checked += 1
+    assert checked >= 30
+
+
+def test_full_size_lmhead_forward(dev):
+    """configs[3]'s forward at its full size (163 840 tokens x 3584 hidden x 152 064 vocabulary, logits
+    never stored): 48 sampled tokens against the oracle (fp32 product of the bf16 operands on the CPU),
+    4096 tokens against an fp32 GEMM + log-softmax on the device, and size-independent properties over
+    all tokens: 0 <= entropy <= ln V, logp <= 0, logsumexp finite, and the static-scratch entry
+    point's limit respected by slicing."""
+    import gc
+    gc.collect()
+    torch.cuda.empty_cache()
+    free, _ = torch.cuda.mem_get_info(dev)
+    if free < 40 * 2 ** 30:
+        pytest.skip("needs more free HBM")
+    tokens, vocab, hdim = 163840, 152064, 3584
+    g = torch.Generator(device=dev).manual_seed(3)
+    hidden = torch.randn(tokens, hdim, generator=g, device=dev).to(torch.bfloat16)
+    weight = (torch.randn(vocab, hdim, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    labels = torch.randint(0, vocab, (tokens,), generator=g, device=dev)
+    lp, ent, lse = mrl.lmhead_logprob(hidden, weight, labels, inv_temperature=1.0)
+    torch.cuda.synchronize()
+    assert torch.isfinite(lse).all().item() and (lp <= 0).all().item()
+    assert (ent >= 0).all().item() and (ent <= math.log(vocab) + 1e-3).all().item()
+    gen = torch.Generator().manual_seed(4)
+    pick = torch.randint(0, tokens, (48,), generator=gen)
+    pick[0], pick[1] = 0, tokens - 1
+    lp_o, h_o, lse_o = o_vocab.lmhead_logprob_entropy(hidden[pick.to(dev)].cpu(), weight.cpu(), labels[pick.to(dev)].cpu())
+    assert (lse[pick.to(dev)].cpu() - lse_o).abs().max().item() < 1e-4
+    assert (lp[pick.to(dev)].cpu() - lp_o).abs().max().item() < 2e-4
+    assert (ent[pick.to(dev)].cpu() - h_o).abs().max().item() < 2e-4
+    # a contiguous block straddling token tiles, fp32 on the device
+    lo = 163840 - 4096 - 77
+    ref = torch.log_softmax(torch.nn.functional.linear(hidden[lo:lo + 4096].float(), weight.float()), -1)
+    assert (lp[lo:lo + 4096] - ref.gather(-1, labels[lo:lo + 4096, None])[:, 0]).abs().max().item() < 2e-4
+    assert (ent[lo:lo + 4096] + (ref.exp() * ref).sum(-1)).abs().max().item() < 2e-4
+    del ref
+    # the same tokens through the entry point that allocates nothing, in slices of its limit
+    lib = _lib.load()
+    limit = lib.mrl_lmhead_static_max_tokens()
+    lp2, ent2, lse2 = (torch.empty_like(lp) for _ in range(3))
+    for c0 in range(0, tokens, limit):
+        n = min(limit, tokens - c0)
+        _lib.call("mrl_lmhead_logprob_fwd_static", hidden.data_ptr() + c0 * hdim * 2, weight.data_ptr(), n, vocab, hdim,
+                  labels.data_ptr() + c0 * 8, _lib.I64, 1.0, lp2.data_ptr() + c0 * 4, ent2.data_ptr() + c0 * 4,
+                  lse2.data_ptr() + c0 * 4, _lib.stream(dev))
+    torch.cuda.synchronize()
+    # the partial statistics of a token do not depend on which other tokens share the call
+    assert torch.equal(lp2, lp) and torch.equal(ent2, ent) and torch.equal(lse2, lse)
 
 
 def _random_fused_case(i, rnd):
