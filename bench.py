@@ -61,6 +61,9 @@ def parse_args():
     ap.add_argument("--path", default="fused", choices=["fused", "split"],
                     help="fused: one sweep computes log-prob, loss and dlogits (1 read + 1 write of [T,V]); "
                          "split: forward sweep, then the backward sweep from the saved logsumexp (2 reads + 1 write)")
+    ap.add_argument("--dtype", default=None, choices=["bf16", "f32"],
+                    help="logits dtype instead of the workload's own (f32 at the configs[1] vocabulary: rows that two "
+                         "workgroups hold in the fused sweep)")
     ap.add_argument("--upstream", type=float, default=1.0,
                     help="scalar the step multiplies the loss by before backward(), as Megatron's schedule does with "
                          "1/num_microbatches; the loss object is not told and learns it from the first backward")
@@ -350,8 +353,12 @@ def run_lmhead_train(args):
 # reads for the copy probe).  Only the default workload has been profiled that way; any other
 # workload, another library build (MRL_LIB_PATH) or a tuning switch (MRL_*) reports null.
 PROFILED_TRAFFIC = {
-    ("c1", "fused", "mrl_fused_logprob_loss"): (104.05e9, "profiles/fused_sweep_persistent_kernel__c1_qwen25_grpo.md"),
-    ("c1", "split", "mrl_vocab_logprob_bwd"): (104.06e9, "profiles/vocab_fwd_kernel_and_bwd_chunk_kernel__c1_split_path.md"),
+    ("c1", "bf16", "fused", "mrl_fused_logprob_loss"):
+        (104.05e9, "profiles/fused_sweep_persistent_kernel__c1_qwen25_grpo.md"),
+    ("c1", "bf16", "split", "mrl_vocab_logprob_bwd"):
+        (104.06e9, "profiles/vocab_fwd_kernel_and_bwd_chunk_kernel__c1_split_path.md"),
+    ("c1", "f32", "fused", "mrl_fused_logprob_loss"):
+        (208.18e9, "profiles/fused_sweep_persistent_kernel_half_rows__c1_fp32_logits.md"),
 }
 
 
@@ -359,7 +366,7 @@ def _profiled_traffic(args, w, dominant):
     """(bytes or None, where the figure comes from)."""
     if args.entropy_coeff != 0.001 or any(k.startswith("MRL_") for k in os.environ):
         return None, None
-    return PROFILED_TRAFFIC.get((args.workload, args.path, dominant), (None, None))
+    return PROFILED_TRAFFIC.get((args.workload, w["dtype"], args.path, dominant), (None, None))
 
 
 def main():
@@ -383,7 +390,10 @@ def main():
         return
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    w = WORKLOADS[args.workload]
+    w = dict(WORKLOADS[args.workload])
+    if args.dtype is not None and args.dtype != w["dtype"]:
+        w["dtype"] = args.dtype
+        w["desc"] += " [logits as %s]" % args.dtype
     plen, rlen, rewards = make_lengths(torch, w, args.seed)
     logits, b, kw, total = build_device_batch(torch, mrl, w, plen, rlen, rewards, dev, args.seed)
     tokens = int(rlen.sum())
@@ -438,11 +448,13 @@ def main():
     }
     # the kernel each entry point dispatches to for this shape (csrc/row_sweep.hip, csrc/vocab_logprob.hip)
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
-    persistent = os.environ.get("MRL_SWEEP_PERSISTENT", "1") != "0" and total > 2 * cus
+    wide = row_bytes > 19 * 1024 * 16                      # a row that two workgroups hold
+    persistent = wide or (os.environ.get("MRL_SWEEP_PERSISTENT", "1") != "0" and total > 2 * cus)
     chunked = os.environ.get("MRL_BWD_CHUNK", "1") != "0" and row_bytes >= 16384 and row_bytes % 16 == 0
     kernel_symbol = {"mrl_vocab_logprob_fwd": "vocab_fwd_kernel",
                      "mrl_vocab_logprob_bwd": "bwd_chunk_kernel" if chunked else "vocab_bwd_kernel",
-                     "mrl_fused_logprob_loss": "fused_sweep_persistent_kernel" if persistent else "fused_sweep_kernel"}
+                     "mrl_fused_logprob_loss": ("fused_sweep_persistent_kernel" + (" (half rows)" if wide else ""))
+                     if persistent else "fused_sweep_kernel"}
     kernels = {}
     for name, nbytes in kernel_bytes.items():
         ms = avg_ms(name)

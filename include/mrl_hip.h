@@ -274,8 +274,16 @@ int mrl_policy_loss_bwd(const float* log_prob, const float* old_log_prob,
  * mrl_scale_rows when autograd later delivers an upstream gradient.
  */
 
-/* Largest vocabulary the row-in-registers kernels hold for a logits dtype (0 = bad dtype). */
+/* Largest vocabulary the row-in-registers kernels hold for a logits dtype (0 = bad dtype): one
+ * workgroup keeps up to 19 456 16-byte vectors of a row in registers, and rows of up to twice that
+ * (311 296 bf16 / fp16 or 155 648 fp32 logits) are cut in two halves held by two workgroups at the
+ * same time, which exchange the statistics of their halves through the workspace. */
 int64_t mrl_fused_max_vocab(int logits_dtype);
+
+/* Bytes of workspace mrl_fused_logprob_loss wants for this shape (16-byte aligned device memory):
+ * 16 for rows that one workgroup holds (the row counter), 16 + 32 * n_rows for wider rows (plus one
+ * 16-byte record per half row); 0 if the fused sweep does not take the shape at all. */
+int64_t mrl_fused_workspace_bytes(int logits_dtype, int64_t n_rows, int64_t vocab);
 
 /* Step 1.  Maps the [batch, width] loss operands onto logits rows.
  *   layout 0, packed [n_rows, V] logits: sequence i owns the rows postprocess_packed_seqs copies
@@ -307,20 +315,25 @@ int mrl_fused_loss_prepare(int layout, int64_t batch, int64_t width, int64_t n_r
  * autograd (models/base/base_training_engine.py:238-270), so the host never knows them in time.  Rows with mask 0 get zero dlogits and are not read.  dlogits may
  * alias logits exactly (in-place).  row_terms float [n_rows * 8] receives {pg, clipped, old-lp,
  * kl, entropy, 1} * mask per row for step 3.  logp / entropy: nullable [n_rows] outputs.
- * has_old = 0 means old_log_prob = log_prob.detach() (ratio 1).  row_ticket (nullable): 4 bytes of
- * device memory owned by the caller, the counter from which the persistent workgroups take their
- * next row (reset by this call on `stream`; it must not be shared by sweeps that can be in flight at
- * the same time, and a captured graph keeps using the address it was captured with).  NULL: rows are
- * walked with a fixed stride, about a twentieth slower on large batches.  Needs 16-byte aligned
- * rows, vocab % (16/elem) == 0 and vocab <= mrl_fused_max_vocab(dtype), else MRL_ERR_UNSUPPORTED
- * (use the split fwd/bwd entry points then). */
+ * has_old = 0 means old_log_prob = log_prob.detach() (ratio 1).  workspace:
+ * mrl_fused_workspace_bytes(dtype, n_rows, vocab) bytes of device memory owned by the caller: the
+ * counter from which the persistent workgroups take their next row and, for rows wider than one
+ * workgroup holds, the records through which the two halves of a row exchange their statistics
+ * (both reset by this call on `stream`; a workspace must not be shared by sweeps that can be in
+ * flight at the same time, and a captured graph keeps using the address it was captured with).
+ * NULL is allowed for rows that one workgroup holds: they are then walked with a fixed stride,
+ * about a twentieth slower on large batches.  Needs 16-byte aligned rows, vocab % (16/elem) == 0 and
+ * vocab <= mrl_fused_max_vocab(dtype), and wide rows (above half of that) cannot be swept in place;
+ * else MRL_ERR_UNSUPPORTED (use the split fwd/bwd entry points then).  The wait of a workgroup for
+ * the other half of its row is bounded: past the bound it computes that half's statistics itself
+ * from memory. */
 int mrl_fused_logprob_loss(const void* logits, int logits_dtype, int64_t n_rows, int64_t vocab,
                            int64_t row_stride, const void* labels, int labels_dtype,
                            float inv_temperature, const float* row_ops, int has_old,
                            float clip_lo, float clip_hi, int kl_penalty, float kl_coef,
                            float entropy_coeff, float grad_scale, const float* grad_scale_dev,
                            void* dlogits, int64_t dlogits_row_stride, float* logp, float* entropy,
-                           float* row_terms, uint32_t* row_ticket, void* stream);
+                           float* row_terms, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Step 3.  Sums row_terms per sequence (tokens with a non-zero mask but no logits row enter with
  * log_prob = entropy = 0, as in the split path) and finalizes out[8] / row_sums exactly like

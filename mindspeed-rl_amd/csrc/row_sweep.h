@@ -21,7 +21,9 @@ struct FusedArgs {
     const float* row_ops; int has_old;
     float clip_lo, clip_hi; int kl_penalty; float kl_coef, entropy_coeff, grad_scale;
     const float* grad_scale_dev;    // nullable device scalar that multiplies grad_scale
-    unsigned int* row_ticket;       // nullable: the caller's row counter of the persistent sweep
+    void* workspace;                // nullable for narrow rows: row counter (+ half-row records)
+    bool wide;                      // rows cut in two halves held by two workgroups
+    int64_t half_elems;             // entries of the first half
     void* dlogits; int64_t d_stride;
     float* logp; float* entropy; float* row_terms;
     bool with_entropy;

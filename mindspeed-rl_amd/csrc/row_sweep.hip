@@ -377,19 +377,101 @@ __device__ __forceinline__ uint32_t broadcast_ticket(uint32_t mine, uint32_t* sl
     return (uint32_t)__builtin_amdgcn_readfirstlane((int)*slot);
 }
 
+// ------------------------------------------------------------------------------ wide rows
+// A row that does not fit the registers of one CU is cut into two halves that two workgroups hold at
+// the same time (units 2 r and 2 r + 1 of the ticket order, so the halves of a row are taken by
+// workgroups that ask for work one after the other).  Each workgroup publishes the statistics of
+// its half - 16 bytes in the caller's workspace, written and read with device-scope atomics only,
+// so that no cache has to be flushed - and picks up the other half's before it computes the row's
+// gradient.  A workgroup publishes BEFORE it waits, and nothing it does before publishing depends on
+// another workgroup, so waits cannot form a cycle; the wait is bounded all the same: when the limit
+// is reached the workgroup reads the other half from memory and computes its statistics itself.
+// That fallback is why wide rows are not swept in place: the other half must still hold logits.
+struct HalfRecord {
+    unsigned long long ms;      // (m, s): never 0, s >= 1 or NaN
+    unsigned long long u1;      // (u, 1)
+};
+
+__device__ __forceinline__ unsigned long long pack2f(float lo, float hi) {
+    return (unsigned long long)__float_as_uint(lo) | ((unsigned long long)__float_as_uint(hi) << 32);
+}
+
+// Statistics of a stretch of a row streamed from memory by the whole workgroup (the fallback above).
+template <int DT, bool kEntropy>
+__device__ __forceinline__ Stats stream_stats(const typename Elem<DT>::T* base, int n_vec, float k, Stats* lds) {
+    using E = Elem<DT>;
+    constexpr int kVec = E::kVec;
+    const u32x4* vec = reinterpret_cast<const u32x4*>(base);
+    Stats st = {kMaxInit, 0.f, 0.f};
+    for (int idx = threadIdx.x; idx < n_vec; idx += kBlock) {
+        float z[kVec];
+        E::unpack(__builtin_nontemporal_load(vec + idx), z);
+        float vmax = st.m;
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) vmax = fmaxf(vmax, z[i]);
+        grow_max<kEntropy>(st, vmax, k);
+        const float mk = st.m * k;
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) add_one<kEntropy>(st, z[i], k, mk);
+    }
+    __syncthreads();            // lds may still be read by a slow wavefront of the previous reduction
+    return block_reduce_1024<kEntropy>(st, k, lds);
+}
+
+// Publishes `mine` as half `half` of a row, waits (bounded) for the other half and returns the
+// statistics of the whole row, merged in the order (first half, second half) by both workgroups.
+// rec: the row's two records.  other_base / other_vec: where the other half's logits lie.
+template <int DT, bool kEntropy>
+__device__ __forceinline__ Stats exchange_halves(const Stats& mine, int half, HalfRecord* rec, uint32_t spin_limit,
+                                                 const typename Elem<DT>::T* other_base, int other_vec, float k,
+                                                 Stats* lds, Stats* inbox, uint32_t* arrived) {
+    if (threadIdx.x == 0) {
+        __hip_atomic_store(&rec[half].ms, pack2f(mine.m, mine.s), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (kEntropy)
+            __hip_atomic_store(&rec[half].u1, pack2f(mine.u, __uint_as_float(1u)), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        // at most spin_limit polls; with a limit of 0 the record is not looked at at all, so that the
+        // fallback can be exercised deterministically
+        unsigned long long a = 0, b = kEntropy ? 0ull : 1ull;
+        for (uint32_t polls = 0; polls < spin_limit; ++polls) {
+            if (a == 0) a = __hip_atomic_load(&rec[half ^ 1].ms, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (kEntropy && b == 0)
+                b = __hip_atomic_load(&rec[half ^ 1].u1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (a != 0 && b != 0) break;
+            __builtin_amdgcn_s_sleep(4);
+        }
+        const bool ok = a != 0 && b != 0;
+        inbox->m = __uint_as_float((uint32_t)a);
+        inbox->s = __uint_as_float((uint32_t)(a >> 32));
+        inbox->u = kEntropy ? __uint_as_float((uint32_t)b) : 0.f;
+        *arrived = ok ? 1u : 0u;
+    }
+    __syncthreads();
+    Stats other = *inbox;
+    if (*arrived == 0u) other = stream_stats<DT, kEntropy>(other_base, other_vec, k, lds);   // uniform branch
+    return half == 0 ? merge<kEntropy>(mine, other, k) : merge<kEntropy>(other, mine, k);
+}
+
+__global__ void clear_words_kernel(unsigned long long* p, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0ull;
+}
+
 // Persistent variant of the fused sweep: one workgroup per CU walks rows and, as it turns the
 // registers of a row into dlogits, refills them with its NEXT row, so the statistics pass of the next
 // row starts on its first vectors while the last are still arriving - the register file never has to
 // hold two rows.
 // kTicket: the next row is the next unclaimed one (see "row tickets" above), taken while the row is
 // being written; otherwise row r is followed by r + grid.
-template <int DT, int NV, bool kEntropy, bool kTicket>
+// kWide: the units of work are half rows (see "wide rows" above): unit 2 r is the first
+// half_elems entries of row r, unit 2 r + 1 the rest; n_rows then counts units.
+template <int DT, int NV, bool kEntropy, bool kTicket, bool kWide>
 __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
     const typename Elem<DT>::T* logits, int64_t row_stride, int vocab, int64_t n_rows,
     const void* __restrict__ labels, int labels_dtype, float inv_t, const float* __restrict__ row_ops, int has_old,
     Params p, float grad_scale, const float* __restrict__ grad_scale_dev, typename Elem<DT>::T* dlogits,
     int64_t d_stride, float* __restrict__ logp, float* __restrict__ entropy, float* __restrict__ row_terms,
-    unsigned int* row_ticket) {
+    unsigned int* row_ticket, int half_elems, HalfRecord* half_records, uint32_t spin_limit) {
     using E = Elem<DT>;
     using T = typename E::T;
     constexpr int kVec = E::kVec;
@@ -397,10 +479,13 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
     // two slots used in turn: thread 0 may write the ticket of the following row while a slow
     // wavefront has yet to read this one's (one barrier per row separates a slot's reuse)
     __shared__ uint32_t next_row[2];
+    __shared__ Stats inbox;                 // the other half's statistics (wide rows)
+    __shared__ uint32_t arrived;
 
     const int tid = threadIdx.x;
-    const int n_vec = vocab / kVec;
-    const uint32_t row_bytes = (uint32_t)vocab * (uint32_t)sizeof(T);
+    // bytes and vectors of a unit: the whole row, or its first / second half
+    const uint32_t unit_bytes[2] = {(uint32_t)(kWide ? half_elems : vocab) * (uint32_t)sizeof(T),
+                                    (uint32_t)(kWide ? vocab - half_elems : 0) * (uint32_t)sizeof(T)};
     const float k = inv_t * kLog2e;
     const int64_t step = gridDim.x;
     if (grad_scale_dev) grad_scale *= *grad_scale_dev;
@@ -421,10 +506,12 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
         Next n;
         n.r = r2;
         const bool has = r2 < n_rows;
-        const int64_t rn = has ? r2 : r;
+        const int64_t un = has ? r2 : r;                    // unit
+        const int64_t rn = kWide ? (un >> 1) : un;          // row
+        const int hn = kWide ? (int)(un & 1) : 0;
         const bool live = has && (row_ops[rn * MRL_ROW_OPS + MRL_OP_MASK] != 0.f);
         const T* nrow = logits + rn * row_stride;
-        n.row = row_ref(nrow, live ? row_bytes : 0u);
+        n.row = row_ref(nrow + (hn ? half_elems : 0), live ? unit_bytes[hn] : 0u);
         n.y = load_label(labels, labels_dtype, rn);
         n.zy_ptr = nrow + ((n.y >= 0 && n.y < (int64_t)vocab) ? n.y : 0);
         return n;
@@ -457,10 +544,17 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
     }
     int parity = 0;
     while (r < n_rows) {
-        const RowRef dst = row_ref(dlogits + r * d_stride, row_bytes);
-        const float* ops = row_ops + r * MRL_ROW_OPS;
+        const int64_t row = kWide ? (r >> 1) : r;
+        const int half = kWide ? (int)(r & 1) : 0;
+        const int my_first = half ? half_elems : 0;         // first entry of this unit within the row
+        const int n_vec = (int)(unit_bytes[half] / 16u);
+        const RowRef dst = row_ref(dlogits + row * d_stride + my_first, unit_bytes[half]);
+        const float* ops = row_ops + row * MRL_ROW_OPS;
         const float m = ops[MRL_OP_MASK];
         const bool y_ok = (y >= 0) && (y < (int64_t)vocab);
+        // the label's entry gets its one-hot term from the unit that holds it
+        const int64_t y_here = y - my_first;
+        const bool y_mine = y_ok && (!kWide || (y_here >= 0 && y_here < (int64_t)(unit_bytes[half] / sizeof(T))));
         Next nx;
         if (!kTicket) nx = plan(r + step);
         uint32_t zy_next = 0;
@@ -469,10 +563,16 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
         if (m != 0.f) {
             const float z_y = E::from_bits(zy_bits);
             const Stats st = thread_stats<DT, NV, kEntropy>(v, n_vec, k);
-            const Stats tot = block_reduce_1024<kEntropy>(st, k, lds);
+            Stats tot = block_reduce_1024<kEntropy>(st, k, lds);
+            if (kWide) {
+                const int other_first = half ? 0 : half_elems;
+                tot = exchange_halves<DT, kEntropy>(tot, half, half_records + row * 2, spin_limit,
+                                                    logits + row * row_stride + other_first,
+                                                    (int)(unit_bytes[half ^ 1] / 16u), k, lds, &inbox, &arrived);
+            }
             float lse;
             const RowScalars s = row_scalars<kEntropy>(tot, k, inv_t, y_ok, z_y, ops, has_old, p, grad_scale, m, lse);
-            if (tid == 0) write_row_outputs(r, s, m, logp, entropy, row_terms);
+            if (tid == 0 && half == 0) write_row_outputs(row, s, m, logp, entropy, row_terms);
             if (s.g_lp != 0.f || s.g_h != 0.f) {
                 const RowGrad g = row_grad<kEntropy>(s, k, inv_t, lse);
                 // the ticket is asked for ahead of the stores and picked up behind the first H of
@@ -483,13 +583,13 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
                 if (kTicket) nx = plan((int64_t)broadcast_ticket(mine, &next_row[parity]));
                 load_part<0, H>(v, nx.row);
                 grad_part<DT, kEntropy, H, NV>(v, g, dst);
-                store_label_grad<DT, kEntropy>(dst, g, y_ok, y, z_y);
+                store_label_grad<DT, kEntropy>(dst, g, y_mine, y_here, z_y);
                 load_part<H, NV>(v, nx.row);
                 zy_next = E::load_bits(nx.zy_ptr);
                 wrote = true;
             }
-        } else if (tid == 0) {
-            write_masked_row_outputs(r, logp, entropy, row_terms);
+        } else if (tid == 0 && half == 0) {
+            write_masked_row_outputs(row, logp, entropy, row_terms);
         }
         if (!wrote) {                       // no gradient for this row: zeros, same order of operations
             uint32_t mine = 0;
@@ -630,29 +730,59 @@ bool persistent_enabled() {
     return on;
 }
 
+// Upper bound of the polls a workgroup spends waiting for the other half of a wide row before it
+// computes that half's statistics itself; MRL_WIDE_SPIN_LIMIT overrides it (0: never look, always compute).
+uint32_t wide_spin_limit() {
+    static const uint32_t limit = [] {
+        const char* e = getenv("MRL_WIDE_SPIN_LIMIT");
+        return e ? (uint32_t)strtoul(e, nullptr, 10) : (1u << 18);
+    }();
+    return limit;
+}
+
+constexpr int64_t kWorkspaceHeader = 16;    // the row counter, padded to the alignment of the records
+
 template <int DT, int NV>
 int launch_fused(const mrl::FusedArgs& a) {
     using T = typename Elem<DT>::T;
     const dim3 block(kBlock);
     const Params p = {a.clip_lo, a.clip_hi, a.kl_coef, a.entropy_coeff, 1.f, a.kl_penalty, 0};
+    unsigned int* counter = reinterpret_cast<unsigned int*>(a.workspace);
+    const bool tk = counter != nullptr;
+#define MRL_FUSEDP_LAUNCH(ENT, TK, WIDE, UNITS, HALF, REC)                                                         \
+    hipLaunchKernelGGL((fused_sweep_persistent_kernel<DT, NV, ENT, TK, WIDE>), pgrid, block, 0, a.stream,           \
+                       (const T*)a.logits, a.row_stride, (int)a.vocab, UNITS, a.labels, a.labels_dtype, a.inv_t,    \
+                       a.row_ops, a.has_old, p, a.grad_scale, a.grad_scale_dev, (T*)a.dlogits, a.d_stride, a.logp,  \
+                       a.entropy, a.row_terms, counter, HALF, REC, wide_spin_limit())
+    if (a.wide) {
+        // half rows: the persistent kernel for every batch size, an even number of workgroups
+        int cus = cu_count();
+        if (cus < 2) return mrl::fail(MRL_ERR_LAUNCH, "mrl_fused_logprob_loss: cannot query the device");
+        const int64_t units = 2 * a.n_rows;
+        const unsigned grid = (unsigned)((int64_t)(cus & ~1) < units ? (cus & ~1) : units);
+        const dim3 pgrid(grid);
+        HalfRecord* rec = reinterpret_cast<HalfRecord*>(reinterpret_cast<char*>(a.workspace) + kWorkspaceHeader);
+        const int64_t words = a.n_rows * 4;
+        hipLaunchKernelGGL(clear_words_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, a.stream,
+                           reinterpret_cast<unsigned long long*>(rec), words);
+        hipLaunchKernelGGL(ticket_reset_kernel, dim3(1), dim3(64), 0, a.stream, counter, grid);
+        const int half = (int)a.half_elems;
+        if (a.with_entropy) MRL_FUSEDP_LAUNCH(true, true, true, units, half, rec);
+        else MRL_FUSEDP_LAUNCH(false, true, true, units, half, rec);
+        return mrl::check_launch("mrl_fused_logprob_loss");
+    }
     const int cus = persistent_enabled() ? cu_count() : 0;
     if (cus > 0 && a.n_rows > 2 * (int64_t)cus) {
         const dim3 pgrid((unsigned)cus);
-#define MRL_FUSEDP_LAUNCH(ENT, TK)                                                                                \
-    hipLaunchKernelGGL((fused_sweep_persistent_kernel<DT, NV, ENT, TK>), pgrid, block, 0, a.stream, (const T*)a.logits, \
-                       a.row_stride, (int)a.vocab, a.n_rows, a.labels, a.labels_dtype, a.inv_t, a.row_ops,         \
-                       a.has_old, p, a.grad_scale, a.grad_scale_dev, (T*)a.dlogits, a.d_stride, a.logp, a.entropy,     \
-                       a.row_terms, a.row_ticket)
         // the workgroups start on rows 0 .. grid-1; the counter hands out the rows behind them
-        const bool tk = a.row_ticket != nullptr;
-        if (tk) hipLaunchKernelGGL(ticket_reset_kernel, dim3(1), dim3(64), 0, a.stream, a.row_ticket, (unsigned)cus);
-        if (a.with_entropy && tk) MRL_FUSEDP_LAUNCH(true, true);
-        else if (a.with_entropy) MRL_FUSEDP_LAUNCH(true, false);
-        else if (tk) MRL_FUSEDP_LAUNCH(false, true);
-        else MRL_FUSEDP_LAUNCH(false, false);
-#undef MRL_FUSEDP_LAUNCH
+        if (tk) hipLaunchKernelGGL(ticket_reset_kernel, dim3(1), dim3(64), 0, a.stream, counter, (unsigned)cus);
+        if (a.with_entropy && tk) MRL_FUSEDP_LAUNCH(true, true, false, a.n_rows, 0, nullptr);
+        else if (a.with_entropy) MRL_FUSEDP_LAUNCH(true, false, false, a.n_rows, 0, nullptr);
+        else if (tk) MRL_FUSEDP_LAUNCH(false, true, false, a.n_rows, 0, nullptr);
+        else MRL_FUSEDP_LAUNCH(false, false, false, a.n_rows, 0, nullptr);
         return mrl::check_launch("mrl_fused_logprob_loss");
     }
+#undef MRL_FUSEDP_LAUNCH
     const dim3 grid((unsigned)a.n_rows);
 #define MRL_FUSED_LAUNCH(ENT)                                                                                  \
     hipLaunchKernelGGL((fused_sweep_kernel<DT, NV, ENT>), grid, block, 0, a.stream, (const T*)a.logits,        \
@@ -737,7 +867,11 @@ bool row_sweep_supported(int dtype, int64_t vocab, const void* in, int64_t in_st
     if (eb == 0) return false;
     const int64_t per_vec = 16 / eb;
     if (vocab % per_vec != 0) return false;
-    if (pick_nv(vocab / per_vec) == 0) return false;
+    const int64_t n_vec = vocab / per_vec;
+    if (pick_nv(n_vec) == 0) {
+        // two halves held by two workgroups: not in place (see "wide rows")
+        if (pick_nv((n_vec + 1) / 2) == 0 || in == out) return false;
+    }
     if (!aligned(in, 16) || !aligned(out, 16)) return false;
     if (n_rows > 1 && ((in_stride * eb) % 16 != 0 || (out_stride * eb) % 16 != 0)) return false;
     return true;
@@ -748,7 +882,16 @@ bool row_sweep_supported(int dtype, int64_t vocab, const void* in, int64_t in_st
 extern "C" int64_t mrl_fused_max_vocab(int logits_dtype) {
     const int eb = mrl::float_dtype_bytes(logits_dtype);
     if (eb == 0) return 0;
-    return (int64_t)kMaxVecPerThread * kBlock * (16 / eb);
+    return 2 * (int64_t)kMaxVecPerThread * kBlock * (16 / eb);      // two workgroups hold a wide row
+}
+
+extern "C" int64_t mrl_fused_workspace_bytes(int logits_dtype, int64_t n_rows, int64_t vocab) {
+    const int eb = mrl::float_dtype_bytes(logits_dtype);
+    if (eb == 0 || n_rows < 0 || vocab <= 0 || vocab % (16 / eb) != 0) return 0;
+    const int64_t n_vec = vocab / (16 / eb);
+    if (pick_nv(n_vec) != 0) return kWorkspaceHeader;
+    if (pick_nv((n_vec + 1) / 2) == 0) return 0;
+    return kWorkspaceHeader + n_rows * (int64_t)sizeof(HalfRecord) * 2;
 }
 
 extern "C" int mrl_fused_logprob_loss(const void* logits, int logits_dtype, int64_t n_rows, int64_t vocab,
@@ -757,7 +900,7 @@ extern "C" int mrl_fused_logprob_loss(const void* logits, int logits_dtype, int6
                                       float clip_hi, int kl_penalty, float kl_coef, float entropy_coeff,
                                       float grad_scale, const float* grad_scale_dev, void* dlogits,
                                       int64_t dlogits_row_stride, float* logp, float* entropy, float* row_terms,
-                                      uint32_t* row_ticket, void* stream) {
+                                      void* workspace, int64_t workspace_bytes, void* stream) {
     const char* fn = "mrl_fused_logprob_loss";
     MRL_REQUIRE(n_rows >= 0 && vocab > 0 && n_rows <= 0x7fffffffLL, MRL_ERR_INVALID_ARG, "%s: n_rows=%lld vocab=%lld",
                 fn, (long long)n_rows, (long long)vocab);
@@ -773,11 +916,12 @@ extern "C" int mrl_fused_logprob_loss(const void* logits, int logits_dtype, int6
                 "%s: inv_temperature=%g must be in (0, 1e6)", fn, (double)inv_temperature);
     if (n_rows == 0) return MRL_OK;
     MRL_REQUIRE(logits && labels && row_ops && dlogits && row_terms, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
-    MRL_REQUIRE(mrl::aligned(row_ticket, 4) && mrl::aligned(grad_scale_dev, 4), MRL_ERR_MISALIGNED,
-                "%s: row_ticket and grad_scale_dev must be 4-byte aligned", fn);
+    MRL_REQUIRE(mrl::aligned(workspace, 16) && mrl::aligned(grad_scale_dev, 4), MRL_ERR_MISALIGNED,
+                "%s: workspace must be 16-byte and grad_scale_dev 4-byte aligned", fn);
     MRL_REQUIRE(mrl::row_sweep_supported(logits_dtype, vocab, logits, row_stride, dlogits, dlogits_row_stride, n_rows),
                 MRL_ERR_UNSUPPORTED,
-                "%s: needs 16-byte aligned rows, vocab %% %d == 0 and vocab <= %lld for this dtype (got vocab=%lld)", fn,
+                "%s: needs 16-byte aligned rows, vocab %% %d == 0 and vocab <= %lld for this dtype (got vocab=%lld); rows "
+                "above half of that are not swept in place", fn,
                 16 / eb, (long long)mrl_fused_max_vocab(logits_dtype), (long long)vocab);
     if (dlogits != logits) {
         const char* x = (const char*)logits;
@@ -792,10 +936,23 @@ extern "C" int mrl_fused_logprob_loss(const void* logits, int logits_dtype, int6
     a.labels = labels; a.labels_dtype = labels_dtype; a.inv_t = inv_temperature; a.row_ops = row_ops;
     a.has_old = has_old; a.clip_lo = clip_lo; a.clip_hi = clip_hi; a.kl_penalty = kl_penalty; a.kl_coef = kl_coef;
     a.entropy_coeff = entropy_coeff; a.grad_scale = grad_scale; a.grad_scale_dev = grad_scale_dev;
-    a.row_ticket = row_ticket; a.dlogits = dlogits; a.d_stride = dlogits_row_stride;
+    a.workspace = workspace; a.dlogits = dlogits; a.d_stride = dlogits_row_stride;
     a.logp = logp; a.entropy = entropy; a.row_terms = row_terms; a.with_entropy = (entropy != nullptr);
     a.stream = mrl::as_stream(stream);
-    const int nv = pick_nv(vocab / (16 / eb));
+    const int64_t n_vec = vocab / (16 / eb);
+    int nv = pick_nv(n_vec);
+    a.wide = (nv == 0);
+    a.half_elems = 0;
+    if (a.wide) {
+        a.half_elems = (n_vec + 1) / 2 * (16 / eb);
+        nv = pick_nv((n_vec + 1) / 2);
+    }
+    if (workspace != nullptr || a.wide) {
+        const int64_t need = mrl_fused_workspace_bytes(logits_dtype, n_rows, vocab);
+        MRL_REQUIRE(workspace != nullptr && workspace_bytes >= need, MRL_ERR_INVALID_ARG,
+                    "%s: workspace of %lld bytes, need %lld (rows of this width are cut in two halves that exchange "
+                    "their statistics through it)", fn, (long long)(workspace ? workspace_bytes : 0), (long long)need);
+    }
     switch (logits_dtype) {
         case MRL_F32: return fused_by_nv<MRL_F32>(nv, a);
         case MRL_BF16: return fused_by_nv<MRL_BF16>(nv, a);

@@ -51,8 +51,9 @@ SIGNATURES = {
     "mrl_fused_max_vocab": [_int],
     "mrl_fused_loss_prepare": [_int, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _int, _vp, _int, _vp, _vp, _vp, _vp, _int,
                                _int, _vp, _vp, _vp, _vp, _vp],
+    "mrl_fused_workspace_bytes": [_int, _i64, _i64],
     "mrl_fused_logprob_loss": [_vp, _int, _i64, _i64, _i64, _vp, _int, _f32, _vp, _int, _f32, _f32, _int, _f32, _f32,
-                               _f32, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp],
+                               _f32, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp],
     "mrl_fused_loss_reduce": [_vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _int, _vp, _int, _f32, _f32, _int, _f32,
                               _f32, _int, _f32, _vp, _vp, _vp],
     "mrl_scale_rows": [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp],
@@ -71,7 +72,7 @@ SIGNATURES = {
     "mrl_copy_bytes": [_vp, _vp, _i64, _vp],
     "mrl_bandwidth_probe": [_int, _vp, _vp, _i64, _i64, _vp],
 }
-_RESTYPES = {"mrl_last_error": ctypes.c_char_p, "mrl_fused_max_vocab": ctypes.c_int64,
+_RESTYPES = {"mrl_last_error": ctypes.c_char_p, "mrl_fused_workspace_bytes": ctypes.c_int64, "mrl_fused_max_vocab": ctypes.c_int64,
              "mrl_lmhead_workspace_bytes": ctypes.c_int64, "mrl_lmhead_static_max_tokens": ctypes.c_int64}
 
 _lib = None

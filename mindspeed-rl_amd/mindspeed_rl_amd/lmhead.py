@@ -92,7 +92,7 @@ class _FusedLmHeadLoss(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, hidden, weight, labels, batch, cfg):
-        from .loss import _expected_scale, _mask_args, _row_ticket
+        from .loss import _expected_scale, _mask_args, _sweep_workspace
         dev = _lib.require_device(hidden, weight, labels)
         hdim = hidden.shape[-1]
         h2d = hidden.detach().reshape(-1, hdim).contiguous()
@@ -139,7 +139,6 @@ class _FusedLmHeadLoss(torch.autograd.Function):
                   _lib.ptr(mask_t), mdt, cfg["seq_mean"], _lib.ptr(row_start), _lib.ptr(row_count),
                   _lib.ptr(seq_msum), _lib.ptr(row_ops), stream)
         grad_scale, scale_dev, applied = _expected_scale(cfg, dev)
-        ticket = _row_ticket(dev)
         # Rows whose mask is zero (prompts, padding, masked tokens) add nothing to the loss, to dWeight or
         # to their own dHidden: when they are more than a twentieth of the rows, the live rows are gathered
         # and only they go through the GEMMs.  The row count sizes the GEMMs, so it is read back (one
@@ -159,6 +158,7 @@ class _FusedLmHeadLoss(torch.autograd.Function):
             ent = torch.empty(max(n_rows, 1), dtype=torch.float32, device=dev) if want_ent else None
         chunk = max(1, min(int(cfg["chunk_rows"]), n_rows))
         logits = torch.empty((chunk, vocab), dtype=h2d.dtype, device=dev)
+        workspace, ws_bytes = _sweep_workspace(logits)
         d_hidden = torch.empty_like(h2d)
         d_weight32 = torch.zeros((vocab, hdim), dtype=torch.float32, device=dev)
         w_t = w.t()
@@ -175,8 +175,8 @@ class _FusedLmHeadLoss(torch.autograd.Function):
                 lab.data_ptr() + c0 * lab.element_size(), _lib.dtype_code(lab), cfg["inv_temperature"],
                 row_ops.data_ptr() + c0 * 32, 0 if old is None else 1, cfg["clip_lo"], cfg["clip_hi"], cfg["kl_penalty"],
                 cfg["kl_coef"], cfg["entropy_coeff"], grad_scale, _lib.ptr(scale_dev), _lib.ptr(z), vocab, None,
-                (ent.data_ptr() + c0 * 4) if want_ent else None, row_terms.data_ptr() + c0 * 32, _lib.ptr(ticket),
-                stream)
+                (ent.data_ptr() + c0 * 4) if want_ent else None, row_terms.data_ptr() + c0 * 32, _lib.ptr(workspace),
+                ws_bytes, stream)
             torch.mm(z, w if w_hv is None else w_hv.t(), out=d_hidden[c0:c1])    # dHidden_c = dlogits_c @ W
             # dW += dlogits_c^T @ hidden_c, accumulated in fp32 by the GEMM itself (no separate add pass,
             # no rounding of the chunk's product to bf16)

@@ -139,14 +139,16 @@ def policy_loss(log_prob, entropy, old_log_prob, ref_log_prob, advantages, mask=
 
 
 # ------------------------------------------------------------------------------------ fused sweep
-def fused_supported(output):
+def fused_supported(output, grad_inplace=False):
     """True if the row-in-registers kernel can take these logits: a floating dtype it knows,
-    16-byte aligned dense rows and a vocabulary that fits the register file."""
+    16-byte aligned dense rows and a vocabulary that fits the register files of one workgroup
+    (or of two, which is not available for an in-place gradient)."""
     if output.dtype not in (torch.float32, torch.bfloat16, torch.float16) or not output.is_cuda:
         return False
     vocab = output.shape[-1]
     per_vec = 16 // output.element_size()
-    if vocab % per_vec != 0 or vocab > _lib.load().mrl_fused_max_vocab(_lib.dtype_code(output)):
+    limit = _lib.load().mrl_fused_max_vocab(_lib.dtype_code(output))
+    if vocab % per_vec != 0 or vocab > (limit // 2 if grad_inplace else limit):
         return False
     return output.is_contiguous() and output.data_ptr() % 16 == 0
 
@@ -166,13 +168,16 @@ class GradScaleState:
         self.rescales = torch.zeros(1, dtype=torch.int32, device=device)
 
 
-def _row_ticket(dev):
-    """The persistent sweep's row counter: four bytes per call from torch's allocator (a sweep in
-    flight never shares its counter).  MRL_SWEEP_TICKET=0 makes the sweep walk rows with a fixed
-    stride instead (a tuning switch)."""
-    if os.environ.get("MRL_SWEEP_TICKET", "1") == "0":
-        return None
-    return torch.empty(1, dtype=torch.int32, device=dev)
+def _sweep_workspace(flat):
+    """(tensor or None, bytes): the fused sweep's workspace for these ``[rows, V]`` logits, from
+    torch's allocator per call (a sweep in flight never shares it): the row counter of the
+    persistent workgroups and, for rows that two workgroups hold, the half-row records.
+    MRL_SWEEP_TICKET=0 withholds it where it is optional, which makes the sweep walk rows with a
+    fixed stride instead (a tuning switch)."""
+    n_bytes = _lib.load().mrl_fused_workspace_bytes(_lib.dtype_code(flat), flat.shape[0], flat.shape[1])
+    if n_bytes <= 16 and os.environ.get("MRL_SWEEP_TICKET", "1") == "0":
+        return None, 0
+    return torch.empty(max(n_bytes, 16), dtype=torch.uint8, device=flat.device), n_bytes
 
 
 def _note_upstream(upstream, applied, state, stream):
@@ -270,13 +275,13 @@ class _FusedLogprobLoss(torch.autograd.Function):
                   _lib.ptr(mask_t), mdt, cfg["seq_mean"], _lib.ptr(row_start), _lib.ptr(row_count),
                   _lib.ptr(seq_msum), _lib.ptr(row_ops), stream)
         grad_scale, scale_dev, applied = _expected_scale(cfg, dev)
-        ticket = _row_ticket(dev)
+        workspace, ws_bytes = _sweep_workspace(flat)
         vocab_ops._timed_call("mrl_fused_logprob_loss", n_rows, dev, _lib.ptr(flat), _lib.dtype_code(flat), n_rows,
                               vocab, vocab, _lib.ptr(lab), _lib.dtype_code(lab), cfg["inv_temperature"],
                               _lib.ptr(row_ops), 0 if old is None else 1, cfg["clip_lo"], cfg["clip_hi"],
                               cfg["kl_penalty"], cfg["kl_coef"], cfg["entropy_coeff"], grad_scale,
                               _lib.ptr(scale_dev), _lib.ptr(dlogits), vocab, None, _lib.ptr(ent), _lib.ptr(row_terms),
-                              _lib.ptr(ticket), stream)
+                              _lib.ptr(workspace), ws_bytes, stream)
         _lib.call("mrl_fused_loss_reduce", _lib.ptr(row_terms), _lib.ptr(row_start), _lib.ptr(row_count), n_seq, width,
                   _lib.ptr(old), _lib.ptr(ref), _lib.ptr(adv), _lib.ptr(mask_t), mdt, _lib.ptr(resp), rdt,
                   cfg["clip_lo"], cfg["clip_hi"], cfg["kl_penalty"], cfg["kl_coef"], cfg["entropy_coeff"],
@@ -331,7 +336,8 @@ def _use_fused(output, kwargs):
     injected = vocab_ops.get_vocab_parallel()
     if injected is not None and injected is not vocab_ops.vocab_parallel_cross_entropy:
         return False            # a caller's own cross entropy must be the one that scores the rows
-    return torch.is_grad_enabled() and output.requires_grad and fused_supported(output)
+    return (torch.is_grad_enabled() and output.requires_grad
+            and fused_supported(output, bool(kwargs.get("grad_inplace", False))))
 
 
 def _fused_kwargs(kwargs, scale_state=None):

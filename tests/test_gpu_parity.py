@@ -1087,14 +1087,18 @@ def test_fused_sweep_specifics(dev):
     loss_o, _ = f.compute_loss(odd, bd_odd, fused=True, **kwd)
     (dz_odd,) = torch.autograd.grad(loss_o, odd)
     assert dz_odd.shape == odd.shape and torch.isfinite(loss_o).item()
-    assert _lib.load().mrl_fused_max_vocab(_lib.BF16) == 19 * 1024 * 8
-    assert _lib.load().mrl_fused_max_vocab(_lib.F32) == 19 * 1024 * 4
+    assert _lib.load().mrl_fused_max_vocab(_lib.BF16) == 2 * 19 * 1024 * 8
+    assert _lib.load().mrl_fused_max_vocab(_lib.F32) == 2 * 19 * 1024 * 4
 
 
 @pytest.mark.parametrize("dtype,vocab", [(torch.bfloat16, 152064), (torch.bfloat16, 129280), (torch.float32, 32000),
-                                         (torch.float16, 65536), (torch.float32, 77824), (torch.bfloat16, 64)])
+                                         (torch.float16, 65536), (torch.float32, 77824), (torch.bfloat16, 64),
+                                         (torch.float32, 152064), (torch.bfloat16, 262144), (torch.float32, 77828),
+                                         (torch.float16, 311296), (torch.float32, 100004)])
 def test_fused_sweep_vocab_sizes(dev, dtype, vocab):
-    """Every register-tile size of the fused kernel (4, 8, 12, 16, 19 vectors per thread)."""
+    """Every register-tile size of the fused kernel (4, 8, 12, 16, 19 vectors per thread), and rows
+    that two workgroups hold (fp32 logits of the configs[1] vocabulary, a 256 k vocabulary in bf16,
+    the first and the last width of that kind, an odd number of vectors)."""
     gen = torch.Generator().manual_seed(vocab)
     logits, b, kw, _, _ = _make_batch(gen, 1, 4, 3, 9, vocab, dtype, 3.0, 1, prompt_hi=2)
     meta = dict(clip_ratio=0.2, kl_coef=0.02, kl_penalty="low_var_kl", entropy_coeff=0.002)
@@ -1113,6 +1117,108 @@ def test_fused_sweep_vocab_sizes(dev, dtype, vocab):
         assert abs(got_stats[k] - want_stats[k]) <= TOL_LOSS_REL * abs(want_stats[k]) + 1e-6, k
     assert (dz.float().cpu() - dz_o).abs().max().item() < TOL_DLOGITS
     assert (dz.float().cpu() - dz_o).abs().max().item() <= 2 ** -8 * dz_o.abs().max().item() + 1e-9
+
+
+@pytest.mark.parametrize("dtype,vocab", [(torch.float32, 152064), (torch.bfloat16, 262144)])
+def test_fused_sweep_wide_rows(dev, dtype, vocab):
+    """Rows that two workgroups hold: more half rows than workgroups (tickets are recycled, partners
+    change), fused against the split kernels and an fp32 torch chain on the device; twice on one
+    stream and on two streams at once with a workspace each, then captured in a graph and replayed
+    with an eager sweep next to it - bit-identical to a lone call every time (both halves of a row
+    merge the two records in the same order)."""
+    rows = 700
+    gen = torch.Generator(device=dev).manual_seed(vocab)
+    cases = []
+    for c in range(2):
+        z = (torch.randn(rows, vocab, generator=gen, device=dev) * 3).to(dtype)
+        y = torch.randint(0, vocab, (rows,), generator=gen, device=dev)
+        y[5], y[6] = -1, vocab
+        ops = torch.zeros(rows, 8, device=dev)
+        ops[:, 0] = -torch.rand(rows, generator=gen, device=dev) * 8
+        ops[:, 1] = -torch.rand(rows, generator=gen, device=dev) * 8
+        ops[:, 2] = torch.randn(rows, generator=gen, device=dev)
+        ops[:, 3] = (torch.rand(rows, generator=gen, device=dev) > 0.2).float()
+        ops[:, 4] = 1.0 / rows
+        ops[:, 5] = 1.0 / rows
+        cases.append((z, y, ops))
+    lib = _lib.load()
+    ws_bytes = lib.mrl_fused_workspace_bytes(_lib.dtype_code(cases[0][0]), rows, vocab)
+    assert ws_bytes == 16 + rows * 32
+
+    def outputs():
+        return (torch.empty(rows, vocab, dtype=dtype, device=dev), torch.empty(rows, device=dev),
+                torch.empty(rows, 8, device=dev))
+
+    def sweep(case, out, ws, stream):
+        z, y, ops = case
+        dz, ent, terms = out
+        _lib.call("mrl_fused_logprob_loss", z.data_ptr(), _lib.dtype_code(z), rows, vocab, vocab, y.data_ptr(),
+                  _lib.I64, 1.0, ops.data_ptr(), 1, 0.8, 1.2, 3, 0.01, 0.002, 1.0, None, dz.data_ptr(), vocab, None,
+                  ent.data_ptr(), terms.data_ptr(), ws.data_ptr(), ws_bytes, stream)
+
+    spaces = [torch.full((ws_bytes,), 0xCD, dtype=torch.uint8, device=dev) for _ in range(3)]
+    want = []
+    for case in cases:
+        out = outputs()
+        sweep(case, out, spaces[0], _lib.stream(dev))
+        torch.cuda.synchronize()
+        want.append(out)
+        z, y, ops = case
+        dz, ent, terms = out
+        # the split kernels on the same rows (independent code): log-prob, entropy and the gradient
+        lp_s, ent_s, lse_s = mrl.vocab_logprob_entropy(z, y)
+        live = ops[:, 3] != 0
+        assert (ent[live] - ent_s[live]).abs().max().item() < 2e-5
+        assert not dz[~live].any().item() and dz[live].float().abs().amax(-1).min().item() > 0
+        # an fp32 torch chain on a slice of the rows
+        pick = torch.arange(0, rows, 23, device=dev)
+        zr = z[pick].float().requires_grad_()
+        logsm = torch.log_softmax(zr, -1)
+        yp = y[pick]
+        y_ok = (yp >= 0) & (yp < vocab)
+        lp_ref = torch.where(y_ok, logsm.gather(-1, yp.clamp(0, vocab - 1)[:, None])[:, 0],
+                             zr.max(-1).values.detach() - torch.logsumexp(zr, -1))
+        p = logsm.exp()
+        h_ref = -(p * logsm).sum(-1)
+        old, ref, adv, m, wpg, invtok = [ops[pick, k] for k in range(6)]
+        ratio = torch.exp(lp_ref - old)
+        pg = torch.maximum(-adv * ratio, -adv * ratio.clamp(0.8, 1.2))
+        kl = 0.5 * (lp_ref - ref) ** 2
+        loss = (pg * m * wpg).sum() + 0.01 * (kl * m * invtok).sum() - 0.002 * (h_ref * m * invtok).sum()
+        (g_ref,) = torch.autograd.grad(loss, zr)
+        scale = g_ref.abs().max().item()
+        rel = 2 ** -7 if dtype != torch.float32 else 2e-5
+        assert (dz[pick].float() - g_ref).abs().max().item() <= rel * scale + 1e-9
+        assert (lp_s[pick][m != 0] - lp_ref.detach()[m != 0]).abs().max().item() < 2e-4
+    # again on the same stream, and two sweeps at once on two streams
+    streams = [torch.cuda.Stream(device=dev) for _ in cases]
+    outs = [outputs() for _ in cases]
+    torch.cuda.synchronize()
+    for _ in range(3):
+        for case, out, s, ws in zip(cases, outs, streams, spaces):
+            sweep(case, out, ws, s.cuda_stream)
+    torch.cuda.synchronize()
+    for got, ref in zip(outs, want):
+        for a, b in zip(got, ref):
+            assert torch.equal(a, b)
+    # captured once, replayed next to an eager sweep
+    g_out = outputs()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        sweep(cases[0], g_out, spaces[2], _lib.stream(dev))
+    side = torch.cuda.Stream(device=dev)
+    for i in range(3):
+        for t in g_out:
+            t.zero_()
+        other = outputs()
+        torch.cuda.synchronize()
+        sweep(cases[1], other, spaces[1], side.cuda_stream)
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(g_out, want[0]):
+            assert torch.equal(a, b), i
+        for a, b in zip(other, want[1]):
+            assert torch.equal(a, b), i
 
 
 @pytest.mark.parametrize("dtype,vocab", [(torch.bfloat16, 8200), (torch.float32, 4100), (torch.float16, 40960)])
@@ -1338,7 +1444,7 @@ def _raw_fused_sweep(z, y, row_ops, dz, ent, terms, stream, ticket=None, scale_d
     rows, vocab = z.shape
     _lib.call("mrl_fused_logprob_loss", z.data_ptr(), _lib.dtype_code(z), rows, vocab, vocab, y.data_ptr(), _lib.I64,
               1.0, row_ops.data_ptr(), 1, 0.8, 1.2, 3, 0.01, 0.002, 1.0, _lib.ptr(scale_dev), dz.data_ptr(), vocab,
-              None, ent.data_ptr(), terms.data_ptr(), _lib.ptr(ticket), stream)
+              None, ent.data_ptr(), terms.data_ptr(), _lib.ptr(ticket), 0 if ticket is None else 16, stream)
 
 
 def _raw_fused_case(dev, seed, rows, vocab):
@@ -1364,7 +1470,7 @@ def test_fused_sweep_on_two_streams_and_in_a_graph(dev):
     which rows are taken."""
     rows, vocab = 1500, 8200
     cases = [_raw_fused_case(dev, 50 + i, rows, vocab) for i in range(2)]
-    tickets = [torch.full((1,), 12345, dtype=torch.int32, device=dev) for _ in range(3)]
+    tickets = [torch.full((4,), 12345, dtype=torch.int32, device=dev) for _ in range(3)]      # 16-byte workspaces
     want = []
     for z, y, ops in cases:
         dz, ent, terms = torch.empty_like(z), torch.empty(rows, device=dev), torch.empty(rows, 8, device=dev)
@@ -1374,7 +1480,7 @@ def test_fused_sweep_on_two_streams_and_in_a_graph(dev):
         assert dz.float().abs().max().item() > 0 and not dz[ops[:, 3] == 0].any().item()
         # every row was handed out exactly once: the counter ends at rows + workgroups
         cus = torch.cuda.get_device_properties(dev).multi_processor_count
-        assert int(tickets[0].item()) == rows + cus
+        assert int(tickets[0][0].item()) == rows + cus
     # no counter: rows are walked with a fixed stride
     z, y, ops = cases[0]
     plain = (torch.empty_like(z), torch.empty(rows, device=dev), torch.empty(rows, 8, device=dev))
@@ -1592,8 +1698,13 @@ def _random_fused_case(i, rnd):
     nvec = rnd.choice([rnd.randint(1, 64), rnd.randint(1, max_vec),
                        rnd.choice([1024 * k + d for k in (4, 8, 12, 16, 19) for d in (-1, 0, 1)])])
     nvec = max(1, min(nvec, max_vec))
-    vocab = nvec * per
     rows = rnd.choice([1, 3, 257, 511, 513, 600, 777, 1100])
+    if i % 6 == 5:
+        # a row that two workgroups hold: between one and two register files wide
+        nvec = rnd.choice([max_vec + 1, 2 * max_vec, 2 * max_vec - 1, rnd.randint(max_vec + 1, 2 * max_vec),
+                           2 * 1024 * rnd.choice([10, 12, 13, 16]) + rnd.choice([-1, 0, 1])])
+        rows = rnd.choice([1, 2, 129, 300, 515])
+    vocab = nvec * per
     inv_t = rnd.choice([1.0, 0.7, 1.3])
     ent_c = rnd.choice([0.0, 0.003])
     dev = torch.device("cuda:0")
@@ -1614,12 +1725,15 @@ def _random_fused_case(i, rnd):
     ent = torch.zeros(rows, device=dev)
     lp = torch.zeros(rows, device=dev)
     terms = torch.zeros(rows, 8, device=dev)
-    ticket = torch.zeros(1, dtype=torch.int32, device=dev)         # every other case walks rows with a fixed stride
+    # every other narrow case walks rows with a fixed stride (no workspace); wide rows need theirs
+    ws_bytes = _lib.load().mrl_fused_workspace_bytes(_lib.dtype_code(z), rows, vocab)
+    assert ws_bytes >= 16
+    workspace = torch.full((ws_bytes,), 0xAB, dtype=torch.uint8, device=dev) if (i % 2 == 0 or ws_bytes > 16) else None
     clip_lo, clip_hi, kl_kind, kl_coef = 0.8, 1.25, 4, 0.01
     _lib.call("mrl_fused_logprob_loss", z.data_ptr(), _lib.dtype_code(z), rows, vocab, vocab, y.data_ptr(), _lib.I64,
               inv_t, ops.data_ptr(), 1, clip_lo, clip_hi, kl_kind, kl_coef, ent_c, 1.0, None, dz.data_ptr(), vocab,
               lp.data_ptr(), ent.data_ptr() if ent_c != 0 else None, terms.data_ptr(),
-              ticket.data_ptr() if i % 2 == 0 else None, _lib.stream(dev))
+              _lib.ptr(workspace), ws_bytes if workspace is not None else 0, _lib.stream(dev))
     zr = (z.float() * inv_t).requires_grad_()
     logsm = torch.log_softmax(zr, -1)
     y_ok = (y >= 0) & (y < vocab)
@@ -2613,7 +2727,11 @@ def test_vocabulary_shards_merge_to_the_full_sweep(dev, dtype, bounds):
     ({"MRL_LMHEAD_V2": "0", "MRL_SWEEP_TICKET": "0"},
      "test_lmhead_logprob_forward or test_lmhead_forward_random_shapes or test_fused_lmhead_policy_loss or "
      "test_fused_sweep_persistent or test_persistent_row_sweeps"),
-], ids=["per_row_sweep_and_loop_backward", "first_lmhead_loop_and_fixed_stride"])
+    # no waiting at all for the other half of a wide row: every workgroup computes the other half's
+    # statistics itself from memory (the path a workgroup takes when its partner is late)
+    ({"MRL_WIDE_SPIN_LIMIT": "0"}, "test_fused_sweep_wide_rows or test_fused_sweep_vocab_sizes or "
+                                   "test_fused_sweep_random_shapes"),
+], ids=["per_row_sweep_and_loop_backward", "first_lmhead_loop_and_fixed_stride", "wide_rows_without_waiting"])
 def test_library_switches_in_child_processes(dev, switches, subset):
     """The library reads its tuning switches once per process, so the kernels behind them (one workgroup
     per row instead of persistent workgroups, the loop backward for every row length, the first

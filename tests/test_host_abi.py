@@ -100,15 +100,26 @@ def test_argument_validation_launches_nothing():
                                    p, None) == -1                                          # kl enum
     assert lib.mrl_copy_bytes(p, p + 1024, 24, None) == -1
     # fused sweep: a vocabulary the registers cannot hold, one that is not a whole number of vectors
-    assert lib.mrl_fused_max_vocab(_lib.BF16) == 155648 and lib.mrl_fused_max_vocab(_lib.I64) == 0
-    for vocab in (155656, 1003):
+    assert lib.mrl_fused_max_vocab(_lib.BF16) == 311296 and lib.mrl_fused_max_vocab(_lib.I64) == 0
+    assert lib.mrl_fused_max_vocab(_lib.F32) == 155648
+    assert lib.mrl_fused_workspace_bytes(_lib.BF16, 100, 152064) == 16
+    assert lib.mrl_fused_workspace_bytes(_lib.F32, 100, 152064) == 16 + 100 * 32
+    assert lib.mrl_fused_workspace_bytes(_lib.BF16, 100, 311304) == 0
+    # a row that two workgroups hold needs the workspace, and cannot be swept in place
+    rc = lib.mrl_fused_logprob_loss(p, _lib.F32, 2, 152064, 152064, p, _lib.I64, 1.0, p, 1, 0.8, 1.2, 4, 0.0, 0.0, 1.0,
+                                    None, p + (1 << 30), 152064, None, None, p, None, 0, None)
+    assert rc == -1 and b"workspace" in lib.mrl_last_error()
+    rc = lib.mrl_fused_logprob_loss(p, _lib.F32, 2, 152064, 152064, p, _lib.I64, 1.0, p, 1, 0.8, 1.2, 4, 0.0, 0.0, 1.0,
+                                    None, p, 152064, None, None, p, p, 1 << 20, None)
+    assert rc == -2 and b"in place" in lib.mrl_last_error()
+    for vocab in (311304, 1003):
         rc = lib.mrl_fused_logprob_loss(p, _lib.BF16, 2, vocab, vocab, p, _lib.I64, 1.0, p, 1, 0.8, 1.2, 4, 0.0, 0.0,
-                                        1.0, None, p, vocab, None, None, p, None, None)
+                                        1.0, None, p, vocab, None, None, p, None, 0, None)
         assert rc == -2, vocab
     assert lib.mrl_fused_logprob_loss(p, _lib.BF16, 2, 64, 64, p, _lib.I64, 1.0, None, 1, 0.8, 1.2, 4, 0.0, 0.0, 1.0,
-                                      None, p, 64, None, None, p, None, None) == -1       # no row operands
+                                      None, p, 64, None, None, p, None, 0, None) == -1    # no row operands
     assert lib.mrl_fused_logprob_loss(p, _lib.BF16, 2, 64, 64, p, _lib.I64, 1.0, p, 1, 0.8, 1.2, 4, 0.0, 0.0, 1.0,
-                                      None, p, 64, None, None, p, p + 2, None) == -3      # misaligned row counter
+                                      None, p, 64, None, None, p, p + 2, 16, None) == -3  # misaligned workspace
     assert lib.mrl_scale_rows(p, _lib.I32, 2, 64, 64, p, p, None) == -2
     assert lib.mrl_scale_rows(p, _lib.BF16, 2, 64, 64, p, None, None) == -1                # no applied scale
     assert lib.mrl_grad_scale_note(p, None, None, None, None) == -1
