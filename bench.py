@@ -318,20 +318,53 @@ def run_lmhead_train(args):
         dh, dw = torch.autograd.grad(loss, [h, wt])
         return loss, stats, dh, dw
 
+    from mindspeed_rl_amd import lmhead
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
     vocab_ops.kernel_events = []
+    lmhead.kernel_events = []
     t0 = time.perf_counter()
     for _ in range(args.steps):
         loss, stats, dh, dw = step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     events, vocab_ops.kernel_events = vocab_ops.kernel_events, None
+    gemm_events, lmhead.kernel_events = lmhead.kernel_events, None
     sweep_ms = sum(s.elapsed_time(e) for (_, s, e, _) in events) / args.steps
+    logits_ms = sum(s.elapsed_time(e) for (n, s, e, _) in gemm_events if n == "mrl_lmhead_logits") / args.steps
+    bwd_ms = sum(s.elapsed_time(e) for (n, s, e, _) in gemm_events if n == "mrl_lmhead_logprob_bwd") / args.steps
     ms = elapsed * 1e3 / args.steps
     flops = 6.0 * total * vocab * hdim                       # forward GEMM + dHidden GEMM + dW GEMM
     tflops = flops / (ms * 1e-3) / 1e12
+    del dh, dw
+    # the library's kernels for the same three products of one chunk (hipBLASLt through torch), timed
+    # alone and scaled to the step: a comparison figure, not part of the path
+    rows = min(args.chunk_rows, total)
+    h_c = hidden[0, :rows]
+    z = torch.empty(rows, vocab, dtype=torch.bfloat16, device=dev)
+    w_hv = weight.t().contiguous()
+    dh_c = torch.empty(rows, hdim, dtype=torch.bfloat16, device=dev)
+    dw32 = torch.zeros(vocab, hdim, dtype=torch.float32, device=dev)
+    h_t = h_c.t().contiguous()
+
+    def library_products():
+        torch.mm(h_c, weight.t(), out=z)
+        torch.mm(z, w_hv.t(), out=dh_c)
+        try:
+            torch.addmm(dw32, z.t(), h_t.t(), out_dtype=torch.float32, out=dw32)
+        except (TypeError, RuntimeError):
+            dw32.add_(torch.mm(z.t(), h_t.t()))
+
+    library_products()
+    s_ev, e_ev = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s_ev.record()
+    for _ in range(3):
+        library_products()
+    e_ev.record()
+    torch.cuda.synchronize()
+    lib_chunk_ms = s_ev.elapsed_time(e_ev) / 3
+    del z, w_hv, dh_c, dw32, h_t
     result = {
         "metric": "tokens/sec for fused lm_head + logprob + GRPO loss fwd+bwd (dHidden, dW); TFLOP/s as % of bf16 dense peak",
         "value": tokens / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -339,10 +372,17 @@ def run_lmhead_train(args):
         "data": "synthetic",
         "config": {"workload": "configs[3]: hidden [%d,3584] x W [152064,3584], GRPO loss as configs[1], logits only for "
                                "%d rows at a time" % (total, args.chunk_rows), "response_tokens": tokens, "accumulate": "f32",
-                   "gemm": "library (hipBLASLt via torch.mm)", "sweep": "fused_sweep_persistent_kernel in place"},
-        "roofline": {"kernel": "whole step (3 library GEMMs + fused sweeps)", "bound": "mfma", "achieved": tflops,
-                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": None, "flops_per_step": flops, "fused_sweeps_ms_per_step": sweep_ms},
+                   "products": "hand-written gfx950 MFMA kernels (gemm_nt_kernel: logits, dHidden, dW)",
+                   "sweep": "fused_sweep_persistent_kernel in place"},
+        "roofline": {"kernel": "whole step (3 matrix products per chunk + fused sweeps + transposed copies)",
+                     "bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "flops_per_step": flops,
+                     "fused_sweeps_ms_per_step": sweep_ms, "logits_products_ms_per_step": logits_ms,
+                     "backward_products_ms_per_step": bwd_ms},
+        "library_products_comparison": {
+            "what": "torch.mm / addmm (hipBLASLt) for the same three products of one %d-row chunk, timed alone" % rows,
+            "ms_per_chunk": lib_chunk_ms, "scaled_to_step_ms": lib_chunk_ms * total / rows,
+            "hand_written_products_ms_per_step": logits_ms + bwd_ms},
         "loss": float(loss.detach()), "stats": stats[1:6],
     }
     print(json.dumps(result), flush=True)

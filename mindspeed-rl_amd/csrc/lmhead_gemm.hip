@@ -1,0 +1,457 @@
+// bf16 matrix products of the lm_head training step for gfx950, on the tile loop of the fused
+// lm_head forward (lmhead.hip): operands go from global memory straight into LDS
+// (buffer_load ... lds), two 64 KiB stages, XOR-swizzled 16-byte chunks, v_mfma_f32_32x32x16_bf16,
+// fragments of the next sub-step requested before the MFMAs of the current one.
+//
+// One kernel covers the three products of the step, because each of them can be put in the form
+//
+//     out[n][m] (+)= sum_k A[m][k] * B[n][k]          A: [M, K], B: [N, K], both with k contiguous
+//
+// (the MFMA's M is the fast dimension of the output: in the 32x32 result layout a lane owns ONE
+// column n and 4 consecutive rows m at a time, i.e. 8 contiguous bytes of bf16 or 16 of fp32):
+//
+//     logits[t][v]  = sum_h W[v][h]      * hidden[t][h]      A = W,         B = hidden chunk
+//     dHidden[t][h] = sum_v Wt[h][v]     * dlogits[t][v]     A = W^T copy,  B = dlogits chunk
+//     dW[v][h]     += sum_t hiddenT[h][t] * dlogitsT[v][t]    A = hidden^T,  B = dlogits^T (copies)
+//
+// The transposed copies are made by transpose_bf16_kernel; their padded tails are zero so that the
+// k dimension can always be walked in whole steps of 64.
+//
+// Work distribution: one persistent 512-thread workgroup per CU (2 x 4 wavefronts, wavefront tile
+// 128 x 64) walks output tiles of 256 x 256.  Tiles are numbered so that 32 consecutive numbers are
+// 8 tiles along m by 4 along n, and the 32 workgroups that share an XCD (and its L2) take 32
+// consecutive numbers at a time: the 4 that stream the same A tile and the 8 that stream the same
+// B tile run side by side (see tile_coords for the order of the groups of 32).  The loop runs over
+// the flattened (tile, k-step) sequence of a workgroup, so the first loads of its next tile are in
+// flight while the current one is stored.
+#include <stdlib.h>
+
+#include "lmhead_gemm.h"
+#include "mrl_internal.h"
+#include "vocab_common.h"
+
+namespace {
+
+using namespace mrl_vocab;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+// Wavefront layout of the 256 x 256 tile: 2 wavefronts along m (128 rows of A each) by kWavesN along
+// n.  With 4 along n (512 threads, two wavefronts per SIMD) a wavefront owns 128 x 64 = 4 x 2 MFMA
+// blocks; with 2 along n (256 threads, one wavefront per SIMD) 128 x 128 = 4 x 4 blocks in 256
+// accumulator registers, which needs a third fewer fragment bytes from LDS per flop.
+#ifndef MRL_GEMM_WAVES_N
+#define MRL_GEMM_WAVES_N 4
+#endif
+constexpr int kWavesN = MRL_GEMM_WAVES_N;
+constexpr int kWaves = 2 * kWavesN;
+constexpr int kThreads = 64 * kWaves;
+constexpr int kTB = 8 / kWavesN;                 // 32-row blocks of B per wavefront
+constexpr int kLoadsPerWave = 32 / kWaves;       // 8-row groups of an operand that a wavefront brings in
+constexpr int BM = 256;                          // rows of A per tile
+constexpr int BN = 256;                          // rows of B per tile
+constexpr int BK = 64;                           // k elements per LDS stage
+constexpr int kOperandBytes = 256 * BK * 2;      // one operand of one stage: 256 rows x 128 bytes
+constexpr int kStageBytes = 2 * kOperandBytes;   // A then B
+constexpr int kLdsStages = 2 * kStageBytes;      // two stages
+constexpr int kLdsTurn = 32 * 1024;              // where the wavefronts turn their result blocks (store_tile)
+constexpr int kLdsBytes = kLdsStages + kLdsTurn;
+constexpr int kTilesAlongN = 4;                  // tiles along n in a group of consecutive tile numbers
+
+// Element offset (row * ld + column, without the k-step) of the chunk that lane `lane` of wavefront
+// `wave` brings in with its load j (0..3) of an operand tile with `rows_valid` rows left (rows beyond
+// are clamped to the last valid one; their products are never stored).  Physical slot of a 16-byte
+// chunk inside its 256-byte pair of rows: logical slot ^ (pair & 15), logical = (row & 1) * 8 + chunk.
+__device__ __forceinline__ int64_t stage_src_offset(int wave, int lane, int j, int64_t ld, int rows_valid) {
+    const int phys_row = (wave * kLoadsPerWave + j) * 8 + (lane >> 3);
+    const int pair = phys_row >> 1;
+    const int slot = ((phys_row & 1) << 3) | (lane & 7);
+    const int logical = slot ^ (pair & 15);
+    int row = 2 * pair + (logical >> 3);
+    if (row >= rows_valid) row = rows_valid - 1;
+    return (int64_t)row * ld + (logical & 7) * 8;
+}
+
+struct TileGrid {
+    int tiles_m, tiles_n;
+    int64_t total;
+};
+
+// Tile number -> (tile along m, tile along n).  Tiles are numbered panel by panel, a panel being
+// kPanelM tiles along m by all tiles along n; inside a panel 32 consecutive numbers are 8 (m) x 4 (n)
+// tiles, and consecutive groups of 32 walk along n.  The 8 XCDs therefore work on the same 8 tiles of
+// A at the same time (one fetch from memory serves all of them) with 4 tiles of B each, and a
+// workgroup keeps its tile of A from one of its tiles to the next.
+constexpr int kPanelM = 8;
+__device__ __forceinline__ void tile_coords(const TileGrid& g, int64_t t, int& tm, int& tn) {
+    const int64_t per_panel = (int64_t)kPanelM * g.tiles_n;
+    const int p = (int)(t / per_panel);
+    const int idx = (int)(t - (int64_t)p * per_panel);
+    const int pm = min(kPanelM, g.tiles_m - p * kPanelM);       // rows of tiles in this panel
+    const int ng = idx / (pm * kTilesAlongN);
+    const int rem = idx - ng * (pm * kTilesAlongN);
+    const int width = min(kTilesAlongN, g.tiles_n - ng * kTilesAlongN);
+    tm = p * kPanelM + rem / width;
+    tn = ng * kTilesAlongN + rem % width;
+}
+
+// kAccumulate: out is fp32 and the product is added to it; else out is bf16 and overwritten.
+template <bool kAccumulate>
+__global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(const uint16_t* __restrict__ A, int64_t lda, int M,
+                                                              const uint16_t* __restrict__ B, int64_t ldb, int N, int K,
+                                                              void* __restrict__ out, int64_t ldo) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wv = wave / kWavesN, wt = wave % kWavesN;
+
+    TileGrid grid;
+    grid.tiles_m = (M + BM - 1) / BM;
+    grid.tiles_n = (N + BN - 1) / BN;
+    grid.total = (int64_t)grid.tiles_m * grid.tiles_n;
+    // workgroups are dealt round-robin to the 8 XCDs: the gridDim / 8 workgroups of an XCD take
+    // consecutive tile numbers
+    const int per_xcd = gridDim.x >> 3;
+    const int64_t first_tile = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    const int64_t tile_stride = gridDim.x;
+    if (first_tile >= grid.total) return;
+    const int my_tiles = (int)((grid.total - 1 - first_tile) / tile_stride) + 1;
+    const int n_ksteps = K / BK;
+    const int n_stages = my_tiles * n_ksteps;
+
+    // ---- loader state: the tile whose stages are being requested
+    int64_t load_tile = first_tile;
+    int load_k = 0;
+    int a_off[kLoadsPerWave], b_off[kLoadsPerWave];
+    mrl::rsrc_t a_rsrc, b_rsrc;
+    auto set_load_tile = [&](int64_t t) {
+        int tm, tn;
+        tile_coords(grid, t, tm, tn);
+        const int rows_a = min(BM, M - tm * BM), rows_b = min(BN, N - tn * BN);
+#pragma unroll
+        for (int j = 0; j < kLoadsPerWave; ++j) {
+            a_off[j] = (int)(stage_src_offset(wave, lane, j, lda, rows_a) * 2);
+            b_off[j] = (int)(stage_src_offset(wave, lane, j, ldb, rows_b) * 2);
+        }
+        // one descriptor per tile: byte offsets inside a tile stay below 2^32 for any operand size
+        a_rsrc = mrl::make_rsrc(A + (int64_t)tm * BM * lda, 0xffffffffu);
+        b_rsrc = mrl::make_rsrc(B + (int64_t)tn * BN * ldb, 0xffffffffu);
+    };
+    auto issue_next = [&](int buf) {
+        const uint32_t k_bytes = (uint32_t)(load_k * BK * 2);
+        unsigned char* dst = smem + buf * kStageBytes + (wave * kLoadsPerWave) * 1024;
+#pragma unroll
+        for (int j = 0; j < kLoadsPerWave; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (void __attribute__((address_space(3)))*)(dst + j * 1024), 16,
+                                                 a_off[j], k_bytes, 0, 0);
+#pragma unroll
+        for (int j = 0; j < kLoadsPerWave; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc,
+                                                 (void __attribute__((address_space(3)))*)(dst + kOperandBytes + j * 1024),
+                                                 16, b_off[j], k_bytes, 0, 0);
+        if (++load_k == n_ksteps) {
+            load_k = 0;
+            load_tile += tile_stride;
+            if (load_tile < grid.total) set_load_tile(load_tile);
+        }
+    };
+
+    // fragment addresses: row (lane & 31) of a 32-row block, chunk 2 ks + (lane >> 5)
+    const int frag_pair = (lane & 31) >> 1;
+    const int frag_slot = (((lane & 1) << 3) | (lane >> 5)) ^ frag_pair;          // ^ (2 ks) per k sub-step
+    const int a_frag = (wv * 64) * 256 + frag_pair * 256;                          // + vb * 16 * 256
+    const int b_frag = kOperandBytes + (wt * 16 * kTB) * 256 + frag_pair * 256;    // + tb * 16 * 256
+    struct Frags {
+        bf16x8 a[4], b[kTB];
+    };
+    auto read_frags = [&](Frags& f, const unsigned char* stage, int ks) {
+        const int slot_bytes = (frag_slot ^ (2 * ks)) * 16;
+#pragma unroll
+        for (int vb = 0; vb < 4; ++vb)
+            f.a[vb] = *reinterpret_cast<const bf16x8*>(stage + a_frag + vb * 16 * 256 + slot_bytes);
+#pragma unroll
+        for (int tb = 0; tb < kTB; ++tb)
+            f.b[tb] = *reinterpret_cast<const bf16x8*>(stage + b_frag + tb * 16 * 256 + slot_bytes);
+    };
+    floatx16 acc[4][kTB];
+    auto zero_acc = [&]() {
+#pragma unroll
+        for (int vb = 0; vb < 4; ++vb)
+#pragma unroll
+            for (int tb = 0; tb < kTB; ++tb)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc[vb][tb][i] = 0.f;
+    };
+    auto mma = [&](const Frags& f) {
+#pragma unroll
+        for (int vb = 0; vb < 4; ++vb)
+#pragma unroll
+            for (int tb = 0; tb < kTB; ++tb)
+                acc[vb][tb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[vb], f.b[tb], acc[vb][tb], 0, 0, 0);
+    };
+    // The finished tile.  A lane holds column n = lane & 31 of each 32 x 32 block and rows
+    // (i / 4) * 8 + (lane >> 5) * 4 + (i & 3), i.e. four runs of 4 consecutive m: stored like that, a
+    // store instruction would touch 32 output rows with 16 bytes each.  Each wavefront therefore turns
+    // its blocks through a private slice of LDS (the 32 KiB the two stages leave free): [32 n][128 bytes
+    // of m] at a time, 16-byte chunks XOR-swizzled by the row, written in the MFMA layout and read back
+    // as 8 lanes x 16 bytes per output row, so that every store covers whole 128-byte lines.
+    unsigned char* turn = smem + kLdsStages + wave * (kLdsTurn / kWaves);
+    auto store_tile = [&](int64_t t) {
+        int tm, tn;
+        tile_coords(grid, t, tm, tn);
+        const int row_w = lane & 31, half = lane >> 5;           // writer: its n, its run of 4 inside a run of 8
+        const int row_r = lane >> 3, chunk_r = lane & 7;          // reader: n within a group of 8, 16-byte chunk
+        constexpr int kBlocksPerPass = kAccumulate ? 1 : 2;       // 32 fp32 or 64 bf16 entries of m are 128 bytes
+#pragma unroll
+        for (int tb = 0; tb < kTB; ++tb) {
+            const int n0 = tn * BN + wt * (32 * kTB) + tb * 32;
+#pragma unroll
+            for (int vb0 = 0; vb0 < 4; vb0 += kBlocksPerPass) {
+                const int m0 = tm * BM + wv * 128 + vb0 * 32;
+#pragma unroll
+                for (int vbi = 0; vbi < kBlocksPerPass; ++vbi) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const floatx16& c = acc[vb0 + vbi][tb];
+                        if (kAccumulate) {
+                            const int chunk = (q * 2 + half) ^ (row_w & 7);
+                            *reinterpret_cast<float4*>(turn + row_w * 128 + chunk * 16) =
+                                make_float4(c[q * 4 + 0], c[q * 4 + 1], c[q * 4 + 2], c[q * 4 + 3]);
+                        } else {
+                            const int chunk = (vbi * 4 + q) ^ (row_w & 7);
+                            uint2 w;
+                            w.x = Elem<MRL_BF16>::pack2(c[q * 4 + 0], c[q * 4 + 1]);
+                            w.y = Elem<MRL_BF16>::pack2(c[q * 4 + 2], c[q * 4 + 3]);
+                            *reinterpret_cast<uint2*>(turn + row_w * 128 + chunk * 16 + half * 8) = w;
+                        }
+                    }
+                }
+                __builtin_amdgcn_s_waitcnt(0xC07F);            // lgkmcnt(0): the slice is written
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int row = g * 8 + row_r;
+                    const u32x4 v = *reinterpret_cast<const u32x4*>(turn + row * 128 + ((chunk_r ^ (row & 7)) * 16));
+                    const int n = n0 + row;
+                    const int m = m0 + chunk_r * (kAccumulate ? 4 : 8);
+                    if (n < N && m < M) {                      // M % 8 == 0: a chunk is inside or outside
+                        if (kAccumulate) {
+                            float4* p = reinterpret_cast<float4*>(reinterpret_cast<float*>(out) + (int64_t)n * ldo + m);
+                            float4 c = *p;
+                            c.x += __uint_as_float(v.x);
+                            c.y += __uint_as_float(v.y);
+                            c.z += __uint_as_float(v.z);
+                            c.w += __uint_as_float(v.w);
+                            *p = c;
+                        } else {
+                            *reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(out) + (int64_t)n * ldo + m) = v;
+                        }
+                    }
+                }
+                __builtin_amdgcn_s_waitcnt(0xC07F);            // the slice has been read: it may be rewritten
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+
+    Frags f0, f1;
+    set_load_tile(load_tile);
+    issue_next(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0): stage 0 has landed
+    __syncthreads();
+    if (n_stages > 1) issue_next(1);
+    read_frags(f0, smem, 0);
+    int stage_idx = 0;
+    for (int mine = 0; mine < my_tiles; ++mine) {
+        zero_acc();
+        for (int kstep = 0; kstep < n_ksteps; ++kstep, ++stage_idx) {
+            const int buf = stage_idx & 1;
+            const unsigned char* stage = smem + buf * kStageBytes;
+            // software pipeline: the fragments of sub-step ks+1 are requested before the MFMAs of ks
+            read_frags(f1, stage, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(f0);
+            __builtin_amdgcn_sched_barrier(0);
+            read_frags(f0, stage, 2);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(f1);
+            __builtin_amdgcn_sched_barrier(0);
+            read_frags(f1, stage, 3);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(f0);
+            __builtin_amdgcn_sched_barrier(0);
+            // The last fragments of this stage are in registers and the next stage has landed: after the
+            // barrier this buffer may be overwritten, and the first fragments of the next stage are
+            // requested before the last MFMAs of this one are issued.  The barrier and the read are
+            // unconditional (after the last stage the read fetches unused bytes of the other buffer).
+            __builtin_amdgcn_s_waitcnt(0x0070);        // vmcnt(0) lgkmcnt(0)
+            __syncthreads();
+            read_frags(f0, smem + (buf ^ 1) * kStageBytes, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(f1);
+            __builtin_amdgcn_sched_barrier(0);
+            // the stage after next goes into the buffer that the barrier has just freed
+            if (stage_idx + 2 < n_stages) issue_next(buf);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        store_tile(first_tile + (int64_t)mine * tile_stride);
+    }
+}
+
+// dst[c][r] = src[r][c] for r < rows, c < cols; dst has `dst_rows` >= cols rows of `ld_dst` >= rows
+// entries, and everything outside the transposed block (the padding that lets a product walk k in
+// whole steps) is written as zero.  64 x 64 tiles through LDS, 16-bit elements.
+__global__ __launch_bounds__(256) void transpose_bf16_kernel(const uint16_t* __restrict__ src, int64_t ld_src, int rows,
+                                                             int cols, uint16_t* __restrict__ dst, int64_t ld_dst,
+                                                             int dst_rows) {
+    __shared__ uint16_t tile[64][66];
+    const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int r = r0 + ty * 16 + i, c = c0 + tx;
+        tile[ty * 16 + i][tx] = (r < rows && c < cols) ? src[(int64_t)r * ld_src + c] : (uint16_t)0;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int c = c0 + ty * 16 + i, r = r0 + tx;
+        if (c < dst_rows && r < ld_dst) dst[(int64_t)c * ld_dst + r] = tile[tx][ty * 16 + i];
+    }
+}
+
+int persistent_grid() {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    return n & ~7;          // a whole number of workgroups per XCD
+}
+
+}  // namespace
+
+namespace mrl {
+
+int gemm_nt_bf16(const char* fn, const void* a, int64_t lda, int64_t m, const void* b, int64_t ldb, int64_t n, int64_t k,
+                 void* out, int64_t ldo, bool accumulate_f32, hipStream_t stream) {
+    MRL_REQUIRE(m > 0 && n > 0 && k > 0 && k % BK == 0 && m % 8 == 0, MRL_ERR_UNSUPPORTED,
+                "%s: product of m=%lld n=%lld k=%lld (k must be a multiple of %d, m of 8)", fn, (long long)m, (long long)n,
+                (long long)k, BK);
+    MRL_REQUIRE(m <= 0x7fffffffLL && n <= 0x7fffffffLL && k <= 0x7fffffffLL, MRL_ERR_UNSUPPORTED, "%s: size out of range",
+                fn);
+    MRL_REQUIRE(lda >= k && ldb >= k && ldo >= m && lda % 8 == 0 && ldb % 8 == 0 && ldo % 8 == 0, MRL_ERR_INVALID_ARG,
+                "%s: leading dimensions lda=%lld ldb=%lld ldo=%lld", fn, (long long)lda, (long long)ldb, (long long)ldo);
+    MRL_REQUIRE(256 * lda * 2 < (1LL << 31) && 256 * ldb * 2 < (1LL << 31), MRL_ERR_UNSUPPORTED,
+                "%s: a tile of 256 rows must stay below 2 GiB", fn);
+    MRL_REQUIRE(aligned(a, 16) && aligned(b, 16) && aligned(out, 16), MRL_ERR_MISALIGNED,
+                "%s: operands must be 16-byte aligned", fn);
+    const int grid = persistent_grid();
+    MRL_REQUIRE(grid >= 8, MRL_ERR_LAUNCH, "%s: cannot query the device", fn);
+    static const hipError_t attr0 = hipFuncSetAttribute((const void*)gemm_nt_kernel<false>,
+                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    static const hipError_t attr1 = hipFuncSetAttribute((const void*)gemm_nt_kernel<true>,
+                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    MRL_REQUIRE(attr0 == hipSuccess && attr1 == hipSuccess, MRL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS", fn,
+                kLdsBytes);
+    if (accumulate_f32) {
+        hipLaunchKernelGGL(gemm_nt_kernel<true>, dim3((unsigned)grid), dim3(kThreads), kLdsBytes, stream,
+                           (const uint16_t*)a, lda, (int)m, (const uint16_t*)b, ldb, (int)n, (int)k, out, ldo);
+    } else {
+        hipLaunchKernelGGL(gemm_nt_kernel<false>, dim3((unsigned)grid), dim3(kThreads), kLdsBytes, stream,
+                           (const uint16_t*)a, lda, (int)m, (const uint16_t*)b, ldb, (int)n, (int)k, out, ldo);
+    }
+    return check_launch(fn);
+}
+
+int transpose_bf16(const char* fn, const void* src, int64_t ld_src, int64_t rows, int64_t cols, void* dst, int64_t ld_dst,
+                   int64_t dst_rows, hipStream_t stream) {
+    MRL_REQUIRE(rows >= 0 && cols >= 0 && ld_src >= cols && ld_dst >= rows && dst_rows >= cols, MRL_ERR_INVALID_ARG,
+                "%s: transpose of %lld x %lld (ld %lld) into %lld x %lld", fn, (long long)rows, (long long)cols,
+                (long long)ld_src, (long long)dst_rows, (long long)ld_dst);
+    if (dst_rows == 0 || ld_dst == 0) return MRL_OK;
+    const int64_t gx = (ld_dst + 63) / 64, gy = (dst_rows + 63) / 64;
+    MRL_REQUIRE(gx <= 0x7fffffffLL && gy <= 65535, MRL_ERR_UNSUPPORTED, "%s: grid too large", fn);
+    hipLaunchKernelGGL(transpose_bf16_kernel, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, stream,
+                       (const uint16_t*)src, ld_src, (int)rows, (int)cols, (uint16_t*)dst, ld_dst, (int)dst_rows);
+    return check_launch(fn);
+}
+
+}  // namespace mrl
+
+// ------------------------------------------------------------------------------------------ C ABI
+static int64_t round_up(int64_t x, int64_t to) { return (x + to - 1) / to * to; }
+
+extern "C" int mrl_lmhead_logits(const void* hidden, const void* weight, int64_t n_tokens, int64_t vocab,
+                                 int64_t hidden_dim, void* logits, int64_t logits_row_stride, void* stream) {
+    const char* fn = "mrl_lmhead_logits";
+    MRL_REQUIRE(n_tokens >= 0 && vocab > 0 && hidden_dim > 0, MRL_ERR_INVALID_ARG,
+                "%s: n_tokens=%lld vocab=%lld hidden_dim=%lld", fn, (long long)n_tokens, (long long)vocab,
+                (long long)hidden_dim);
+    MRL_REQUIRE(hidden_dim % BK == 0 && vocab % 8 == 0 && logits_row_stride % 8 == 0, MRL_ERR_UNSUPPORTED,
+                "%s: hidden_dim=%lld must be a multiple of %d, vocab=%lld and the row stride of 8", fn, (long long)hidden_dim, BK,
+                (long long)vocab);
+    MRL_REQUIRE(logits_row_stride >= vocab, MRL_ERR_INVALID_ARG, "%s: logits_row_stride below vocab", fn);
+    if (n_tokens == 0) return MRL_OK;
+    MRL_REQUIRE(hidden && weight && logits, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+    return mrl::gemm_nt_bf16(fn, weight, hidden_dim, vocab, hidden, hidden_dim, n_tokens, hidden_dim, logits,
+                             logits_row_stride, false, mrl::as_stream(stream));
+}
+
+extern "C" int64_t mrl_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t vocab, int64_t hidden_dim) {
+    if (n_tokens <= 0 || vocab <= 0 || hidden_dim <= 0) return 0;
+    const int64_t t_pad = round_up(n_tokens, BK);
+    // dlogits^T [vocab, t_pad] and hidden^T [hidden_dim, t_pad]
+    return (round_up(vocab, 8) + hidden_dim) * t_pad * 2;
+}
+
+extern "C" int mrl_lmhead_transpose_weight(const void* weight, int64_t vocab, int64_t hidden_dim, void* weight_t,
+                                           int64_t weight_t_row_stride, void* stream) {
+    const char* fn = "mrl_lmhead_transpose_weight";
+    MRL_REQUIRE(vocab > 0 && hidden_dim > 0 && weight_t_row_stride >= vocab && weight_t_row_stride % BK == 0,
+                MRL_ERR_INVALID_ARG, "%s: vocab=%lld hidden_dim=%lld row stride=%lld (a multiple of %d, at least vocab)", fn,
+                (long long)vocab, (long long)hidden_dim, (long long)weight_t_row_stride, BK);
+    MRL_REQUIRE(weight && weight_t, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+    return mrl::transpose_bf16(fn, weight, hidden_dim, vocab, hidden_dim, weight_t, weight_t_row_stride, hidden_dim,
+                               mrl::as_stream(stream));
+}
+
+extern "C" int mrl_lmhead_logprob_bwd(const void* hidden, const void* weight_t, int64_t weight_t_row_stride,
+                                      const void* dlogits, int64_t dlogits_row_stride, int64_t n_tokens, int64_t vocab,
+                                      int64_t hidden_dim, void* d_hidden, float* d_weight, void* workspace,
+                                      int64_t workspace_bytes, void* stream) {
+    const char* fn = "mrl_lmhead_logprob_bwd";
+    MRL_REQUIRE(n_tokens >= 0 && vocab > 0 && hidden_dim > 0, MRL_ERR_INVALID_ARG,
+                "%s: n_tokens=%lld vocab=%lld hidden_dim=%lld", fn, (long long)n_tokens, (long long)vocab,
+                (long long)hidden_dim);
+    MRL_REQUIRE(hidden_dim % BK == 0, MRL_ERR_UNSUPPORTED, "%s: hidden_dim=%lld must be a multiple of %d", fn,
+                (long long)hidden_dim, BK);
+    MRL_REQUIRE(weight_t_row_stride % BK == 0 && weight_t_row_stride >= vocab && dlogits_row_stride >= weight_t_row_stride,
+                MRL_ERR_INVALID_ARG,
+                "%s: weight_t_row_stride=%lld must be a multiple of %d and at least vocab, dlogits_row_stride=%lld at "
+                "least that (the padding columns of both must hold zeros)", fn, (long long)weight_t_row_stride, BK,
+                (long long)dlogits_row_stride);
+    if (n_tokens == 0) return MRL_OK;
+    MRL_REQUIRE(hidden && weight_t && dlogits && d_hidden && d_weight && workspace, MRL_ERR_INVALID_ARG, "%s: NULL pointer",
+                fn);
+    MRL_REQUIRE(workspace_bytes >= mrl_lmhead_bwd_workspace_bytes(n_tokens, vocab, hidden_dim), MRL_ERR_INVALID_ARG,
+                "%s: workspace of %lld bytes, need %lld", fn, (long long)workspace_bytes,
+                (long long)mrl_lmhead_bwd_workspace_bytes(n_tokens, vocab, hidden_dim));
+    MRL_REQUIRE(mrl::aligned(workspace, 16), MRL_ERR_MISALIGNED, "%s: workspace must be 16-byte aligned", fn);
+    hipStream_t s = mrl::as_stream(stream);
+    const int64_t k_vocab = weight_t_row_stride;             // the padded vocabulary: zeros beyond `vocab`
+    // dHidden[t][h] = sum_v Wt[h][v] * dlogits[t][v]
+    int rc = mrl::gemm_nt_bf16(fn, weight_t, weight_t_row_stride, hidden_dim, dlogits, dlogits_row_stride, n_tokens,
+                               k_vocab, d_hidden, hidden_dim, false, s);
+    if (rc != MRL_OK) return rc;
+    // dW[v][h] += sum_t hidden^T[h][t] * dlogits^T[v][t], over transposed copies with zero tails
+    const int64_t t_pad = round_up(n_tokens, BK);
+    const int64_t v4 = round_up(vocab, 8);
+    uint16_t* dz_t = reinterpret_cast<uint16_t*>(workspace);
+    uint16_t* h_t = dz_t + v4 * t_pad;
+    rc = mrl::transpose_bf16(fn, dlogits, dlogits_row_stride, n_tokens, vocab, dz_t, t_pad, v4, s);
+    if (rc != MRL_OK) return rc;
+    rc = mrl::transpose_bf16(fn, hidden, hidden_dim, n_tokens, hidden_dim, h_t, t_pad, hidden_dim, s);
+    if (rc != MRL_OK) return rc;
+    return mrl::gemm_nt_bf16(fn, h_t, t_pad, hidden_dim, dz_t, t_pad, vocab, t_pad, d_weight, hidden_dim, true, s);
+}

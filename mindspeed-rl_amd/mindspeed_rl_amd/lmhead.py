@@ -14,6 +14,19 @@ from . import _lib, vocab_ops
 kernel_events = None
 
 
+def _timed(name, rows, dev, *args):
+    """_lib.call with HIP events around it when kernel_events is a list."""
+    if kernel_events is None:
+        _lib.call(name, *args)
+        return
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    stream = torch.cuda.current_stream(dev)
+    start.record(stream)
+    _lib.call(name, *args)
+    end.record(stream)
+    kernel_events.append((name, start, end, rows))
+
+
 def lmhead_logprob(hidden, weight, labels, inv_temperature=1.0, want_entropy=True, row_active=None):
     """``hidden`` ``[..., H]`` bf16, ``weight`` ``[V, H]`` bf16 (``nn.Linear`` layout), ``labels``
     ``[...]`` int32/int64 -> ``(logp, entropy, lse)`` fp32 shaped like ``labels`` (entropy is zeros
@@ -74,26 +87,25 @@ def lmhead_logprob(hidden, weight, labels, inv_temperature=1.0, want_entropy=Tru
     return logp.view(lead), ent_out, lse.view(lead)
 
 
-def _accumulate_fp32(acc, a, b):
-    """acc (fp32) += a @ b for 16-bit operands, with the library GEMM writing fp32 in place."""
-    try:
-        torch.addmm(acc, a, b, out_dtype=torch.float32, out=acc)
-    except (TypeError, RuntimeError):        # a torch build without the fp32-output GEMM
-        acc.add_(torch.mm(a, b))
+def _round_up(x, to):
+    return (x + to - 1) // to * to
 
 
 class _FusedLmHeadLoss(torch.autograd.Function):
     """(hidden, weight) -> (loss, out[8]) with dHidden and dWeight produced during the forward.
 
-    The rows are processed in chunks: ``logits_c = hidden_c @ weight^T`` (a plain library GEMM),
+    The rows are processed in chunks: ``logits_c = hidden_c @ weight^T`` (``mrl_lmhead_logits``),
     the fused sweep turns the chunk into dlogits in place (one read, one write), then
-    ``dHidden_c = dlogits_c @ weight`` and ``dWeight += dlogits_c^T @ hidden_c`` (library GEMMs,
-    fp32 accumulation across chunks).  Only ``chunk_rows x V`` logits exist at any time."""
+    ``dHidden_c = dlogits_c @ weight`` and ``dWeight += dlogits_c^T @ hidden_c``
+    (``mrl_lmhead_logprob_bwd``, fp32 accumulation across chunks in stream order).  All three
+    products run on the hand-written bf16 MFMA kernels; only ``chunk_rows x V`` logits exist at any
+    time."""
 
     @staticmethod
     def forward(ctx, hidden, weight, labels, batch, cfg):
         from .loss import _expected_scale, _mask_args, _sweep_workspace
         dev = _lib.require_device(hidden, weight, labels)
+        lib = _lib.load()
         hdim = hidden.shape[-1]
         h2d = hidden.detach().reshape(-1, hdim).contiguous()
         w = weight.detach().contiguous()
@@ -141,7 +153,7 @@ class _FusedLmHeadLoss(torch.autograd.Function):
         grad_scale, scale_dev, applied = _expected_scale(cfg, dev)
         # Rows whose mask is zero (prompts, padding, masked tokens) add nothing to the loss, to dWeight or
         # to their own dHidden: when they are more than a twentieth of the rows, the live rows are gathered
-        # and only they go through the GEMMs.  The row count sizes the GEMMs, so it is read back (one
+        # and only they go through the products.  The row count sizes the products, so it is read back (one
         # host synchronisation per call; compact_rows=False avoids it).
         live = None
         if cfg["compact_rows"] and n_rows > 0:
@@ -157,35 +169,35 @@ class _FusedLmHeadLoss(torch.autograd.Function):
             terms_all, row_terms = row_terms, torch.empty(max(n_rows, 1) * 8, dtype=torch.float32, device=dev)
             ent = torch.empty(max(n_rows, 1), dtype=torch.float32, device=dev) if want_ent else None
         chunk = max(1, min(int(cfg["chunk_rows"]), n_rows))
-        logits = torch.empty((chunk, vocab), dtype=h2d.dtype, device=dev)
-        workspace, ws_bytes = _sweep_workspace(logits)
+        # the chunk of logits: rows padded to whole k-steps of the backward products; the padding
+        # columns are zeroed once and never written (they meet the zero padding of the transposed weight)
+        v_pad = _round_up(vocab, 64)
+        if v_pad != vocab:
+            logits = torch.zeros((chunk, v_pad), dtype=h2d.dtype, device=dev)
+        else:
+            logits = torch.empty((chunk, v_pad), dtype=h2d.dtype, device=dev)
         d_hidden = torch.empty_like(h2d)
         d_weight32 = torch.zeros((vocab, hdim), dtype=torch.float32, device=dev)
-        w_t = w.t()
-        # The library's GEMM for dlogits_c @ W is a third faster when W is laid out [H, V] (6.7 against
-        # 9.4 ms per 8192-row chunk at V = 152064, H = 3584), so one transposed copy is made per step.
-        w_hv = w_t.contiguous() if n_rows > 8192 else None
+        w_t = torch.empty((hdim, v_pad), dtype=w.dtype, device=dev)
+        _lib.call("mrl_lmhead_transpose_weight", _lib.ptr(w), vocab, hdim, _lib.ptr(w_t), v_pad, stream)
+        bwd_bytes = lib.mrl_lmhead_bwd_workspace_bytes(chunk, vocab, hdim)
+        bwd_ws = torch.empty(max(bwd_bytes, 16), dtype=torch.uint8, device=dev)
+        sweep_bytes = lib.mrl_fused_workspace_bytes(_lib.dtype_code(logits), chunk, vocab)
+        sweep_ws = torch.empty(max(sweep_bytes, 16), dtype=torch.uint8, device=dev)
+        esz = h2d.element_size()
         for c0 in range(0, n_rows, chunk):
-            c1 = min(n_rows, c0 + chunk)
-            rows = c1 - c0
-            z = logits[:rows]
-            torch.mm(h2d[c0:c1], w_t, out=z)                      # plain GEMM (hipBLASLt)
+            rows = min(n_rows, c0 + chunk) - c0
+            h_c = h2d.data_ptr() + c0 * hdim * esz
+            _timed("mrl_lmhead_logits", rows, dev, h_c, _lib.ptr(w), rows, vocab, hdim, _lib.ptr(logits), v_pad, stream)
             vocab_ops._timed_call(
-                "mrl_fused_logprob_loss", rows, dev, _lib.ptr(z), _lib.dtype_code(z), rows, vocab, vocab,
+                "mrl_fused_logprob_loss", rows, dev, _lib.ptr(logits), _lib.dtype_code(logits), rows, vocab, v_pad,
                 lab.data_ptr() + c0 * lab.element_size(), _lib.dtype_code(lab), cfg["inv_temperature"],
                 row_ops.data_ptr() + c0 * 32, 0 if old is None else 1, cfg["clip_lo"], cfg["clip_hi"], cfg["kl_penalty"],
-                cfg["kl_coef"], cfg["entropy_coeff"], grad_scale, _lib.ptr(scale_dev), _lib.ptr(z), vocab, None,
-                (ent.data_ptr() + c0 * 4) if want_ent else None, row_terms.data_ptr() + c0 * 32, _lib.ptr(workspace),
-                ws_bytes, stream)
-            torch.mm(z, w if w_hv is None else w_hv.t(), out=d_hidden[c0:c1])    # dHidden_c = dlogits_c @ W
-            # dW += dlogits_c^T @ hidden_c, accumulated in fp32 by the GEMM itself (no separate add pass,
-            # no rounding of the chunk's product to bf16)
-            if cfg["fp32_dw_gemm"]:
-                d_weight32.addmm_(z.t().float(), h2d[c0:c1].float())
-            else:
-                # the hidden chunk goes in as the transpose of an [H, rows] copy: the library picks a faster
-                # kernel for that operand layout (7.5 against 8.7 ms per chunk), the copy is 59 MB
-                _accumulate_fp32(d_weight32, z.t(), h2d[c0:c1].t().contiguous().t())
+                cfg["kl_coef"], cfg["entropy_coeff"], grad_scale, _lib.ptr(scale_dev), _lib.ptr(logits), v_pad, None,
+                (ent.data_ptr() + c0 * 4) if want_ent else None, row_terms.data_ptr() + c0 * 32, _lib.ptr(sweep_ws),
+                sweep_bytes, stream)
+            _timed("mrl_lmhead_logprob_bwd", rows, dev, h_c, _lib.ptr(w_t), v_pad, _lib.ptr(logits), v_pad, rows, vocab,
+                   hdim, d_hidden.data_ptr() + c0 * hdim * esz, _lib.ptr(d_weight32), _lib.ptr(bwd_ws), bwd_bytes, stream)
         if live is not None:
             compact_dh, compact_terms = d_hidden, row_terms
             d_hidden = torch.zeros_like(h_all)
@@ -215,7 +227,7 @@ class _FusedLmHeadLoss(torch.autograd.Function):
 def fused_lmhead_policy_loss(hidden, weight, batch, *, packed, seqlens=None, cu_seqlens=None, mask=None,
                              ref_log_prob=None, clip_low, clip_high, kl_penalty=None, kl_coef=0.0, entropy_coeff=0.0,
                              token_level_loss=True, loss_scale=1.0, inv_temperature=1.0, expected_upstream=None,
-                             scale_state=None, chunk_rows=32768, fp32_dw_gemm=False, compact_rows=True):
+                             scale_state=None, chunk_rows=32768, compact_rows=True):
     """Policy loss straight from the hidden states: ``hidden`` is packed ``[1, T, H]`` (or padded
     ``[B, S, H]``) bf16, ``weight`` the ``[V, H]`` bf16 lm_head weight; ``batch`` as for
     :func:`mindspeed_rl_amd.fused_logprob_policy_loss` (``labels, responses, response_length,
@@ -231,13 +243,14 @@ def fused_lmhead_policy_loss(hidden, weight, batch, *, packed, seqlens=None, cu_
         kl_code = _lib.KL_BY_NAME[kl_penalty]
     else:
         raise NotImplementedError
-    if hidden.dtype not in (torch.bfloat16, torch.float16) or weight.dtype != hidden.dtype:
-        raise TypeError("hidden and weight must both be bfloat16 (or float16)")
+    if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise TypeError("hidden and weight must both be bfloat16")
+    if hidden.shape[-1] % 64 != 0 or weight.shape[0] % 8 != 0:
+        raise ValueError("hidden_dim must be a multiple of 64 and the vocabulary of 8")
     cfg = dict(packed=bool(packed), seqlens=seqlens, cu=cu_seqlens, mask=mask, ref_log_prob=ref_log_prob,
                clip_lo=float(1.0 - clip_low), clip_hi=float(1.0 + clip_high), kl_penalty=kl_code,
                kl_coef=float(kl_coef), entropy_coeff=float(entropy_coeff), seq_mean=0 if token_level_loss else 1,
                loss_scale=float(loss_scale), inv_temperature=float(inv_temperature),
                expected_upstream=None if expected_upstream is None else float(expected_upstream),
-               scale_state=scale_state, chunk_rows=int(chunk_rows), fp32_dw_gemm=bool(fp32_dw_gemm),
-               compact_rows=bool(compact_rows))
+               scale_state=scale_state, chunk_rows=int(chunk_rows), compact_rows=bool(compact_rows))
     return _FusedLmHeadLoss.apply(hidden, weight, batch["labels"], batch, cfg)

@@ -1412,6 +1412,52 @@ def test_fused_lmhead_policy_loss(dev, chunk_rows):
     assert (dw.float().cpu() * 2 - dw_want).abs().max().item() <= 2e-2 * dw_want.abs().max().item()
 
 
+@pytest.mark.parametrize("tokens,vocab,hdim", [(517, 4352, 3584), (300, 1000, 128), (64, 4096 + 24, 256), (1, 8, 64),
+                                               (777, 2048, 192), (4100, 520, 64)])
+def test_lmhead_products_through_the_c_abi(dev, tokens, vocab, hdim):
+    """The three matrix products of the lm_head training step, hand-written for the matrix cores:
+    logits = hidden W^T (mrl_lmhead_logits), dHidden = dlogits W and dWeight += dlogits^T hidden
+    (mrl_lmhead_logprob_bwd), against fp32 products of the same bf16 operands on the CPU: ragged token
+    and vocabulary tiles, a vocabulary that is no multiple of the 64-wide k-step (zero padding), two
+    accumulating calls into one dWeight, untouched padding."""
+    gen = torch.Generator().manual_seed(tokens * 7 + vocab)
+    h = torch.randn(tokens, hdim, generator=gen).to(torch.bfloat16)
+    w = (torch.randn(vocab, hdim, generator=gen) * (2.0 / hdim ** 0.5)).to(torch.bfloat16)
+    dz = (torch.randn(tokens, vocab, generator=gen) * 0.01).to(torch.bfloat16)
+    hd, wd = h.to(dev), w.to(dev)
+    lib = _lib.load()
+    stream = _lib.stream(dev)
+    v_pad = (vocab + 63) // 64 * 64
+    z = torch.full((tokens, v_pad), 7.0, dtype=torch.bfloat16, device=dev)
+    _lib.call("mrl_lmhead_logits", hd.data_ptr(), wd.data_ptr(), tokens, vocab, hdim, z.data_ptr(), v_pad, stream)
+    want_z = h.float() @ w.float().t()
+    err = (z[:, :vocab].float().cpu() - want_z).abs().max().item()
+    assert err <= 2 ** -8 * want_z.abs().max().item() + 1e-6                   # one bf16 rounding of the result
+    assert (z[:, vocab:] == 7.0).all().item()                                   # the padding is not written
+    # backward: the padding of dlogits and of the transposed weight must be zero
+    dzd = torch.zeros((tokens, v_pad), dtype=torch.bfloat16, device=dev)
+    dzd[:, :vocab] = dz.to(dev)
+    w_t = torch.full((hdim, v_pad), 3.0, dtype=torch.bfloat16, device=dev)
+    _lib.call("mrl_lmhead_transpose_weight", wd.data_ptr(), vocab, hdim, w_t.data_ptr(), v_pad, stream)
+    assert torch.equal(w_t[:, :vocab].cpu(), w.t()) and not w_t[:, vocab:].any().item()
+    ws_bytes = lib.mrl_lmhead_bwd_workspace_bytes(tokens, vocab, hdim)
+    ws = torch.full((ws_bytes,), 0xFF, dtype=torch.uint8, device=dev)
+    dh = torch.full((tokens, hdim), 5.0, dtype=torch.bfloat16, device=dev)
+    dw = torch.ones(vocab, hdim, dtype=torch.float32, device=dev)
+    for _ in range(2):                                                           # dWeight accumulates
+        _lib.call("mrl_lmhead_logprob_bwd", hd.data_ptr(), w_t.data_ptr(), v_pad, dzd.data_ptr(), v_pad, tokens, vocab,
+                  hdim, dh.data_ptr(), dw.data_ptr(), ws.data_ptr(), ws_bytes, stream)
+    want_dh = dz.float() @ w.float()
+    want_dw = 1.0 + 2.0 * (dz.float().t() @ h.float())
+    assert (dh.float().cpu() - want_dh).abs().max().item() <= 2 ** -7 * want_dh.abs().max().item() + 1e-9
+    assert (dw.cpu() - want_dw).abs().max().item() <= 2 ** -7 * (want_dw - 1.0).abs().max().item() + 1e-6
+    # rejected shapes: nothing is launched
+    assert lib.mrl_lmhead_logits(hd.data_ptr(), wd.data_ptr(), tokens, vocab, hdim - 8, z.data_ptr(), v_pad, stream) == -2
+    assert lib.mrl_lmhead_logprob_bwd(hd.data_ptr(), w_t.data_ptr(), v_pad, dzd.data_ptr(), v_pad, tokens, vocab, hdim,
+                                      dh.data_ptr(), dw.data_ptr(), ws.data_ptr(), 16, stream) == -1
+    assert b"workspace" in lib.mrl_last_error()
+
+
 def test_copy_kernel_moves_bytes(dev):
     src = torch.randint(0, 255, (1 << 20,), dtype=torch.uint8, device=dev)
     dst = torch.zeros_like(src)

@@ -128,6 +128,16 @@ def test_argument_validation_launches_nothing():
     assert lib.mrl_lmhead_logprob_fwd(p, p, 4, 1000, 100, p, _lib.I64, 1.0, p, None, None, p, 1 << 20, None) != 0
     assert lib.mrl_lmhead_logprob_fwd(p, p, 4, 1000, 128, p, _lib.I64, 1.0, p, None, None, p, 16, None) != 0
     assert b"workspace" in lib.mrl_last_error()
+    # products of the lm_head training step
+    assert lib.mrl_lmhead_logits(p, p, 4, 1000, 100, p, 1000, None) == -2                   # hidden_dim % 64
+    assert lib.mrl_lmhead_logits(p, p, 4, 1001, 128, p, 1008, None) == -2                   # vocab % 8
+    assert lib.mrl_lmhead_logits(p, p, 4, 1000, 128, p, 992, None) == -1                    # row stride below vocab
+    assert lib.mrl_lmhead_logits(None, None, 0, 1000, 128, None, 1000, None) == 0
+    assert lib.mrl_lmhead_bwd_workspace_bytes(100, 1000, 128) == (1000 + 128) * 128 * 2
+    assert lib.mrl_lmhead_transpose_weight(p, 1000, 128, p, 1000, None) == -1               # stride not a multiple of 64
+    assert lib.mrl_lmhead_logprob_bwd(p, p, 1024, p, 1000, 4, 1000, 128, p, p, p, 1 << 30, None) == -1
+    assert b"dlogits_row_stride" in lib.mrl_last_error()
+    assert lib.mrl_lmhead_logprob_bwd(p, p, 1024, p, 1024, 4, 1000, 128, p, p, None, 0, None) == -1
     # PPO value side
     assert lib.mrl_gae_scan(p, p + 512, 2, 8, 1.0, 0.95, p, p + 1024, None) == -1 and b"alias" in lib.mrl_last_error()
     assert lib.mrl_gae_scan(p, p + 512, 2, 0, 1.0, 0.95, p + 1024, p + 2048, None) == -1
