@@ -302,23 +302,44 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(const uint16_t* __
 
 // dst[c][r] = src[r][c] for r < rows, c < cols; dst has `dst_rows` >= cols rows of `ld_dst` >= rows
 // entries, and everything outside the transposed block (the padding that lets a product walk k in
-// whole steps) is written as zero.  64 x 64 tiles through LDS, 16-bit elements.
+// whole steps) is written as zero.  64 x 64 tiles of 16-bit elements through LDS: 16-byte loads along
+// the source rows, 16-byte stores along the destination rows (8 two-byte LDS reads down a column
+// each; the row pitch of 33 words keeps them on different banks).  ld_src, ld_dst % 8 == 0.
 __global__ __launch_bounds__(256) void transpose_bf16_kernel(const uint16_t* __restrict__ src, int64_t ld_src, int rows,
                                                              int cols, uint16_t* __restrict__ dst, int64_t ld_dst,
                                                              int dst_rows) {
     __shared__ uint16_t tile[64][66];
     const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
-    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const int r = r0 + ty * 16 + i, c = c0 + tx;
-        tile[ty * 16 + i][tx] = (r < rows && c < cols) ? src[(int64_t)r * ld_src + c] : (uint16_t)0;
+    for (int i = 0; i < 2; ++i) {
+        const int v = threadIdx.x + i * 256;
+        const int r = v >> 3, cv = (v & 7) * 8;
+        uint32_t w[4] = {0u, 0u, 0u, 0u};
+        if (r0 + r < rows) {
+            const uint16_t* p = src + (int64_t)(r0 + r) * ld_src + c0 + cv;
+            if (c0 + cv + 8 <= cols) {
+                const u32x4 x = *reinterpret_cast<const u32x4*>(p);
+                w[0] = x.x; w[1] = x.y; w[2] = x.z; w[3] = x.w;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (c0 + cv + e < cols) w[e >> 1] |= (uint32_t)p[e] << ((e & 1) * 16);
+            }
+        }
+        uint32_t* t = reinterpret_cast<uint32_t*>(&tile[r][cv]);
+        t[0] = w[0]; t[1] = w[1]; t[2] = w[2]; t[3] = w[3];
     }
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const int c = c0 + ty * 16 + i, r = r0 + tx;
-        if (c < dst_rows && r < ld_dst) dst[(int64_t)c * ld_dst + r] = tile[tx][ty * 16 + i];
+    for (int i = 0; i < 2; ++i) {
+        const int v = threadIdx.x + i * 256;
+        const int c = v >> 3, rv = (v & 7) * 8;
+        if (c0 + c >= dst_rows || r0 + rv >= ld_dst) continue;
+        uint32_t w[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            w[e] = (uint32_t)tile[rv + 2 * e][c] | ((uint32_t)tile[rv + 2 * e + 1][c] << 16);
+        *reinterpret_cast<u32x4*>(dst + (int64_t)(c0 + c) * ld_dst + r0 + rv) = mrl::make_u32x4(w[0], w[1], w[2], w[3]);
     }
 }
 
@@ -366,9 +387,10 @@ int gemm_nt_bf16(const char* fn, const void* a, int64_t lda, int64_t m, const vo
 
 int transpose_bf16(const char* fn, const void* src, int64_t ld_src, int64_t rows, int64_t cols, void* dst, int64_t ld_dst,
                    int64_t dst_rows, hipStream_t stream) {
-    MRL_REQUIRE(rows >= 0 && cols >= 0 && ld_src >= cols && ld_dst >= rows && dst_rows >= cols, MRL_ERR_INVALID_ARG,
-                "%s: transpose of %lld x %lld (ld %lld) into %lld x %lld", fn, (long long)rows, (long long)cols,
-                (long long)ld_src, (long long)dst_rows, (long long)ld_dst);
+    MRL_REQUIRE(rows >= 0 && cols >= 0 && ld_src >= cols && ld_dst >= rows && dst_rows >= cols && ld_src % 8 == 0 &&
+                    ld_dst % 8 == 0 && aligned(src, 16) && aligned(dst, 16),
+                MRL_ERR_INVALID_ARG, "%s: transpose of %lld x %lld (ld %lld) into %lld x %lld (16-byte aligned rows)", fn,
+                (long long)rows, (long long)cols, (long long)ld_src, (long long)dst_rows, (long long)ld_dst);
     if (dst_rows == 0 || ld_dst == 0) return MRL_OK;
     const int64_t gx = (ld_dst + 63) / 64, gy = (dst_rows + 63) / 64;
     MRL_REQUIRE(gx <= 0x7fffffffLL && gy <= 65535, MRL_ERR_UNSUPPORTED, "%s: grid too large", fn);
