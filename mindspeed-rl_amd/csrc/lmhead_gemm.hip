@@ -37,14 +37,9 @@ using namespace mrl_vocab;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-// Wavefront layout of the 256 x 256 tile: 2 wavefronts along m (128 rows of A each) by kWavesN along
-// n.  With 4 along n (512 threads, two wavefronts per SIMD) a wavefront owns 128 x 64 = 4 x 2 MFMA
-// blocks; with 2 along n (256 threads, one wavefront per SIMD) 128 x 128 = 4 x 4 blocks in 256
-// accumulator registers, which needs a third fewer fragment bytes from LDS per flop.
-#ifndef MRL_GEMM_WAVES_N
-#define MRL_GEMM_WAVES_N 4
-#endif
-constexpr int kWavesN = MRL_GEMM_WAVES_N;
+// Wavefront layout of the 256 x 256 tile: 2 wavefronts along m (128 rows of A each) by 4 along n
+// (512 threads, two wavefronts per SIMD); a wavefront owns 128 x 64 = 4 x 2 MFMA blocks.
+constexpr int kWavesN = 4;
 constexpr int kWaves = 2 * kWavesN;
 constexpr int kThreads = 64 * kWaves;
 constexpr int kTB = 8 / kWavesN;                 // 32-row blocks of B per wavefront
@@ -103,7 +98,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(const uint16_t* __
                                                               void* __restrict__ out, int64_t ldo) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wv = wave / kWavesN, wt = wave % kWavesN;
 
     TileGrid grid;
@@ -256,48 +251,61 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(const uint16_t* __
         }
     };
 
-    Frags f0, f1;
+    // Two-group schedule.  Wavefronts w and w + 4 share a SIMD; the four of group 0 (wave < 4) and the
+    // four of group 1 alternate between a memory phase (stage requests, fragment reads) and a compute
+    // phase (16 MFMAs), half a period apart: while one wavefront of a SIMD feeds the matrix pipe the
+    // other one issues its loads, and neither holds up the other's instruction stream.  Workgroup
+    // barriers between the phases keep the groups in step; group 1 passes one barrier before its first
+    // phase and group 0 one after its last, so that every wavefront passes the same number.
+    // Barrier p (counted from 1) is the one group 0 passes p-th in the loop.  Stage s is read by group 0
+    // between barriers 4s and 4s+3, by group 1 between 4s+1 and 4s+4; it is requested by both at the
+    // start of their first memory phase of stage s-1 (after 4s-4: stage s-2, whose buffer it takes,
+    // has been read by everybody) and every wavefront waits for its own requests before it arrives at
+    // barrier 4s.
+    const int group = wave >> 2;
+    auto barrier = [&]() {
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    Frags fa, fb;
     set_load_tile(load_tile);
     issue_next(0);
-    __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0): stage 0 has landed
-    __syncthreads();
     if (n_stages > 1) issue_next(1);
-    read_frags(f0, smem, 0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0): stages 0 and 1 have landed
+    __syncthreads();
+    if (group == 1) barrier();
     int stage_idx = 0;
     for (int mine = 0; mine < my_tiles; ++mine) {
         zero_acc();
         for (int kstep = 0; kstep < n_ksteps; ++kstep, ++stage_idx) {
             const int buf = stage_idx & 1;
             const unsigned char* stage = smem + buf * kStageBytes;
-            // software pipeline: the fragments of sub-step ks+1 are requested before the MFMAs of ks
-            read_frags(f1, stage, 1);
-            __builtin_amdgcn_sched_barrier(0);
-            mma(f0);
-            __builtin_amdgcn_sched_barrier(0);
-            read_frags(f0, stage, 2);
-            __builtin_amdgcn_sched_barrier(0);
-            mma(f1);
-            __builtin_amdgcn_sched_barrier(0);
-            read_frags(f1, stage, 3);
-            __builtin_amdgcn_sched_barrier(0);
-            mma(f0);
-            __builtin_amdgcn_sched_barrier(0);
-            // The last fragments of this stage are in registers and the next stage has landed: after the
-            // barrier this buffer may be overwritten, and the first fragments of the next stage are
-            // requested before the last MFMAs of this one are issued.  The barrier and the read are
-            // unconditional (after the last stage the read fetches unused bytes of the other buffer).
-            __builtin_amdgcn_s_waitcnt(0x0070);        // vmcnt(0) lgkmcnt(0)
-            __syncthreads();
-            read_frags(f0, smem + (buf ^ 1) * kStageBytes, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            mma(f1);
-            __builtin_amdgcn_sched_barrier(0);
-            // the stage after next goes into the buffer that the barrier has just freed
-            if (stage_idx + 2 < n_stages) issue_next(buf);
-            __builtin_amdgcn_sched_barrier(0);
+            if (stage_idx >= 1 && stage_idx + 1 < n_stages) issue_next(buf ^ 1);
+            read_frags(fa, stage, 0);
+            read_frags(fb, stage, 1);
+            __builtin_amdgcn_s_waitcnt(0xC07F);        // lgkmcnt(0)
+            barrier();
+            __builtin_amdgcn_s_setprio(1);
+            mma(fa);
+            mma(fb);
+            __builtin_amdgcn_s_setprio(0);
+            barrier();
+            read_frags(fa, stage, 2);
+            read_frags(fb, stage, 3);
+            if (group == 1) __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0)
+            else __builtin_amdgcn_s_waitcnt(0xC07F);
+            barrier();
+            __builtin_amdgcn_s_setprio(1);
+            mma(fa);
+            mma(fb);
+            __builtin_amdgcn_s_setprio(0);
+            if (group == 0) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+            barrier();
         }
         store_tile(first_tile + (int64_t)mine * tile_stride);
     }
+    if (group == 0) barrier();
 }
 
 // dst[c][r] = src[r][c] for r < rows, c < cols; dst has `dst_rows` >= cols rows of `ld_dst` >= rows
