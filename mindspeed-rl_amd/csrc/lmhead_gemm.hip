@@ -1,14 +1,14 @@
-// bf16 matrix products of the lm_head training step for gfx950, on the tile loop of the fused
-// lm_head forward (lmhead.hip): operands go from global memory straight into LDS
-// (buffer_load ... lds), two 64 KiB stages, XOR-swizzled 16-byte chunks, v_mfma_f32_32x32x16_bf16,
-// fragments of the next sub-step requested before the MFMAs of the current one.
+// bf16 matrix products of the lm_head training step for gfx950: operands go from global memory
+// straight into LDS (buffer_load ... lds), two 64 KiB stages, XOR-swizzled 16-byte chunks,
+// v_mfma_f32_16x16x32_bf16 (at the board's power limit this shape runs about 18 % faster than the
+// same flops as 32x32x16), memory instructions placed between the MFMAs of one instruction stream.
 //
 // One kernel covers the three products of the step, because each of them can be put in the form
 //
 //     out[n][m] (+)= sum_k A[m][k] * B[n][k]          A: [M, K], B: [N, K], both with k contiguous
 //
-// (the MFMA's M is the fast dimension of the output: in the 32x32 result layout a lane owns ONE
-// column n and 4 consecutive rows m at a time, i.e. 8 contiguous bytes of bf16 or 16 of fp32):
+// (the MFMA's M is the fast dimension of the output: in the 16x16 result layout a lane owns ONE
+// column n and 4 consecutive rows m, i.e. 8 contiguous bytes of bf16 or 16 of fp32):
 //
 //     logits[t][v]  = sum_h W[v][h]      * hidden[t][h]      A = W,         B = hidden chunk
 //     dHidden[t][h] = sum_v Wt[h][v]     * dlogits[t][v]     A = W^T copy,  B = dlogits chunk
@@ -17,13 +17,13 @@
 // The transposed copies are made by transpose_bf16_kernel; their padded tails are zero so that the
 // k dimension can always be walked in whole steps of 64.
 //
-// Work distribution: one persistent 512-thread workgroup per CU (2 x 4 wavefronts, wavefront tile
-// 128 x 64) walks output tiles of 256 x 256.  Tiles are numbered so that 32 consecutive numbers are
-// 8 tiles along m by 4 along n, and the 32 workgroups that share an XCD (and its L2) take 32
-// consecutive numbers at a time: the 4 that stream the same A tile and the 8 that stream the same
-// B tile run side by side (see tile_coords for the order of the groups of 32).  The loop runs over
-// the flattened (tile, k-step) sequence of a workgroup, so the first loads of its next tile are in
-// flight while the current one is stored.
+// Work distribution: one persistent 256-thread workgroup per CU (2 x 2 wavefronts, one per SIMD,
+// wavefront tile 128 x 128 in 256 accumulator registers) walks output tiles of 256 x 256.  Tiles are
+// numbered so that 32 consecutive numbers are 8 tiles along m by 4 along n, and the 32 workgroups
+// that share an XCD (and its L2) take 32 consecutive numbers at a time: the 4 that stream the same A
+// tile and the 8 that stream the same B tile run side by side (see tile_coords for the order of the
+// groups of 32).  The loop runs over the flattened (tile, k-step) sequence of a workgroup, so the
+// first loads of its next tile are in flight while the current one is stored.
 #include <stdlib.h>
 
 #include "lmhead_gemm.h"
@@ -35,14 +35,14 @@ namespace {
 using namespace mrl_vocab;
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-// Wavefront layout of the 256 x 256 tile: 2 wavefronts along m (128 rows of A each) by 4 along n
-// (512 threads, two wavefronts per SIMD); a wavefront owns 128 x 64 = 4 x 2 MFMA blocks.
-constexpr int kWavesN = 4;
+// Wavefront layout of the 256 x 256 tile: 2 wavefronts along m (128 rows of A each) by 2 along n
+// (128 rows of B each); a wavefront owns 8 x 8 MFMA blocks of 16 x 16.
+constexpr int kWavesN = 2;
 constexpr int kWaves = 2 * kWavesN;
 constexpr int kThreads = 64 * kWaves;
-constexpr int kTB = 8 / kWavesN;                 // 32-row blocks of B per wavefront
+constexpr int kBlocks = 8;                       // 16-row blocks of A, and of B, per wavefront
 constexpr int kLoadsPerWave = 32 / kWaves;       // 8-row groups of an operand that a wavefront brings in
 constexpr int BM = 256;                          // rows of A per tile
 constexpr int BN = 256;                          // rows of B per tile
@@ -55,7 +55,7 @@ constexpr int kLdsBytes = kLdsStages + kLdsTurn;
 constexpr int kTilesAlongN = 4;                  // tiles along n in a group of consecutive tile numbers
 
 // Element offset (row * ld + column, without the k-step) of the chunk that lane `lane` of wavefront
-// `wave` brings in with its load j (0..3) of an operand tile with `rows_valid` rows left (rows beyond
+// `wave` brings in with its load j (0..7) of an operand tile with `rows_valid` rows left (rows beyond
 // are clamped to the last valid one; their products are never stored).  Physical slot of a 16-byte
 // chunk inside its 256-byte pair of rows: logical slot ^ (pair & 15), logical = (row & 1) * 8 + chunk.
 __device__ __forceinline__ int64_t stage_src_offset(int wave, int lane, int j, int64_t ld, int rows_valid) {
@@ -113,7 +113,6 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(const uint16_t* __
     if (first_tile >= grid.total) return;
     const int my_tiles = (int)((grid.total - 1 - first_tile) / tile_stride) + 1;
     const int n_ksteps = K / BK;
-    const int n_stages = my_tiles * n_ksteps;
 
     // ---- loader state: the tile whose stages are being requested
     int64_t load_tile = first_tile;
@@ -133,18 +132,21 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(const uint16_t* __
         a_rsrc = mrl::make_rsrc(A + (int64_t)tm * BM * lda, 0xffffffffu);
         b_rsrc = mrl::make_rsrc(B + (int64_t)tn * BN * ldb, 0xffffffffu);
     };
-    auto issue_next = [&](int buf) {
+    // request i (0..15) of the stage being requested: the wavefront's 8 row groups of A, then of B
+    auto issue_one = [&](int buf, int i) {
         const uint32_t k_bytes = (uint32_t)(load_k * BK * 2);
         unsigned char* dst = smem + buf * kStageBytes + (wave * kLoadsPerWave) * 1024;
-#pragma unroll
-        for (int j = 0; j < kLoadsPerWave; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (void __attribute__((address_space(3)))*)(dst + j * 1024), 16,
-                                                 a_off[j], k_bytes, 0, 0);
-#pragma unroll
-        for (int j = 0; j < kLoadsPerWave; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc,
-                                                 (void __attribute__((address_space(3)))*)(dst + kOperandBytes + j * 1024),
-                                                 16, b_off[j], k_bytes, 0, 0);
+        if (i < kLoadsPerWave)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (void __attribute__((address_space(3)))*)(dst + i * 1024), 16,
+                                                 a_off[i], k_bytes, 0, 0);
+        else
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                b_rsrc, (void __attribute__((address_space(3)))*)(dst + kOperandBytes + (i - kLoadsPerWave) * 1024), 16,
+                b_off[i - kLoadsPerWave], k_bytes, 0, 0);
+    };
+    // After the last stage of the last tile the requests go on (the schedule below has no branches):
+    // they fetch valid bytes of the last tile into a buffer that nobody reads any more.
+    auto stage_issued = [&]() {
         if (++load_k == n_ksteps) {
             load_k = 0;
             load_tile += tile_stride;
@@ -152,82 +154,99 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(const uint16_t* __
         }
     };
 
-    // fragment addresses: row (lane & 31) of a 32-row block, chunk 2 ks + (lane >> 5)
-    const int frag_pair = (lane & 31) >> 1;
-    const int frag_slot = (((lane & 1) << 3) | (lane >> 5)) ^ frag_pair;          // ^ (2 ks) per k sub-step
-    const int a_frag = (wv * 64) * 256 + frag_pair * 256;                          // + vb * 16 * 256
-    const int b_frag = kOperandBytes + (wt * 16 * kTB) * 256 + frag_pair * 256;    // + tb * 16 * 256
+    // Fragment addresses.  A lane reads row (lane & 15) of a 16-row block (8 row pairs, 2 KiB), chunk
+    // 4 ks + (lane >> 4) of its 8: inside the block its pair is (lane >> 1) & 7, the pair's low bits
+    // are ((block & 1) << 3) | that, and the physical slot is the logical one XOR those bits.
+    int frag_off[2][2];                                   // [block parity][k sub-step of 32]
+#pragma unroll
+    for (int par = 0; par < 2; ++par)
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const int pair_in_block = (lane >> 1) & 7;
+            const int slot = ((((lane & 1) ^ par) << 3) | ((4 * ks + (lane >> 4)) ^ pair_in_block));
+            frag_off[par][ks] = pair_in_block * 256 + slot * 16;
+        }
+    const int a_frag = (wv * kBlocks) * 2048;                            // + vb * 2048
+    const int b_frag = kOperandBytes + (wt * kBlocks) * 2048;            // + tb * 2048
     struct Frags {
-        bf16x8 a[4], b[kTB];
+        bf16x8 a[kBlocks], b[kBlocks];
     };
-    auto read_frags = [&](Frags& f, const unsigned char* stage, int ks) {
-        const int slot_bytes = (frag_slot ^ (2 * ks)) * 16;
-#pragma unroll
-        for (int vb = 0; vb < 4; ++vb)
-            f.a[vb] = *reinterpret_cast<const bf16x8*>(stage + a_frag + vb * 16 * 256 + slot_bytes);
-#pragma unroll
-        for (int tb = 0; tb < kTB; ++tb)
-            f.b[tb] = *reinterpret_cast<const bf16x8*>(stage + b_frag + tb * 16 * 256 + slot_bytes);
+    // read r (0..15) of a fragment set, in the order the MFMAs need them: a0, all of b, a1..a7
+    auto read1 = [&](Frags& f, const unsigned char* stage, int ks, int r) {
+        if (r == 0) f.a[0] = *reinterpret_cast<const bf16x8*>(stage + a_frag + frag_off[0][ks]);
+        else if (r <= kBlocks)
+            f.b[r - 1] = *reinterpret_cast<const bf16x8*>(stage + b_frag + (r - 1) * 2048 + frag_off[(r - 1) & 1][ks]);
+        else
+            f.a[r - kBlocks] =
+                *reinterpret_cast<const bf16x8*>(stage + a_frag + (r - kBlocks) * 2048 + frag_off[(r - kBlocks) & 1][ks]);
     };
-    floatx16 acc[4][kTB];
+    floatx4 acc[kBlocks][kBlocks];
     auto zero_acc = [&]() {
 #pragma unroll
-        for (int vb = 0; vb < 4; ++vb)
+        for (int vb = 0; vb < kBlocks; ++vb)
 #pragma unroll
-            for (int tb = 0; tb < kTB; ++tb)
+            for (int tb = 0; tb < kBlocks; ++tb)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) acc[vb][tb][i] = 0.f;
+                for (int i = 0; i < 4; ++i) acc[vb][tb][i] = 0.f;
     };
-    auto mma = [&](const Frags& f) {
+    // Empty statements that demand every accumulator in the accumulator half of the register file:
+    // placed after the zeroing and before the store, they keep the allocator from spreading the 64
+    // four-register values over both halves (and copying them around inside the k loop).
+    auto pin_acc = [&]() {
 #pragma unroll
-        for (int vb = 0; vb < 4; ++vb)
+        for (int vb = 0; vb < kBlocks; ++vb)
 #pragma unroll
-            for (int tb = 0; tb < kTB; ++tb)
-                acc[vb][tb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[vb], f.b[tb], acc[vb][tb], 0, 0, 0);
+            for (int tb = 0; tb < kBlocks; ++tb) asm volatile("" : "+a"(acc[vb][tb]));
     };
-    // The finished tile.  A lane holds column n = lane & 31 of each 32 x 32 block and rows
-    // (i / 4) * 8 + (lane >> 5) * 4 + (i & 3), i.e. four runs of 4 consecutive m: stored like that, a
-    // store instruction would touch 32 output rows with 16 bytes each.  Each wavefront therefore turns
-    // its blocks through a private slice of LDS (the 32 KiB the two stages leave free): [32 n][128 bytes
-    // of m] at a time, 16-byte chunks XOR-swizzled by the row, written in the MFMA layout and read back
-    // as 8 lanes x 16 bytes per output row, so that every store covers whole 128-byte lines.
+    auto mfma1 = [&](const Frags& f, int i) {
+        const int vb = i / kBlocks, tb = i % kBlocks;
+        acc[vb][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.a[vb], f.b[tb], acc[vb][tb], 0, 0, 0);
+    };
+    // The finished tile.  A lane holds column n = lane & 15 of each 16 x 16 block and rows
+    // 4 (lane >> 4) .. + 3 of it: stored like that, a store instruction would touch 16 output rows with
+    // 8 or 16 bytes each.  Each wavefront therefore turns its blocks through a private 8 KiB of LDS:
+    // [64 n][128 bytes of m] at a time (4 blocks along n by 4 along m for bf16, by 2 for fp32), 16-byte
+    // chunks XOR-swizzled by the row pair, written in the MFMA layout and read back as 8 lanes x 16 bytes
+    // per output row, so that every store covers whole 128-byte lines.
     unsigned char* turn = smem + kLdsStages + wave * (kLdsTurn / kWaves);
     auto store_tile = [&](int64_t t) {
         int tm, tn;
         tile_coords(grid, t, tm, tn);
-        const int row_w = lane & 31, half = lane >> 5;           // writer: its n, its run of 4 inside a run of 8
+        const int row_w = lane & 15, quarter = lane >> 4;        // writer: its n, its run of 4 m inside the block
         const int row_r = lane >> 3, chunk_r = lane & 7;          // reader: n within a group of 8, 16-byte chunk
-        constexpr int kBlocksPerPass = kAccumulate ? 1 : 2;       // 32 fp32 or 64 bf16 entries of m are 128 bytes
+        constexpr int kMPerPass = kAccumulate ? 2 : 4;            // 32 fp32 or 64 bf16 entries of m are 128 bytes
 #pragma unroll
-        for (int tb = 0; tb < kTB; ++tb) {
-            const int n0 = tn * BN + wt * (32 * kTB) + tb * 32;
+        for (int tb0 = 0; tb0 < kBlocks; tb0 += 4) {
+            const int n0 = tn * BN + wt * 128 + tb0 * 16;
 #pragma unroll
-            for (int vb0 = 0; vb0 < 4; vb0 += kBlocksPerPass) {
-                const int m0 = tm * BM + wv * 128 + vb0 * 32;
+            for (int vb0 = 0; vb0 < kBlocks; vb0 += kMPerPass) {
+                const int m0 = tm * BM + wv * 128 + vb0 * 16;
 #pragma unroll
-                for (int vbi = 0; vbi < kBlocksPerPass; ++vbi) {
+                for (int tbi = 0; tbi < 4; ++tbi) {
+                    const int row = tbi * 16 + row_w;
+                    unsigned char* line = turn + row * 128;
+                    const int key = (row >> 1) & 7;
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const floatx16& c = acc[vb0 + vbi][tb];
+                    for (int vbi = 0; vbi < kMPerPass; ++vbi) {
+                        const floatx4& c = acc[vb0 + vbi][tb0 + tbi];
                         if (kAccumulate) {
-                            const int chunk = (q * 2 + half) ^ (row_w & 7);
-                            *reinterpret_cast<float4*>(turn + row_w * 128 + chunk * 16) =
-                                make_float4(c[q * 4 + 0], c[q * 4 + 1], c[q * 4 + 2], c[q * 4 + 3]);
+                            *reinterpret_cast<float4*>(line + (((vbi * 4 + quarter) ^ key) * 16)) =
+                                make_float4(c[0], c[1], c[2], c[3]);
                         } else {
-                            const int chunk = (vbi * 4 + q) ^ (row_w & 7);
                             uint2 w;
-                            w.x = Elem<MRL_BF16>::pack2(c[q * 4 + 0], c[q * 4 + 1]);
-                            w.y = Elem<MRL_BF16>::pack2(c[q * 4 + 2], c[q * 4 + 3]);
-                            *reinterpret_cast<uint2*>(turn + row_w * 128 + chunk * 16 + half * 8) = w;
+                            w.x = Elem<MRL_BF16>::pack2(c[0], c[1]);
+                            w.y = Elem<MRL_BF16>::pack2(c[2], c[3]);
+                            *reinterpret_cast<uint2*>(line + (((vbi * 2 + (quarter >> 1)) ^ key) * 16) + (quarter & 1) * 8) = w;
                         }
                     }
                 }
                 __builtin_amdgcn_s_waitcnt(0xC07F);            // lgkmcnt(0): the slice is written
                 __builtin_amdgcn_wave_barrier();
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
+                for (int g = 0; g < 8; ++g) {
                     const int row = g * 8 + row_r;
-                    const u32x4 v = *reinterpret_cast<const u32x4*>(turn + row * 128 + ((chunk_r ^ (row & 7)) * 16));
+                    const u32x4 v =
+                        *reinterpret_cast<const u32x4*>(turn + row * 128 + ((chunk_r ^ ((row >> 1) & 7)) * 16));
                     const int n = n0 + row;
                     const int m = m0 + chunk_r * (kAccumulate ? 4 : 8);
                     if (n < N && m < M) {                      // M % 8 == 0: a chunk is inside or outside
@@ -251,61 +270,72 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(const uint16_t* __
         }
     };
 
-    // Two-group schedule.  Wavefronts w and w + 4 share a SIMD; the four of group 0 (wave < 4) and the
-    // four of group 1 alternate between a memory phase (stage requests, fragment reads) and a compute
-    // phase (16 MFMAs), half a period apart: while one wavefront of a SIMD feeds the matrix pipe the
-    // other one issues its loads, and neither holds up the other's instruction stream.  Workgroup
-    // barriers between the phases keep the groups in step; group 1 passes one barrier before its first
-    // phase and group 0 one after its last, so that every wavefront passes the same number.
-    // Barrier p (counted from 1) is the one group 0 passes p-th in the loop.  Stage s is read by group 0
-    // between barriers 4s and 4s+3, by group 1 between 4s+1 and 4s+4; it is requested by both at the
-    // start of their first memory phase of stage s-1 (after 4s-4: stage s-2, whose buffer it takes,
-    // has been read by everybody) and every wavefront waits for its own requests before it arrives at
-    // barrier 4s.
-    const int group = wave >> 2;
-    auto barrier = [&]() {
-        __builtin_amdgcn_sched_barrier(0);
-        asm volatile("s_barrier" ::: "memory");
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    Frags fa, fb;
+    // One wavefront per SIMD: memory instructions are placed between the MFMAs of the same instruction
+    // stream (an MFMA holds the matrix pipe for 16 cycles, other instructions issue meanwhile).  A
+    // stage s (buffer s & 1) is two sub-steps of 64 MFMAs, each on a fragment set that was read during
+    // the sub-step before:
+    //   sub-step 0: MFMAs on G0 | reads G1 (s, k 32..63)  | requests 12..15 of stage s+1
+    //   wait for own requests and reads, barrier: stage s+1 has landed, buffer s & 1 is free
+    //   sub-step 1: MFMAs on G1 | reads G0 (s+1, k 0..31) | requests 0..11 of stage s+2 (into buffer s & 1)
+#define MRL_SB __builtin_amdgcn_sched_barrier(0)
+    constexpr int kMfmas = kBlocks * kBlocks, kReads = 2 * kBlocks, kLoads = 2 * kLoadsPerWave;
+    static_assert(kMfmas == 64 && kReads == 16 && kLoads == 16, "the schedule below is written for these counts");
+    Frags G0, G1;
     set_load_tile(load_tile);
-    issue_next(0);
-    if (n_stages > 1) issue_next(1);
-    __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0): stages 0 and 1 have landed
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) issue_one(0, i);
+    stage_issued();
+    __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0): stage 0 has landed
     __syncthreads();
-    if (group == 1) barrier();
+#pragma unroll
+    for (int r = 0; r < kReads; ++r) read1(G0, smem, 0, r);
+#pragma unroll
+    for (int i = 0; i < 12; ++i) issue_one(1, i);
     int stage_idx = 0;
     for (int mine = 0; mine < my_tiles; ++mine) {
         zero_acc();
+        pin_acc();
         for (int kstep = 0; kstep < n_ksteps; ++kstep, ++stage_idx) {
             const int buf = stage_idx & 1;
             const unsigned char* stage = smem + buf * kStageBytes;
-            if (stage_idx >= 1 && stage_idx + 1 < n_stages) issue_next(buf ^ 1);
-            read_frags(fa, stage, 0);
-            read_frags(fb, stage, 1);
-            __builtin_amdgcn_s_waitcnt(0xC07F);        // lgkmcnt(0)
-            barrier();
-            __builtin_amdgcn_s_setprio(1);
-            mma(fa);
-            mma(fb);
-            __builtin_amdgcn_s_setprio(0);
-            barrier();
-            read_frags(fa, stage, 2);
-            read_frags(fb, stage, 3);
-            if (group == 1) __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0)
-            else __builtin_amdgcn_s_waitcnt(0xC07F);
-            barrier();
-            __builtin_amdgcn_s_setprio(1);
-            mma(fa);
-            mma(fb);
-            __builtin_amdgcn_s_setprio(0);
-            if (group == 0) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
-            barrier();
+            const unsigned char* other = smem + (buf ^ 1) * kStageBytes;
+            MRL_SB;
+#pragma unroll
+            for (int i = 0; i < kMfmas; ++i) {
+                mfma1(G0, i);
+                MRL_SB;
+                if (i % 3 == 0 && i / 3 < kReads) {
+                    read1(G1, stage, 1, i / 3);
+                    MRL_SB;
+                }
+                if (i % 6 == 1 && i / 6 < 4) {
+                    issue_one(buf ^ 1, 12 + i / 6);
+                    MRL_SB;
+                }
+            }
+            stage_issued();
+            __builtin_amdgcn_s_waitcnt(0x0070);        // vmcnt(0) lgkmcnt(0)
+            asm volatile("s_barrier" ::: "memory");
+            MRL_SB;
+#pragma unroll
+            for (int i = 0; i < kMfmas; ++i) {
+                mfma1(G1, i);
+                MRL_SB;
+                if (i % 3 == 0 && i / 3 < kReads) {
+                    read1(G0, other, 0, i / 3);
+                    MRL_SB;
+                }
+                if (i % 5 == 1 && i / 5 < 12) {
+                    issue_one(buf, i / 5);
+                    MRL_SB;
+                }
+            }
         }
+        pin_acc();
         store_tile(first_tile + (int64_t)mine * tile_stride);
     }
-    if (group == 0) barrier();
+    __builtin_amdgcn_s_waitcnt(0x0F70);                // nothing is in flight into LDS when the workgroup ends
+#undef MRL_SB
 }
 
 // dst[c][r] = src[r][c] for r < rows, c < cols; dst has `dst_rows` >= cols rows of `ld_dst` >= rows

@@ -31,6 +31,10 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void* base, uint32_t bytes) {
 __device__ __forceinline__ u32x4 buf_load_nt(rsrc_t r, uint32_t byte_off) {
     return __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 2);
 }
+// a vector at lane offset + wavefront-uniform offset, default cache policy (data that other CUs read too)
+__device__ __forceinline__ u32x4 buf_load(rsrc_t r, uint32_t lane_byte_off, uint32_t uniform_byte_off) {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, (int)lane_byte_off, (int)uniform_byte_off, 0);
+}
 __device__ __forceinline__ void buf_store_nt(u32x4 v, rsrc_t r, uint32_t byte_off) {
     __builtin_amdgcn_raw_buffer_store_b128(v, r, (int)byte_off, 0, 2);
 }
@@ -50,6 +54,7 @@ __device__ __forceinline__ uint32_t buf_atomic_add_u32(rsrc_t r, uint32_t byte_o
 struct rsrc_t {};
 __device__ inline rsrc_t make_rsrc(const void*, uint32_t) { return rsrc_t(); }
 __device__ inline u32x4 buf_load_nt(rsrc_t, uint32_t) { return make_u32x4(0, 0, 0, 0); }
+__device__ inline u32x4 buf_load(rsrc_t, uint32_t, uint32_t) { return make_u32x4(0, 0, 0, 0); }
 __device__ inline void buf_store_nt(u32x4, rsrc_t, uint32_t) {}
 __device__ inline void buf_store_b16(uint16_t, rsrc_t, uint32_t) {}
 __device__ inline void buf_store_b32(uint32_t, rsrc_t, uint32_t) {}
