@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define MRL_VERSION 200
+#define MRL_VERSION 201
 
 enum mrl_status {
     MRL_OK = 0,
@@ -398,22 +398,17 @@ int mrl_lmhead_logprob_fwd(const void* hidden, const void* weight, int64_t n_tok
  *                                dWeight[v, h] += sum_t dlogits[t, v] * hidden[t, h]    (fp32, added)
  *
  * hidden [n_tokens, hidden_dim] and weight [vocab, hidden_dim] are dense bf16, hidden_dim % 64 == 0,
- * vocab % 4 == 0; logits / dlogits rows are logits_row_stride apart.  The backward wants the weight
- * a second time as weight_t [hidden_dim, weight_t_row_stride] = weight transposed, the row stride a
- * multiple of 64 and at least vocab, zeros in the padding (mrl_lmhead_transpose_weight makes it,
- * once per step), and dlogits rows at least that long with zeros (anything finite) in their
- * padding.  dWeight is accumulated chunk after chunk in stream order, without atomics, so the
- * result does not depend on timing.  workspace: mrl_lmhead_bwd_workspace_bytes(...) bytes, 16-byte
- * aligned, for the transposed copies of the dlogits and hidden chunks.  Nothing here allocates. */
+ * vocab % 8 == 0; logits / dlogits rows are logits_row_stride / dlogits_row_stride apart.  The
+ * backward reads hidden, weight and dlogits as they lie (no transposed copies, no workspace); it
+ * wants dlogits_row_stride a multiple of 64 (and at least vocab) with zeros in the padding columns,
+ * since it reads whole steps of 64 columns; n_tokens is arbitrary.  dWeight is accumulated chunk
+ * after chunk in stream order, without atomics, so the result does not depend on timing.  Nothing
+ * here allocates. */
 int mrl_lmhead_logits(const void* hidden, const void* weight, int64_t n_tokens, int64_t vocab,
                       int64_t hidden_dim, void* logits, int64_t logits_row_stride, void* stream);
-int mrl_lmhead_transpose_weight(const void* weight, int64_t vocab, int64_t hidden_dim, void* weight_t,
-                                int64_t weight_t_row_stride, void* stream);
-int64_t mrl_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t vocab, int64_t hidden_dim);
-int mrl_lmhead_logprob_bwd(const void* hidden, const void* weight_t, int64_t weight_t_row_stride,
-                           const void* dlogits, int64_t dlogits_row_stride, int64_t n_tokens,
-                           int64_t vocab, int64_t hidden_dim, void* d_hidden, float* d_weight,
-                           void* workspace, int64_t workspace_bytes, void* stream);
+int mrl_lmhead_logprob_bwd(const void* hidden, const void* weight, const void* dlogits,
+                           int64_t dlogits_row_stride, int64_t n_tokens, int64_t vocab,
+                           int64_t hidden_dim, void* d_hidden, float* d_weight, void* stream);
 
 /* mrl_lmhead_logprob_fwd for callers that cannot allocate device memory or pass a workspace (code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in

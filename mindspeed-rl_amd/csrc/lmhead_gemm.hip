@@ -11,11 +11,14 @@
 // column n and 4 consecutive rows m, i.e. 8 contiguous bytes of bf16 or 16 of fp32):
 //
 //     logits[t][v]  = sum_h W[v][h]      * hidden[t][h]      A = W,         B = hidden chunk
-//     dHidden[t][h] = sum_v Wt[h][v]     * dlogits[t][v]     A = W^T copy,  B = dlogits chunk
-//     dW[v][h]     += sum_t hiddenT[h][t] * dlogitsT[v][t]    A = hidden^T,  B = dlogits^T (copies)
+//     dHidden[t][h] = sum_v W[v][h]      * dlogits[t][v]     A = W (k-major), B = dlogits chunk
+//     dW[v][h]     += sum_t hidden[t][h]   * dlogits[t][v]     A = hidden,    B = dlogits chunk, both k-major
 //
-// The transposed copies are made by transpose_bf16_kernel; their padded tails are zero so that the
-// k dimension can always be walked in whole steps of 64.
+// An operand may also be given "k-major", as [K, rows] with the rows contiguous (kATrans / kBTrans):
+// its stage is then 64 k-rows by 256 rows of the operand in LDS, and the fragments (8 consecutive k per lane) come
+// out of ds_read_b64_tr_b16, the LDS read of gfx950 that transposes 4 x 4 blocks of 16-bit entries
+// across lanes.  dHidden uses it for W, dW for both operands, hidden [t][h] and dlogits [t][v] as they lie;
+// rows of k beyond K read as zero through the range check of the buffer descriptor, so K needs no padding there.
 //
 // Work distribution: one persistent 256-thread workgroup per CU (2 x 2 wavefronts, one per SIMD,
 // wavefront tile 128 x 128 in 256 accumulator registers) walks output tiles of 256 x 256.  Tiles are
@@ -68,32 +71,52 @@ __device__ __forceinline__ int64_t stage_src_offset(int wave, int lane, int j, i
     return (int64_t)row * ld + (logical & 7) * 8;
 }
 
+// The same for a k-major operand [K, rows].  Its stage is cut into 4 column blocks of 64 rows of the
+// operand; a column block holds its 64 k-rows at a pitch of 128 bytes (8 KiB), and load j of a
+// wavefront fills 1 KiB with 8 k-rows of one column block, 8 lanes per 128-byte line as for the
+// k-contiguous operand.  Inside a k-row the four 32-byte segments (16 rows of the operand, what one
+// fragment read takes from it) are permuted: byte offset ^ (f(k) << 5), f(k) = (k >> 1 & 1) |
+// ((k >> 3 & 1) << 1); with the bank half that k & 1 selects, the 8 k-rows that half a wavefront
+// reads at a time fall on different banks.  Rows at or beyond `rows_valid` (a multiple of 8) are
+// clamped to the last valid chunk.
+__device__ __forceinline__ int tr_swizzle(int k) { return (((k >> 1) & 1) | (((k >> 3) & 1) << 1)) << 5; }
+__device__ __forceinline__ int64_t stage_src_offset_kmajor(int wave, int lane, int j, int64_t ld, int rows_valid) {
+    const int q = wave * kLoadsPerWave + j;
+    const int k = 8 * (q & 7) + (lane >> 3);
+    const int byte = ((lane & 7) * 16) ^ tr_swizzle(k);
+    int row = (q >> 3) * 64 + (byte >> 1);
+    if (row >= rows_valid) row = rows_valid - 8;
+    return (int64_t)k * ld + row;
+}
+
 struct TileGrid {
-    int tiles_m, tiles_n;
+    int tiles_m, tiles_n, panel_m;
     int64_t total;
 };
 
 // Tile number -> (tile along m, tile along n).  Tiles are numbered panel by panel, a panel being
-// kPanelM tiles along m by all tiles along n; inside a panel 32 consecutive numbers are 8 (m) x 4 (n)
-// tiles, and consecutive groups of 32 walk along n.  The 8 XCDs therefore work on the same 8 tiles of
-// A at the same time (one fetch from memory serves all of them) with 4 tiles of B each, and a
-// workgroup keeps its tile of A from one of its tiles to the next.
-constexpr int kPanelM = 8;
+// panel_m tiles along m by all tiles along n; inside a panel consecutive numbers walk m first inside
+// a group of 4 tiles along n (4 consecutive numbers are one tile of A with 4 tiles of B), and the groups
+// walk along n.  With panel_m = 8 the 32 workgroups of an XCD hold 8 (m) x 4 (n) tiles and the 8 XCDs
+// 8 x 32; with 32 an XCD still holds 8 x 4 and the chip 32 x 8, which fetches less from beyond the L2
+// (B is passed over a quarter as often).
+// A workgroup keeps its tile of A from one of its tiles to the next.
 __device__ __forceinline__ void tile_coords(const TileGrid& g, int64_t t, int& tm, int& tn) {
-    const int64_t per_panel = (int64_t)kPanelM * g.tiles_n;
+    const int64_t per_panel = (int64_t)g.panel_m * g.tiles_n;
     const int p = (int)(t / per_panel);
     const int idx = (int)(t - (int64_t)p * per_panel);
-    const int pm = min(kPanelM, g.tiles_m - p * kPanelM);       // rows of tiles in this panel
+    const int pm = min(g.panel_m, g.tiles_m - p * g.panel_m);   // rows of tiles in this panel
     const int ng = idx / (pm * kTilesAlongN);
     const int rem = idx - ng * (pm * kTilesAlongN);
     const int width = min(kTilesAlongN, g.tiles_n - ng * kTilesAlongN);
-    tm = p * kPanelM + rem / width;
+    tm = p * g.panel_m + rem / width;
     tn = ng * kTilesAlongN + rem % width;
 }
 
 // kAccumulate: out is fp32 and the product is added to it; else out is bf16 and overwritten.
-template <bool kAccumulate>
-__global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(const uint16_t* __restrict__ A, int64_t lda, int M,
+// kATrans / kBTrans: the operand is k-major, [K, M] or [K, N]; else [M, K] or [N, K].
+template <bool kAccumulate, bool kATrans, bool kBTrans>
+__global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const uint16_t* __restrict__ A, int64_t lda, int M,
                                                               const uint16_t* __restrict__ B, int64_t ldb, int N, int K,
                                                               void* __restrict__ out, int64_t ldo) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -105,6 +128,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(const uint16_t* __
     grid.tiles_m = (M + BM - 1) / BM;
     grid.tiles_n = (N + BN - 1) / BN;
     grid.total = (int64_t)grid.tiles_m * grid.tiles_n;
+    // panels of 8 rows of tiles line up with the 8 x 4 blocks of an XCD; tall products take 32
+    grid.panel_m = grid.tiles_m >= 64 ? 32 : 8;
     // workgroups are dealt round-robin to the 8 XCDs: the gridDim / 8 workgroups of an XCD take
     // consecutive tile numbers
     const int per_xcd = gridDim.x >> 3;
@@ -112,37 +137,53 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(const uint16_t* __
     const int64_t tile_stride = gridDim.x;
     if (first_tile >= grid.total) return;
     const int my_tiles = (int)((grid.total - 1 - first_tile) / tile_stride) + 1;
-    const int n_ksteps = K / BK;
+    const int n_ksteps = (K + BK - 1) / BK;           // a last partial step only with k-major operands
 
     // ---- loader state: the tile whose stages are being requested
     int64_t load_tile = first_tile;
     int load_k = 0;
     int a_off[kLoadsPerWave], b_off[kLoadsPerWave];
     mrl::rsrc_t a_rsrc, b_rsrc;
+    int load_tm = 0, load_tn = 0;
+    // A k-major operand takes a descriptor per stage: its base moves by 64 k-rows (which may be more
+    // than the 4 GiB that an offset can span), and its range ends with row K, so that the k-rows of a
+    // last partial step read as zero.
+    auto set_load_stage = [&]() {
+        const int k0 = load_k * BK;
+        const int64_t k_rows = min(BK, K - k0);
+        if (kATrans)
+            a_rsrc = mrl::make_rsrc(A + (int64_t)k0 * lda + (int64_t)load_tm * BM,
+                                    (uint32_t)((k_rows * lda - (int64_t)load_tm * BM) * 2));
+        if (kBTrans)
+            b_rsrc = mrl::make_rsrc(B + (int64_t)k0 * ldb + (int64_t)load_tn * BN,
+                                    (uint32_t)((k_rows * ldb - (int64_t)load_tn * BN) * 2));
+    };
     auto set_load_tile = [&](int64_t t) {
-        int tm, tn;
-        tile_coords(grid, t, tm, tn);
-        const int rows_a = min(BM, M - tm * BM), rows_b = min(BN, N - tn * BN);
+        tile_coords(grid, t, load_tm, load_tn);
+        const int rows_a = min(BM, M - load_tm * BM), rows_b = min(BN, N - load_tn * BN);
 #pragma unroll
         for (int j = 0; j < kLoadsPerWave; ++j) {
-            a_off[j] = (int)(stage_src_offset(wave, lane, j, lda, rows_a) * 2);
-            b_off[j] = (int)(stage_src_offset(wave, lane, j, ldb, rows_b) * 2);
+            a_off[j] = (int)((kATrans ? stage_src_offset_kmajor(wave, lane, j, lda, rows_a)
+                                      : stage_src_offset(wave, lane, j, lda, rows_a)) * 2);
+            b_off[j] = (int)((kBTrans ? stage_src_offset_kmajor(wave, lane, j, ldb, rows_b)
+                                      : stage_src_offset(wave, lane, j, ldb, rows_b)) * 2);
         }
         // one descriptor per tile: byte offsets inside a tile stay below 2^32 for any operand size
-        a_rsrc = mrl::make_rsrc(A + (int64_t)tm * BM * lda, 0xffffffffu);
-        b_rsrc = mrl::make_rsrc(B + (int64_t)tn * BN * ldb, 0xffffffffu);
+        if (!kATrans) a_rsrc = mrl::make_rsrc(A + (int64_t)load_tm * BM * lda, 0xffffffffu);
+        if (!kBTrans) b_rsrc = mrl::make_rsrc(B + (int64_t)load_tn * BN * ldb, 0xffffffffu);
+        set_load_stage();
     };
-    // request i (0..15) of the stage being requested: the wavefront's 8 row groups of A, then of B
+    // request i (0..15) of the stage being requested: the wavefront's 8 groups of A, then of B
     auto issue_one = [&](int buf, int i) {
         const uint32_t k_bytes = (uint32_t)(load_k * BK * 2);
         unsigned char* dst = smem + buf * kStageBytes + (wave * kLoadsPerWave) * 1024;
         if (i < kLoadsPerWave)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (void __attribute__((address_space(3)))*)(dst + i * 1024), 16,
-                                                 a_off[i], k_bytes, 0, 0);
+                                                 a_off[i], kATrans ? 0u : k_bytes, 0, 0);
         else
             __builtin_amdgcn_raw_ptr_buffer_load_lds(
                 b_rsrc, (void __attribute__((address_space(3)))*)(dst + kOperandBytes + (i - kLoadsPerWave) * 1024), 16,
-                b_off[i - kLoadsPerWave], k_bytes, 0, 0);
+                b_off[i - kLoadsPerWave], kBTrans ? 0u : k_bytes, 0, 0);
     };
     // After the last stage of the last tile the requests go on (the schedule below has no branches):
     // they fetch valid bytes of the last tile into a buffer that nobody reads any more.
@@ -151,6 +192,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(const uint16_t* __
             load_k = 0;
             load_tile += tile_stride;
             if (load_tile < grid.total) set_load_tile(load_tile);
+            else set_load_stage();
+        } else {
+            set_load_stage();
         }
     };
 
@@ -166,19 +210,48 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(const uint16_t* __
             const int slot = ((((lane & 1) ^ par) << 3) | ((4 * ks + (lane >> 4)) ^ pair_in_block));
             frag_off[par][ks] = pair_in_block * 256 + slot * 16;
         }
-    const int a_frag = (wv * kBlocks) * 2048;                            // + vb * 2048
-    const int b_frag = kOperandBytes + (wt * kBlocks) * 2048;            // + tb * 2048
+    // The same for a k-major operand: k-row 32 ks + 8 (lane >> 4) + 4 r + ((lane >> 2) & 3) for the two
+    // reads r = 0, 1 of a fragment, 8 bytes at row 16 block + 4 (lane & 3) of it (column block
+    // block >> 2, segment block & 3 of the k-row); after the transposing read, lane i of each 16 holds
+    // row 16 block + i for 4 consecutive k.
+    int tr_off[4];                                        // [block & 3]
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int g = lane >> 4, kk = (lane >> 2) & 3;
+        tr_off[j] = (8 * g + kk) * 128 + ((j * 32) ^ tr_swizzle(8 * g + kk)) + (lane & 3) * 8;
+    }
     struct Frags {
         bf16x8 a[kBlocks], b[kBlocks];
     };
+    // fragment of 16-row block `blk` (0..15 inside the tile) of an operand whose stage starts at `op`
+    auto read_kcontig = [&](const unsigned char* op, int blk, int ks) {
+        return *reinterpret_cast<const bf16x8*>(op + blk * 2048 + frag_off[blk & 1][ks]);
+    };
+    // The transposing read goes out as inline assembly: through the builtin the compiler cannot tell it
+    // from an access to the bytes that the requests in flight are writing and waits for all of them
+    // (vmcnt(0)) before every read.  The price: it does not wait for the result either - the loop
+    // below does (lgkmcnt(0) before a sub-step consumes fragments read during the one before).
+    const unsigned smem_lds = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
+    auto read_kmajor = [&](const unsigned char* op, int blk, int ks) {
+        typedef long long2v __attribute__((ext_vector_type(2)));
+        const unsigned addr = smem_lds + (unsigned)(op - smem) + (blk >> 2) * 8192 + ks * (32 * 128) + tr_off[blk & 3];
+        long2v both;
+        long lo, hi;
+        asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo) : "v"(addr) : "memory");
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:512" : "=v"(hi) : "v"(addr) : "memory");
+        both[0] = lo;
+        both[1] = hi;
+        return __builtin_bit_cast(bf16x8, both);
+    };
     // read r (0..15) of a fragment set, in the order the MFMAs need them: a0, all of b, a1..a7
     auto read1 = [&](Frags& f, const unsigned char* stage, int ks, int r) {
-        if (r == 0) f.a[0] = *reinterpret_cast<const bf16x8*>(stage + a_frag + frag_off[0][ks]);
-        else if (r <= kBlocks)
-            f.b[r - 1] = *reinterpret_cast<const bf16x8*>(stage + b_frag + (r - 1) * 2048 + frag_off[(r - 1) & 1][ks]);
+        const bool is_a = r == 0 || r > kBlocks;
+        const int blk = r == 0 ? 0 : (r <= kBlocks ? r - 1 : r - kBlocks);
+        if (is_a)
+            f.a[blk] = kATrans ? read_kmajor(stage, wv * kBlocks + blk, ks) : read_kcontig(stage, wv * kBlocks + blk, ks);
         else
-            f.a[r - kBlocks] =
-                *reinterpret_cast<const bf16x8*>(stage + a_frag + (r - kBlocks) * 2048 + frag_off[(r - kBlocks) & 1][ks]);
+            f.b[blk] = kBTrans ? read_kmajor(stage + kOperandBytes, wt * kBlocks + blk, ks)
+                               : read_kcontig(stage + kOperandBytes, wt * kBlocks + blk, ks);
     };
     floatx4 acc[kBlocks][kBlocks];
     auto zero_acc = [&]() {
@@ -300,6 +373,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(const uint16_t* __
             const unsigned char* stage = smem + buf * kStageBytes;
             const unsigned char* other = smem + (buf ^ 1) * kStageBytes;
             MRL_SB;
+            if (kATrans || kBTrans) __builtin_amdgcn_s_waitcnt(0xC07F);      // lgkmcnt(0): G0 has arrived
+            MRL_SB;
 #pragma unroll
             for (int i = 0; i < kMfmas; ++i) {
                 mfma1(G0, i);
@@ -338,49 +413,6 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(const uint16_t* __
 #undef MRL_SB
 }
 
-// dst[c][r] = src[r][c] for r < rows, c < cols; dst has `dst_rows` >= cols rows of `ld_dst` >= rows
-// entries, and everything outside the transposed block (the padding that lets a product walk k in
-// whole steps) is written as zero.  64 x 64 tiles of 16-bit elements through LDS: 16-byte loads along
-// the source rows, 16-byte stores along the destination rows (8 two-byte LDS reads down a column
-// each; the row pitch of 33 words keeps them on different banks).  ld_src, ld_dst % 8 == 0.
-__global__ __launch_bounds__(256) void transpose_bf16_kernel(const uint16_t* __restrict__ src, int64_t ld_src, int rows,
-                                                             int cols, uint16_t* __restrict__ dst, int64_t ld_dst,
-                                                             int dst_rows) {
-    __shared__ uint16_t tile[64][66];
-    const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int v = threadIdx.x + i * 256;
-        const int r = v >> 3, cv = (v & 7) * 8;
-        uint32_t w[4] = {0u, 0u, 0u, 0u};
-        if (r0 + r < rows) {
-            const uint16_t* p = src + (int64_t)(r0 + r) * ld_src + c0 + cv;
-            if (c0 + cv + 8 <= cols) {
-                const u32x4 x = *reinterpret_cast<const u32x4*>(p);
-                w[0] = x.x; w[1] = x.y; w[2] = x.z; w[3] = x.w;
-            } else {
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    if (c0 + cv + e < cols) w[e >> 1] |= (uint32_t)p[e] << ((e & 1) * 16);
-            }
-        }
-        uint32_t* t = reinterpret_cast<uint32_t*>(&tile[r][cv]);
-        t[0] = w[0]; t[1] = w[1]; t[2] = w[2]; t[3] = w[3];
-    }
-    __syncthreads();
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int v = threadIdx.x + i * 256;
-        const int c = v >> 3, rv = (v & 7) * 8;
-        if (c0 + c >= dst_rows || r0 + rv >= ld_dst) continue;
-        uint32_t w[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-            w[e] = (uint32_t)tile[rv + 2 * e][c] | ((uint32_t)tile[rv + 2 * e + 1][c] << 16);
-        *reinterpret_cast<u32x4*>(dst + (int64_t)(c0 + c) * ld_dst + r0 + rv) = mrl::make_u32x4(w[0], w[1], w[2], w[3]);
-    }
-}
-
 int persistent_grid() {
     int dev = 0, n = 0;
     if (hipGetDevice(&dev) != hipSuccess) return 0;
@@ -392,56 +424,52 @@ int persistent_grid() {
 
 namespace mrl {
 
-int gemm_nt_bf16(const char* fn, const void* a, int64_t lda, int64_t m, const void* b, int64_t ldb, int64_t n, int64_t k,
-                 void* out, int64_t ldo, bool accumulate_f32, hipStream_t stream) {
-    MRL_REQUIRE(m > 0 && n > 0 && k > 0 && k % BK == 0 && m % 8 == 0, MRL_ERR_UNSUPPORTED,
-                "%s: product of m=%lld n=%lld k=%lld (k must be a multiple of %d, m of 8)", fn, (long long)m, (long long)n,
-                (long long)k, BK);
+template <bool kAccumulate, bool kATrans, bool kBTrans>
+static int launch_gemm(const char* fn, int grid, const void* a, int64_t lda, int64_t m, const void* b, int64_t ldb, int64_t n,
+                       int64_t k, void* out, int64_t ldo, hipStream_t stream) {
+    static const hipError_t attr = hipFuncSetAttribute((const void*)gemm_kernel<kAccumulate, kATrans, kBTrans>,
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    MRL_REQUIRE(attr == hipSuccess, MRL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS", fn, kLdsBytes);
+    hipLaunchKernelGGL((gemm_kernel<kAccumulate, kATrans, kBTrans>), dim3((unsigned)grid), dim3(kThreads), kLdsBytes, stream,
+                       (const uint16_t*)a, lda, (int)m, (const uint16_t*)b, ldb, (int)n, (int)k, out, ldo);
+    return check_launch(fn);
+}
+
+int gemm_bf16(const char* fn, const void* a, int64_t lda, int64_t m, bool a_kmajor, const void* b, int64_t ldb, int64_t n,
+              bool b_kmajor, int64_t k, void* out, int64_t ldo, bool accumulate_f32, hipStream_t stream) {
+    MRL_REQUIRE(m > 0 && n > 0 && k > 0 && m % 8 == 0, MRL_ERR_UNSUPPORTED, "%s: product of m=%lld n=%lld k=%lld (m must be a multiple of 8)",
+                fn, (long long)m, (long long)n, (long long)k);
     MRL_REQUIRE(m <= 0x7fffffffLL && n <= 0x7fffffffLL && k <= 0x7fffffffLL, MRL_ERR_UNSUPPORTED, "%s: size out of range",
                 fn);
-    MRL_REQUIRE(lda >= k && ldb >= k && ldo >= m && lda % 8 == 0 && ldb % 8 == 0 && ldo % 8 == 0, MRL_ERR_INVALID_ARG,
-                "%s: leading dimensions lda=%lld ldb=%lld ldo=%lld", fn, (long long)lda, (long long)ldb, (long long)ldo);
+    const int64_t k_steps = (k + BK - 1) / BK * BK;        // what a k-contiguous operand is read up to
+    MRL_REQUIRE((a_kmajor || b_kmajor) || k % BK == 0, MRL_ERR_UNSUPPORTED,
+                "%s: k=%lld must be a multiple of %d when no operand is k-major", fn, (long long)k, BK);
+    MRL_REQUIRE(!b_kmajor || n % 8 == 0, MRL_ERR_UNSUPPORTED, "%s: n=%lld must be a multiple of 8 for a k-major b", fn,
+                (long long)n);
+    MRL_REQUIRE(lda >= (a_kmajor ? m : k_steps) && ldb >= (b_kmajor ? n : k_steps) && ldo >= m && lda % 8 == 0 &&
+                    ldb % 8 == 0 && ldo % 8 == 0,
+                MRL_ERR_INVALID_ARG, "%s: leading dimensions lda=%lld ldb=%lld ldo=%lld", fn, (long long)lda, (long long)ldb,
+                (long long)ldo);
+    // what one buffer descriptor has to span: a tile of 256 rows, or a stage of 64 k-rows
     MRL_REQUIRE(256 * lda * 2 < (1LL << 31) && 256 * ldb * 2 < (1LL << 31), MRL_ERR_UNSUPPORTED,
-                "%s: a tile of 256 rows must stay below 2 GiB", fn);
+                "%s: 256 rows of an operand must stay below 2 GiB", fn);
     MRL_REQUIRE(aligned(a, 16) && aligned(b, 16) && aligned(out, 16), MRL_ERR_MISALIGNED,
                 "%s: operands must be 16-byte aligned", fn);
     const int grid = persistent_grid();
     MRL_REQUIRE(grid >= 8, MRL_ERR_LAUNCH, "%s: cannot query the device", fn);
-    static const hipError_t attr0 = hipFuncSetAttribute((const void*)gemm_nt_kernel<false>,
-                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-    static const hipError_t attr1 = hipFuncSetAttribute((const void*)gemm_nt_kernel<true>,
-                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-    MRL_REQUIRE(attr0 == hipSuccess && attr1 == hipSuccess, MRL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS", fn,
-                kLdsBytes);
-    if (accumulate_f32) {
-        hipLaunchKernelGGL(gemm_nt_kernel<true>, dim3((unsigned)grid), dim3(kThreads), kLdsBytes, stream,
-                           (const uint16_t*)a, lda, (int)m, (const uint16_t*)b, ldb, (int)n, (int)k, out, ldo);
-    } else {
-        hipLaunchKernelGGL(gemm_nt_kernel<false>, dim3((unsigned)grid), dim3(kThreads), kLdsBytes, stream,
-                           (const uint16_t*)a, lda, (int)m, (const uint16_t*)b, ldb, (int)n, (int)k, out, ldo);
-    }
-    return check_launch(fn);
-}
-
-int transpose_bf16(const char* fn, const void* src, int64_t ld_src, int64_t rows, int64_t cols, void* dst, int64_t ld_dst,
-                   int64_t dst_rows, hipStream_t stream) {
-    MRL_REQUIRE(rows >= 0 && cols >= 0 && ld_src >= cols && ld_dst >= rows && dst_rows >= cols && ld_src % 8 == 0 &&
-                    ld_dst % 8 == 0 && aligned(src, 16) && aligned(dst, 16),
-                MRL_ERR_INVALID_ARG, "%s: transpose of %lld x %lld (ld %lld) into %lld x %lld (16-byte aligned rows)", fn,
-                (long long)rows, (long long)cols, (long long)ld_src, (long long)dst_rows, (long long)ld_dst);
-    if (dst_rows == 0 || ld_dst == 0) return MRL_OK;
-    const int64_t gx = (ld_dst + 63) / 64, gy = (dst_rows + 63) / 64;
-    MRL_REQUIRE(gx <= 0x7fffffffLL && gy <= 65535, MRL_ERR_UNSUPPORTED, "%s: grid too large", fn);
-    hipLaunchKernelGGL(transpose_bf16_kernel, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, stream,
-                       (const uint16_t*)src, ld_src, (int)rows, (int)cols, (uint16_t*)dst, ld_dst, (int)dst_rows);
-    return check_launch(fn);
+    if (!a_kmajor && !b_kmajor && !accumulate_f32)
+        return launch_gemm<false, false, false>(fn, grid, a, lda, m, b, ldb, n, k, out, ldo, stream);
+    if (a_kmajor && !b_kmajor && !accumulate_f32)
+        return launch_gemm<false, true, false>(fn, grid, a, lda, m, b, ldb, n, k, out, ldo, stream);
+    if (a_kmajor && b_kmajor && accumulate_f32)
+        return launch_gemm<true, true, true>(fn, grid, a, lda, m, b, ldb, n, k, out, ldo, stream);
+    MRL_REQUIRE(false, MRL_ERR_UNSUPPORTED, "%s: this combination of operand layouts is not built", fn);
+    return MRL_ERR_UNSUPPORTED;
 }
 
 }  // namespace mrl
 
 // ------------------------------------------------------------------------------------------ C ABI
-static int64_t round_up(int64_t x, int64_t to) { return (x + to - 1) / to * to; }
-
 extern "C" int mrl_lmhead_logits(const void* hidden, const void* weight, int64_t n_tokens, int64_t vocab,
                                  int64_t hidden_dim, void* logits, int64_t logits_row_stride, void* stream) {
     const char* fn = "mrl_lmhead_logits";
@@ -454,64 +482,31 @@ extern "C" int mrl_lmhead_logits(const void* hidden, const void* weight, int64_t
     MRL_REQUIRE(logits_row_stride >= vocab, MRL_ERR_INVALID_ARG, "%s: logits_row_stride below vocab", fn);
     if (n_tokens == 0) return MRL_OK;
     MRL_REQUIRE(hidden && weight && logits, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
-    return mrl::gemm_nt_bf16(fn, weight, hidden_dim, vocab, hidden, hidden_dim, n_tokens, hidden_dim, logits,
-                             logits_row_stride, false, mrl::as_stream(stream));
+    return mrl::gemm_bf16(fn, weight, hidden_dim, vocab, false, hidden, hidden_dim, n_tokens, false, hidden_dim, logits,
+                          logits_row_stride, false, mrl::as_stream(stream));
 }
 
-extern "C" int64_t mrl_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t vocab, int64_t hidden_dim) {
-    if (n_tokens <= 0 || vocab <= 0 || hidden_dim <= 0) return 0;
-    const int64_t t_pad = round_up(n_tokens, BK);
-    // dlogits^T [vocab, t_pad] and hidden^T [hidden_dim, t_pad]
-    return (round_up(vocab, 8) + hidden_dim) * t_pad * 2;
-}
-
-extern "C" int mrl_lmhead_transpose_weight(const void* weight, int64_t vocab, int64_t hidden_dim, void* weight_t,
-                                           int64_t weight_t_row_stride, void* stream) {
-    const char* fn = "mrl_lmhead_transpose_weight";
-    MRL_REQUIRE(vocab > 0 && hidden_dim > 0 && weight_t_row_stride >= vocab && weight_t_row_stride % BK == 0,
-                MRL_ERR_INVALID_ARG, "%s: vocab=%lld hidden_dim=%lld row stride=%lld (a multiple of %d, at least vocab)", fn,
-                (long long)vocab, (long long)hidden_dim, (long long)weight_t_row_stride, BK);
-    MRL_REQUIRE(weight && weight_t, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
-    return mrl::transpose_bf16(fn, weight, hidden_dim, vocab, hidden_dim, weight_t, weight_t_row_stride, hidden_dim,
-                               mrl::as_stream(stream));
-}
-
-extern "C" int mrl_lmhead_logprob_bwd(const void* hidden, const void* weight_t, int64_t weight_t_row_stride,
-                                      const void* dlogits, int64_t dlogits_row_stride, int64_t n_tokens, int64_t vocab,
-                                      int64_t hidden_dim, void* d_hidden, float* d_weight, void* workspace,
-                                      int64_t workspace_bytes, void* stream) {
+extern "C" int mrl_lmhead_logprob_bwd(const void* hidden, const void* weight, const void* dlogits,
+                                      int64_t dlogits_row_stride, int64_t n_tokens, int64_t vocab, int64_t hidden_dim,
+                                      void* d_hidden, float* d_weight, void* stream) {
     const char* fn = "mrl_lmhead_logprob_bwd";
     MRL_REQUIRE(n_tokens >= 0 && vocab > 0 && hidden_dim > 0, MRL_ERR_INVALID_ARG,
                 "%s: n_tokens=%lld vocab=%lld hidden_dim=%lld", fn, (long long)n_tokens, (long long)vocab,
                 (long long)hidden_dim);
-    MRL_REQUIRE(hidden_dim % BK == 0, MRL_ERR_UNSUPPORTED, "%s: hidden_dim=%lld must be a multiple of %d", fn,
-                (long long)hidden_dim, BK);
-    MRL_REQUIRE(weight_t_row_stride % BK == 0 && weight_t_row_stride >= vocab && dlogits_row_stride >= weight_t_row_stride,
-                MRL_ERR_INVALID_ARG,
-                "%s: weight_t_row_stride=%lld must be a multiple of %d and at least vocab, dlogits_row_stride=%lld at "
-                "least that (the padding columns of both must hold zeros)", fn, (long long)weight_t_row_stride, BK,
-                (long long)dlogits_row_stride);
+    MRL_REQUIRE(hidden_dim % 8 == 0 && vocab % 8 == 0, MRL_ERR_UNSUPPORTED,
+                "%s: hidden_dim=%lld and vocab=%lld must be multiples of 8", fn, (long long)hidden_dim, (long long)vocab);
+    MRL_REQUIRE(dlogits_row_stride % BK == 0 && dlogits_row_stride >= vocab, MRL_ERR_INVALID_ARG,
+                "%s: dlogits_row_stride=%lld must be a multiple of %d and at least vocab (the padding columns must hold "
+                "zeros)", fn, (long long)dlogits_row_stride, BK);
     if (n_tokens == 0) return MRL_OK;
-    MRL_REQUIRE(hidden && weight_t && dlogits && d_hidden && d_weight && workspace, MRL_ERR_INVALID_ARG, "%s: NULL pointer",
-                fn);
-    MRL_REQUIRE(workspace_bytes >= mrl_lmhead_bwd_workspace_bytes(n_tokens, vocab, hidden_dim), MRL_ERR_INVALID_ARG,
-                "%s: workspace of %lld bytes, need %lld", fn, (long long)workspace_bytes,
-                (long long)mrl_lmhead_bwd_workspace_bytes(n_tokens, vocab, hidden_dim));
-    MRL_REQUIRE(mrl::aligned(workspace, 16), MRL_ERR_MISALIGNED, "%s: workspace must be 16-byte aligned", fn);
+    MRL_REQUIRE(hidden && weight && dlogits && d_hidden && d_weight, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
     hipStream_t s = mrl::as_stream(stream);
-    const int64_t k_vocab = weight_t_row_stride;             // the padded vocabulary: zeros beyond `vocab`
-    // dHidden[t][h] = sum_v Wt[h][v] * dlogits[t][v]
-    int rc = mrl::gemm_nt_bf16(fn, weight_t, weight_t_row_stride, hidden_dim, dlogits, dlogits_row_stride, n_tokens,
-                               k_vocab, d_hidden, hidden_dim, false, s);
+    // dHidden[t][h] = sum_v W[v][h] * dlogits[t][v]: the weight as it lies is the k-major operand; its rows
+    // beyond vocab read as zero, dlogits is read up to the next multiple of 64 columns
+    int rc = mrl::gemm_bf16(fn, weight, hidden_dim, hidden_dim, true, dlogits, dlogits_row_stride, n_tokens, false, vocab,
+                            d_hidden, hidden_dim, false, s);
     if (rc != MRL_OK) return rc;
-    // dW[v][h] += sum_t hidden^T[h][t] * dlogits^T[v][t], over transposed copies with zero tails
-    const int64_t t_pad = round_up(n_tokens, BK);
-    const int64_t v4 = round_up(vocab, 8);
-    uint16_t* dz_t = reinterpret_cast<uint16_t*>(workspace);
-    uint16_t* h_t = dz_t + v4 * t_pad;
-    rc = mrl::transpose_bf16(fn, dlogits, dlogits_row_stride, n_tokens, vocab, dz_t, t_pad, v4, s);
-    if (rc != MRL_OK) return rc;
-    rc = mrl::transpose_bf16(fn, hidden, hidden_dim, n_tokens, hidden_dim, h_t, t_pad, hidden_dim, s);
-    if (rc != MRL_OK) return rc;
-    return mrl::gemm_nt_bf16(fn, h_t, t_pad, hidden_dim, dz_t, t_pad, vocab, t_pad, d_weight, hidden_dim, true, s);
+    // dW[v][h] += sum_t hidden[t][h] * dlogits[t][v]: both operands k-major as they lie, any n_tokens
+    return mrl::gemm_bf16(fn, hidden, hidden_dim, hidden_dim, true, dlogits, dlogits_row_stride, vocab, true, n_tokens,
+                          d_weight, hidden_dim, true, s);
 }

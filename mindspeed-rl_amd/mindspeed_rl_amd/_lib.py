@@ -61,9 +61,7 @@ SIGNATURES = {
     "mrl_lmhead_workspace_bytes": [_i64, _i64],
     "mrl_lmhead_logprob_fwd": [_vp, _vp, _i64, _i64, _i64, _vp, _int, _f32, _vp, _vp, _vp, _vp, _i64, _vp],
     "mrl_lmhead_logits": [_vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp],
-    "mrl_lmhead_transpose_weight": [_vp, _i64, _i64, _vp, _i64, _vp],
-    "mrl_lmhead_bwd_workspace_bytes": [_i64, _i64, _i64],
-    "mrl_lmhead_logprob_bwd": [_vp, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _vp],
+    "mrl_lmhead_logprob_bwd": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp],
     "mrl_lmhead_static_max_tokens": [],
     "mrl_lmhead_logprob_fwd_static": [_vp, _vp, _i64, _i64, _i64, _vp, _int, _f32, _vp, _vp, _vp, _vp],
     "mrl_group_standardize": [_vp, _int, _i64, _i64, ctypes.c_double, _vp, _vp],
@@ -77,7 +75,7 @@ SIGNATURES = {
     "mrl_bandwidth_probe": [_int, _vp, _vp, _i64, _i64, _vp],
 }
 _RESTYPES = {"mrl_last_error": ctypes.c_char_p, "mrl_fused_workspace_bytes": ctypes.c_int64, "mrl_fused_max_vocab": ctypes.c_int64,
-             "mrl_lmhead_workspace_bytes": ctypes.c_int64, "mrl_lmhead_bwd_workspace_bytes": ctypes.c_int64, "mrl_lmhead_static_max_tokens": ctypes.c_int64}
+             "mrl_lmhead_workspace_bytes": ctypes.c_int64, "mrl_lmhead_static_max_tokens": ctypes.c_int64}
 
 _lib = None
 

@@ -169,8 +169,8 @@ class _FusedLmHeadLoss(torch.autograd.Function):
             terms_all, row_terms = row_terms, torch.empty(max(n_rows, 1) * 8, dtype=torch.float32, device=dev)
             ent = torch.empty(max(n_rows, 1), dtype=torch.float32, device=dev) if want_ent else None
         chunk = max(1, min(int(cfg["chunk_rows"]), n_rows))
-        # the chunk of logits: rows padded to whole k-steps of the backward products; the padding
-        # columns are zeroed once and never written (they meet the zero padding of the transposed weight)
+        # the chunk of logits: rows padded to whole k-steps of the dHidden product; the padding columns
+        # are zeroed once and never written (they meet rows of the weight that read as zero)
         v_pad = _round_up(vocab, 64)
         if v_pad != vocab:
             logits = torch.zeros((chunk, v_pad), dtype=h2d.dtype, device=dev)
@@ -178,10 +178,6 @@ class _FusedLmHeadLoss(torch.autograd.Function):
             logits = torch.empty((chunk, v_pad), dtype=h2d.dtype, device=dev)
         d_hidden = torch.empty_like(h2d)
         d_weight32 = torch.zeros((vocab, hdim), dtype=torch.float32, device=dev)
-        w_t = torch.empty((hdim, v_pad), dtype=w.dtype, device=dev)
-        _lib.call("mrl_lmhead_transpose_weight", _lib.ptr(w), vocab, hdim, _lib.ptr(w_t), v_pad, stream)
-        bwd_bytes = lib.mrl_lmhead_bwd_workspace_bytes(chunk, vocab, hdim)
-        bwd_ws = torch.empty(max(bwd_bytes, 16), dtype=torch.uint8, device=dev)
         sweep_bytes = lib.mrl_fused_workspace_bytes(_lib.dtype_code(logits), chunk, vocab)
         sweep_ws = torch.empty(max(sweep_bytes, 16), dtype=torch.uint8, device=dev)
         esz = h2d.element_size()
@@ -196,8 +192,8 @@ class _FusedLmHeadLoss(torch.autograd.Function):
                 cfg["kl_coef"], cfg["entropy_coeff"], grad_scale, _lib.ptr(scale_dev), _lib.ptr(logits), v_pad, None,
                 (ent.data_ptr() + c0 * 4) if want_ent else None, row_terms.data_ptr() + c0 * 32, _lib.ptr(sweep_ws),
                 sweep_bytes, stream)
-            _timed("mrl_lmhead_logprob_bwd", rows, dev, h_c, _lib.ptr(w_t), v_pad, _lib.ptr(logits), v_pad, rows, vocab,
-                   hdim, d_hidden.data_ptr() + c0 * hdim * esz, _lib.ptr(d_weight32), _lib.ptr(bwd_ws), bwd_bytes, stream)
+            _timed("mrl_lmhead_logprob_bwd", rows, dev, h_c, _lib.ptr(w), _lib.ptr(logits), v_pad, rows, vocab, hdim,
+                   d_hidden.data_ptr() + c0 * hdim * esz, _lib.ptr(d_weight32), stream)
         if live is not None:
             compact_dh, compact_terms = d_hidden, row_terms
             d_hidden = torch.zeros_like(h_all)

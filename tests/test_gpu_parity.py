@@ -1418,13 +1418,20 @@ def test_lmhead_products_through_the_c_abi(dev, tokens, vocab, hdim):
     """The three matrix products of the lm_head training step, hand-written for the matrix cores:
     logits = hidden W^T (mrl_lmhead_logits), dHidden = dlogits W and dWeight += dlogits^T hidden
     (mrl_lmhead_logprob_bwd), against fp32 products of the same bf16 operands on the CPU: ragged token
-    and vocabulary tiles, a vocabulary that is no multiple of the 64-wide k-step (zero padding), two
-    accumulating calls into one dWeight, untouched padding."""
+    and vocabulary tiles, a vocabulary and token counts that are no multiples of the 64-wide k-step, two
+    accumulating calls into one dWeight, untouched padding.  The backward reads hidden, weight and
+    dlogits as they lie: memory right behind hidden and weight is filled with NaN to show that rows of k
+    beyond the operand are not read."""
     gen = torch.Generator().manual_seed(tokens * 7 + vocab)
     h = torch.randn(tokens, hdim, generator=gen).to(torch.bfloat16)
     w = (torch.randn(vocab, hdim, generator=gen) * (2.0 / hdim ** 0.5)).to(torch.bfloat16)
     dz = (torch.randn(tokens, vocab, generator=gen) * 0.01).to(torch.bfloat16)
-    hd, wd = h.to(dev), w.to(dev)
+    # 64 rows of NaN behind each operand: a k-step that ran past the last row would pick them up
+    hbuf = torch.full((tokens + 64, hdim), float("nan"), dtype=torch.bfloat16, device=dev)
+    wbuf = torch.full((vocab + 64, hdim), float("nan"), dtype=torch.bfloat16, device=dev)
+    hbuf[:tokens] = h.to(dev)
+    wbuf[:vocab] = w.to(dev)
+    hd, wd = hbuf[:tokens], wbuf[:vocab]
     lib = _lib.load()
     stream = _lib.stream(dev)
     v_pad = (vocab + 63) // 64 * 64
@@ -1434,28 +1441,25 @@ def test_lmhead_products_through_the_c_abi(dev, tokens, vocab, hdim):
     err = (z[:, :vocab].float().cpu() - want_z).abs().max().item()
     assert err <= 2 ** -8 * want_z.abs().max().item() + 1e-6                   # one bf16 rounding of the result
     assert (z[:, vocab:] == 7.0).all().item()                                   # the padding is not written
-    # backward: the padding of dlogits and of the transposed weight must be zero
-    dzd = torch.zeros((tokens, v_pad), dtype=torch.bfloat16, device=dev)
-    dzd[:, :vocab] = dz.to(dev)
-    w_t = torch.full((hdim, v_pad), 3.0, dtype=torch.bfloat16, device=dev)
-    _lib.call("mrl_lmhead_transpose_weight", wd.data_ptr(), vocab, hdim, w_t.data_ptr(), v_pad, stream)
-    assert torch.equal(w_t[:, :vocab].cpu(), w.t()) and not w_t[:, vocab:].any().item()
-    ws_bytes = lib.mrl_lmhead_bwd_workspace_bytes(tokens, vocab, hdim)
-    ws = torch.full((ws_bytes,), 0xFF, dtype=torch.uint8, device=dev)
+    # backward: the padding columns of dlogits must be zero; rows behind its last one hold NaN
+    dzbuf = torch.full((tokens + 64, v_pad), float("nan"), dtype=torch.bfloat16, device=dev)
+    dzbuf[:tokens] = 0
+    dzbuf[:tokens, :vocab] = dz.to(dev)
+    dzd = dzbuf[:tokens]
     dh = torch.full((tokens, hdim), 5.0, dtype=torch.bfloat16, device=dev)
     dw = torch.ones(vocab, hdim, dtype=torch.float32, device=dev)
     for _ in range(2):                                                           # dWeight accumulates
-        _lib.call("mrl_lmhead_logprob_bwd", hd.data_ptr(), w_t.data_ptr(), v_pad, dzd.data_ptr(), v_pad, tokens, vocab,
-                  hdim, dh.data_ptr(), dw.data_ptr(), ws.data_ptr(), ws_bytes, stream)
+        _lib.call("mrl_lmhead_logprob_bwd", hd.data_ptr(), wd.data_ptr(), dzd.data_ptr(), v_pad, tokens, vocab, hdim,
+                  dh.data_ptr(), dw.data_ptr(), stream)
     want_dh = dz.float() @ w.float()
     want_dw = 1.0 + 2.0 * (dz.float().t() @ h.float())
     assert (dh.float().cpu() - want_dh).abs().max().item() <= 2 ** -7 * want_dh.abs().max().item() + 1e-9
     assert (dw.cpu() - want_dw).abs().max().item() <= 2 ** -7 * (want_dw - 1.0).abs().max().item() + 1e-6
     # rejected shapes: nothing is launched
     assert lib.mrl_lmhead_logits(hd.data_ptr(), wd.data_ptr(), tokens, vocab, hdim - 8, z.data_ptr(), v_pad, stream) == -2
-    assert lib.mrl_lmhead_logprob_bwd(hd.data_ptr(), w_t.data_ptr(), v_pad, dzd.data_ptr(), v_pad, tokens, vocab, hdim,
-                                      dh.data_ptr(), dw.data_ptr(), ws.data_ptr(), 16, stream) == -1
-    assert b"workspace" in lib.mrl_last_error()
+    assert lib.mrl_lmhead_logprob_bwd(hd.data_ptr(), wd.data_ptr(), dzd.data_ptr(), v_pad - 8, tokens, vocab, hdim,
+                                      dh.data_ptr(), dw.data_ptr(), stream) == -1
+    assert b"dlogits_row_stride" in lib.mrl_last_error()
 
 
 def test_copy_kernel_moves_bytes(dev):

@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), "libmrl_hip.so lacks %s" % name
     # and the ctypes table binds exactly the declared set
     assert sorted(_lib.SIGNATURES) == declared
-    assert lib.mrl_version() == 200
+    assert lib.mrl_version() == 201
     assert lib.mrl_last_error() == b""
     assert os.path.dirname(_lib.library_path()).startswith(ROOT), "the library must live in-tree"
 
@@ -133,11 +133,11 @@ def test_argument_validation_launches_nothing():
     assert lib.mrl_lmhead_logits(p, p, 4, 1001, 128, p, 1008, None) == -2                   # vocab % 8
     assert lib.mrl_lmhead_logits(p, p, 4, 1000, 128, p, 992, None) == -1                    # row stride below vocab
     assert lib.mrl_lmhead_logits(None, None, 0, 1000, 128, None, 1000, None) == 0
-    assert lib.mrl_lmhead_bwd_workspace_bytes(100, 1000, 128) == (1000 + 128) * 128 * 2
-    assert lib.mrl_lmhead_transpose_weight(p, 1000, 128, p, 1000, None) == -1               # stride not a multiple of 64
-    assert lib.mrl_lmhead_logprob_bwd(p, p, 1024, p, 1000, 4, 1000, 128, p, p, p, 1 << 30, None) == -1
+    assert lib.mrl_lmhead_logprob_bwd(p, p, p, 1000, 4, 1000, 128, p, p, None) == -1        # stride not a multiple of 64
     assert b"dlogits_row_stride" in lib.mrl_last_error()
-    assert lib.mrl_lmhead_logprob_bwd(p, p, 1024, p, 1024, 4, 1000, 128, p, p, None, 0, None) == -1
+    assert lib.mrl_lmhead_logprob_bwd(p, p, p, 1024, 4, 1000, 128, p, None, None) == -1     # NULL dWeight
+    assert lib.mrl_lmhead_logprob_bwd(p, p, p, 1024, 4, 1004, 128, p, p, None) == -2        # vocab % 8
+    assert lib.mrl_lmhead_logprob_bwd(None, None, None, 1024, 0, 1000, 128, None, None, None) == 0
     # PPO value side
     assert lib.mrl_gae_scan(p, p + 512, 2, 8, 1.0, 0.95, p, p + 1024, None) == -1 and b"alias" in lib.mrl_last_error()
     assert lib.mrl_gae_scan(p, p + 512, 2, 0, 1.0, 0.95, p + 1024, p + 2048, None) == -1
