@@ -1,93 +1,38 @@
-// bf16 matrix products of the lm_head training step for gfx950: operands go from global memory
-// straight into LDS (buffer_load ... lds), two 64 KiB stages, XOR-swizzled 16-byte chunks,
-// v_mfma_f32_16x16x32_bf16 (at the board's power limit this shape runs about 18 % faster than the
-// same flops as 32x32x16), memory instructions placed between the MFMAs of one instruction stream.
+// bf16 matrix products of the lm_head training step for gfx950 on the shared tile loop (lmhead_tile.h).
 //
 // One kernel covers the three products of the step, because each of them can be put in the form
 //
-//     out[n][m] (+)= sum_k A[m][k] * B[n][k]          A: [M, K], B: [N, K], both with k contiguous
+//     out[n][m] (+)= sum_k A[m][k] * B[n][k]
 //
 // (the MFMA's M is the fast dimension of the output: in the 16x16 result layout a lane owns ONE
 // column n and 4 consecutive rows m, i.e. 8 contiguous bytes of bf16 or 16 of fp32):
 //
-//     logits[t][v]  = sum_h W[v][h]      * hidden[t][h]      A = W,         B = hidden chunk
+//     logits[t][v]  = sum_h W[v][h]      * hidden[t][h]      A = W,           B = hidden chunk
 //     dHidden[t][h] = sum_v W[v][h]      * dlogits[t][v]     A = W (k-major), B = dlogits chunk
-//     dW[v][h]     += sum_t hidden[t][h]   * dlogits[t][v]     A = hidden,    B = dlogits chunk, both k-major
+//     dW[v][h]     += sum_t hidden[t][h] * dlogits[t][v]     A = hidden,      B = dlogits chunk, both k-major
 //
-// An operand may also be given "k-major", as [K, rows] with the rows contiguous (kATrans / kBTrans):
-// its stage is then 64 k-rows by 256 rows of the operand in LDS, and the fragments (8 consecutive k per lane) come
-// out of ds_read_b64_tr_b16, the LDS read of gfx950 that transposes 4 x 4 blocks of 16-bit entries
-// across lanes.  dHidden uses it for W, dW for both operands, hidden [t][h] and dlogits [t][v] as they lie;
-// rows of k beyond K read as zero through the range check of the buffer descriptor, so K needs no padding there.
+// so the backward reads hidden, W and dlogits as they lie: no transposed copies.
 //
-// Work distribution: one persistent 256-thread workgroup per CU (2 x 2 wavefronts, one per SIMD,
-// wavefront tile 128 x 128 in 256 accumulator registers) walks output tiles of 256 x 256.  Tiles are
+// Work distribution: one persistent workgroup per CU walks output tiles of 256 x 256.  Tiles are
 // numbered so that 32 consecutive numbers are 8 tiles along m by 4 along n, and the 32 workgroups
 // that share an XCD (and its L2) take 32 consecutive numbers at a time: the 4 that stream the same A
 // tile and the 8 that stream the same B tile run side by side (see tile_coords for the order of the
-// groups of 32).  The loop runs over the flattened (tile, k-step) sequence of a workgroup, so the
-// first loads of its next tile are in flight while the current one is stored.
+// groups of 32).
 #include <stdlib.h>
 
 #include "lmhead_gemm.h"
+#include "lmhead_tile.h"
 #include "mrl_internal.h"
 #include "vocab_common.h"
 
 namespace {
 
 using namespace mrl_vocab;
+using namespace mrl_tile;
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-
-// Wavefront layout of the 256 x 256 tile: 2 wavefronts along m (128 rows of A each) by 2 along n
-// (128 rows of B each); a wavefront owns 8 x 8 MFMA blocks of 16 x 16.
-constexpr int kWavesN = 2;
-constexpr int kWaves = 2 * kWavesN;
-constexpr int kThreads = 64 * kWaves;
-constexpr int kBlocks = 8;                       // 16-row blocks of A, and of B, per wavefront
-constexpr int kLoadsPerWave = 32 / kWaves;       // 8-row groups of an operand that a wavefront brings in
-constexpr int BM = 256;                          // rows of A per tile
-constexpr int BN = 256;                          // rows of B per tile
-constexpr int BK = 64;                           // k elements per LDS stage
-constexpr int kOperandBytes = 256 * BK * 2;      // one operand of one stage: 256 rows x 128 bytes
-constexpr int kStageBytes = 2 * kOperandBytes;   // A then B
-constexpr int kLdsStages = 2 * kStageBytes;      // two stages
 constexpr int kLdsTurn = 32 * 1024;              // where the wavefronts turn their result blocks (store_tile)
 constexpr int kLdsBytes = kLdsStages + kLdsTurn;
 constexpr int kTilesAlongN = 4;                  // tiles along n in a group of consecutive tile numbers
-
-// Element offset (row * ld + column, without the k-step) of the chunk that lane `lane` of wavefront
-// `wave` brings in with its load j (0..7) of an operand tile with `rows_valid` rows left (rows beyond
-// are clamped to the last valid one; their products are never stored).  Physical slot of a 16-byte
-// chunk inside its 256-byte pair of rows: logical slot ^ (pair & 15), logical = (row & 1) * 8 + chunk.
-__device__ __forceinline__ int64_t stage_src_offset(int wave, int lane, int j, int64_t ld, int rows_valid) {
-    const int phys_row = (wave * kLoadsPerWave + j) * 8 + (lane >> 3);
-    const int pair = phys_row >> 1;
-    const int slot = ((phys_row & 1) << 3) | (lane & 7);
-    const int logical = slot ^ (pair & 15);
-    int row = 2 * pair + (logical >> 3);
-    if (row >= rows_valid) row = rows_valid - 1;
-    return (int64_t)row * ld + (logical & 7) * 8;
-}
-
-// The same for a k-major operand [K, rows].  Its stage is cut into 4 column blocks of 64 rows of the
-// operand; a column block holds its 64 k-rows at a pitch of 128 bytes (8 KiB), and load j of a
-// wavefront fills 1 KiB with 8 k-rows of one column block, 8 lanes per 128-byte line as for the
-// k-contiguous operand.  Inside a k-row the four 32-byte segments (16 rows of the operand, what one
-// fragment read takes from it) are permuted: byte offset ^ (f(k) << 5), f(k) = (k >> 1 & 1) |
-// ((k >> 3 & 1) << 1); with the bank half that k & 1 selects, the 8 k-rows that half a wavefront
-// reads at a time fall on different banks.  Rows at or beyond `rows_valid` (a multiple of 8) are
-// clamped to the last valid chunk.
-__device__ __forceinline__ int tr_swizzle(int k) { return (((k >> 1) & 1) | (((k >> 3) & 1) << 1)) << 5; }
-__device__ __forceinline__ int64_t stage_src_offset_kmajor(int wave, int lane, int j, int64_t ld, int rows_valid) {
-    const int q = wave * kLoadsPerWave + j;
-    const int k = 8 * (q & 7) + (lane >> 3);
-    const int byte = ((lane & 7) * 16) ^ tr_swizzle(k);
-    int row = (q >> 3) * 64 + (byte >> 1);
-    if (row >= rows_valid) row = rows_valid - 8;
-    return (int64_t)k * ld + row;
-}
 
 struct TileGrid {
     int tiles_m, tiles_n, panel_m;
@@ -113,168 +58,37 @@ __device__ __forceinline__ void tile_coords(const TileGrid& g, int64_t t, int& t
     tn = ng * kTilesAlongN + rem % width;
 }
 
+// The tiles of one workgroup: number first + j * stride.
+struct StridedTiles {
+    TileGrid grid;
+    int64_t first, stride;
+    int n_tiles;
+    __device__ __forceinline__ void coords(int j, int& tm, int& tn) const { tile_coords(grid, first + j * stride, tm, tn); }
+};
+
 // kAccumulate: out is fp32 and the product is added to it; else out is bf16 and overwritten.
 // kATrans / kBTrans: the operand is k-major, [K, M] or [K, N]; else [M, K] or [N, K].
 template <bool kAccumulate, bool kATrans, bool kBTrans>
 __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const uint16_t* __restrict__ A, int64_t lda, int M,
-                                                              const uint16_t* __restrict__ B, int64_t ldb, int N, int K,
-                                                              void* __restrict__ out, int64_t ldo) {
+                                                           const uint16_t* __restrict__ B, int64_t ldb, int N, int K,
+                                                           void* __restrict__ out, int64_t ldo) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wv = wave / kWavesN, wt = wave % kWavesN;
 
-    TileGrid grid;
-    grid.tiles_m = (M + BM - 1) / BM;
-    grid.tiles_n = (N + BN - 1) / BN;
-    grid.total = (int64_t)grid.tiles_m * grid.tiles_n;
+    StridedTiles seq;
+    seq.grid.tiles_m = (M + BM - 1) / BM;
+    seq.grid.tiles_n = (N + BN - 1) / BN;
+    seq.grid.total = (int64_t)seq.grid.tiles_m * seq.grid.tiles_n;
     // panels of 8 rows of tiles line up with the 8 x 4 blocks of an XCD; tall products take 32
-    grid.panel_m = grid.tiles_m >= 64 ? 32 : 8;
+    seq.grid.panel_m = seq.grid.tiles_m >= 64 ? 32 : 8;
     // workgroups are dealt round-robin to the 8 XCDs: the gridDim / 8 workgroups of an XCD take
     // consecutive tile numbers
     const int per_xcd = gridDim.x >> 3;
-    const int64_t first_tile = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    const int64_t tile_stride = gridDim.x;
-    if (first_tile >= grid.total) return;
-    const int my_tiles = (int)((grid.total - 1 - first_tile) / tile_stride) + 1;
-    const int n_ksteps = (K + BK - 1) / BK;           // a last partial step only with k-major operands
+    seq.first = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    seq.stride = gridDim.x;
+    seq.n_tiles = seq.first < seq.grid.total ? (int)((seq.grid.total - 1 - seq.first) / seq.stride) + 1 : 0;
 
-    // ---- loader state: the tile whose stages are being requested
-    int64_t load_tile = first_tile;
-    int load_k = 0;
-    int a_off[kLoadsPerWave], b_off[kLoadsPerWave];
-    mrl::rsrc_t a_rsrc, b_rsrc;
-    int load_tm = 0, load_tn = 0;
-    // A k-major operand takes a descriptor per stage: its base moves by 64 k-rows (which may be more
-    // than the 4 GiB that an offset can span), and its range ends with row K, so that the k-rows of a
-    // last partial step read as zero.
-    auto set_load_stage = [&]() {
-        const int k0 = load_k * BK;
-        const int64_t k_rows = min(BK, K - k0);
-        if (kATrans)
-            a_rsrc = mrl::make_rsrc(A + (int64_t)k0 * lda + (int64_t)load_tm * BM,
-                                    (uint32_t)((k_rows * lda - (int64_t)load_tm * BM) * 2));
-        if (kBTrans)
-            b_rsrc = mrl::make_rsrc(B + (int64_t)k0 * ldb + (int64_t)load_tn * BN,
-                                    (uint32_t)((k_rows * ldb - (int64_t)load_tn * BN) * 2));
-    };
-    auto set_load_tile = [&](int64_t t) {
-        tile_coords(grid, t, load_tm, load_tn);
-        const int rows_a = min(BM, M - load_tm * BM), rows_b = min(BN, N - load_tn * BN);
-#pragma unroll
-        for (int j = 0; j < kLoadsPerWave; ++j) {
-            a_off[j] = (int)((kATrans ? stage_src_offset_kmajor(wave, lane, j, lda, rows_a)
-                                      : stage_src_offset(wave, lane, j, lda, rows_a)) * 2);
-            b_off[j] = (int)((kBTrans ? stage_src_offset_kmajor(wave, lane, j, ldb, rows_b)
-                                      : stage_src_offset(wave, lane, j, ldb, rows_b)) * 2);
-        }
-        // one descriptor per tile: byte offsets inside a tile stay below 2^32 for any operand size
-        if (!kATrans) a_rsrc = mrl::make_rsrc(A + (int64_t)load_tm * BM * lda, 0xffffffffu);
-        if (!kBTrans) b_rsrc = mrl::make_rsrc(B + (int64_t)load_tn * BN * ldb, 0xffffffffu);
-        set_load_stage();
-    };
-    // request i (0..15) of the stage being requested: the wavefront's 8 groups of A, then of B
-    auto issue_one = [&](int buf, int i) {
-        const uint32_t k_bytes = (uint32_t)(load_k * BK * 2);
-        unsigned char* dst = smem + buf * kStageBytes + (wave * kLoadsPerWave) * 1024;
-        if (i < kLoadsPerWave)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (void __attribute__((address_space(3)))*)(dst + i * 1024), 16,
-                                                 a_off[i], kATrans ? 0u : k_bytes, 0, 0);
-        else
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                b_rsrc, (void __attribute__((address_space(3)))*)(dst + kOperandBytes + (i - kLoadsPerWave) * 1024), 16,
-                b_off[i - kLoadsPerWave], kBTrans ? 0u : k_bytes, 0, 0);
-    };
-    // After the last stage of the last tile the requests go on (the schedule below has no branches):
-    // they fetch valid bytes of the last tile into a buffer that nobody reads any more.
-    auto stage_issued = [&]() {
-        if (++load_k == n_ksteps) {
-            load_k = 0;
-            load_tile += tile_stride;
-            if (load_tile < grid.total) set_load_tile(load_tile);
-            else set_load_stage();
-        } else {
-            set_load_stage();
-        }
-    };
-
-    // Fragment addresses.  A lane reads row (lane & 15) of a 16-row block (8 row pairs, 2 KiB), chunk
-    // 4 ks + (lane >> 4) of its 8: inside the block its pair is (lane >> 1) & 7, the pair's low bits
-    // are ((block & 1) << 3) | that, and the physical slot is the logical one XOR those bits.
-    int frag_off[2][2];                                   // [block parity][k sub-step of 32]
-#pragma unroll
-    for (int par = 0; par < 2; ++par)
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            const int pair_in_block = (lane >> 1) & 7;
-            const int slot = ((((lane & 1) ^ par) << 3) | ((4 * ks + (lane >> 4)) ^ pair_in_block));
-            frag_off[par][ks] = pair_in_block * 256 + slot * 16;
-        }
-    // The same for a k-major operand: k-row 32 ks + 8 (lane >> 4) + 4 r + ((lane >> 2) & 3) for the two
-    // reads r = 0, 1 of a fragment, 8 bytes at row 16 block + 4 (lane & 3) of it (column block
-    // block >> 2, segment block & 3 of the k-row); after the transposing read, lane i of each 16 holds
-    // row 16 block + i for 4 consecutive k.
-    int tr_off[4];                                        // [block & 3]
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int g = lane >> 4, kk = (lane >> 2) & 3;
-        tr_off[j] = (8 * g + kk) * 128 + ((j * 32) ^ tr_swizzle(8 * g + kk)) + (lane & 3) * 8;
-    }
-    struct Frags {
-        bf16x8 a[kBlocks], b[kBlocks];
-    };
-    // fragment of 16-row block `blk` (0..15 inside the tile) of an operand whose stage starts at `op`
-    auto read_kcontig = [&](const unsigned char* op, int blk, int ks) {
-        return *reinterpret_cast<const bf16x8*>(op + blk * 2048 + frag_off[blk & 1][ks]);
-    };
-    // The transposing read goes out as inline assembly: through the builtin the compiler cannot tell it
-    // from an access to the bytes that the requests in flight are writing and waits for all of them
-    // (vmcnt(0)) before every read.  The price: it does not wait for the result either - the loop
-    // below does (lgkmcnt(0) before a sub-step consumes fragments read during the one before).
-    const unsigned smem_lds = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
-    auto read_kmajor = [&](const unsigned char* op, int blk, int ks) {
-        typedef long long2v __attribute__((ext_vector_type(2)));
-        const unsigned addr = smem_lds + (unsigned)(op - smem) + (blk >> 2) * 8192 + ks * (32 * 128) + tr_off[blk & 3];
-        long2v both;
-        long lo, hi;
-        asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo) : "v"(addr) : "memory");
-        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:512" : "=v"(hi) : "v"(addr) : "memory");
-        both[0] = lo;
-        both[1] = hi;
-        return __builtin_bit_cast(bf16x8, both);
-    };
-    // read r (0..15) of a fragment set, in the order the MFMAs need them: a0, all of b, a1..a7
-    auto read1 = [&](Frags& f, const unsigned char* stage, int ks, int r) {
-        const bool is_a = r == 0 || r > kBlocks;
-        const int blk = r == 0 ? 0 : (r <= kBlocks ? r - 1 : r - kBlocks);
-        if (is_a)
-            f.a[blk] = kATrans ? read_kmajor(stage, wv * kBlocks + blk, ks) : read_kcontig(stage, wv * kBlocks + blk, ks);
-        else
-            f.b[blk] = kBTrans ? read_kmajor(stage + kOperandBytes, wt * kBlocks + blk, ks)
-                               : read_kcontig(stage + kOperandBytes, wt * kBlocks + blk, ks);
-    };
-    floatx4 acc[kBlocks][kBlocks];
-    auto zero_acc = [&]() {
-#pragma unroll
-        for (int vb = 0; vb < kBlocks; ++vb)
-#pragma unroll
-            for (int tb = 0; tb < kBlocks; ++tb)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[vb][tb][i] = 0.f;
-    };
-    // Empty statements that demand every accumulator in the accumulator half of the register file:
-    // placed after the zeroing and before the store, they keep the allocator from spreading the 64
-    // four-register values over both halves (and copying them around inside the k loop).
-    auto pin_acc = [&]() {
-#pragma unroll
-        for (int vb = 0; vb < kBlocks; ++vb)
-#pragma unroll
-            for (int tb = 0; tb < kBlocks; ++tb) asm volatile("" : "+a"(acc[vb][tb]));
-    };
-    auto mfma1 = [&](const Frags& f, int i) {
-        const int vb = i / kBlocks, tb = i % kBlocks;
-        acc[vb][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.a[vb], f.b[tb], acc[vb][tb], 0, 0, 0);
-    };
     // The finished tile.  A lane holds column n = lane & 15 of each 16 x 16 block and rows
     // 4 (lane >> 4) .. + 3 of it: stored like that, a store instruction would touch 16 output rows with
     // 8 or 16 bytes each.  Each wavefront therefore turns its blocks through a private 8 KiB of LDS:
@@ -282,9 +96,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const uint16_t* __res
     // chunks XOR-swizzled by the row pair, written in the MFMA layout and read back as 8 lanes x 16 bytes
     // per output row, so that every store covers whole 128-byte lines.
     unsigned char* turn = smem + kLdsStages + wave * (kLdsTurn / kWaves);
-    auto store_tile = [&](int64_t t) {
-        int tm, tn;
-        tile_coords(grid, t, tm, tn);
+    auto store_tile = [&](mrl_tile::Accumulators& acc, int tm, int tn) {
         const int row_w = lane & 15, quarter = lane >> 4;        // writer: its n, its run of 4 m inside the block
         const int row_r = lane >> 3, chunk_r = lane & 7;          // reader: n within a group of 8, 16-byte chunk
         constexpr int kMPerPass = kAccumulate ? 2 : 4;            // 32 fp32 or 64 bf16 entries of m are 128 bytes
@@ -343,74 +155,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const uint16_t* __res
         }
     };
 
-    // One wavefront per SIMD: memory instructions are placed between the MFMAs of the same instruction
-    // stream (an MFMA holds the matrix pipe for 16 cycles, other instructions issue meanwhile).  A
-    // stage s (buffer s & 1) is two sub-steps of 64 MFMAs, each on a fragment set that was read during
-    // the sub-step before:
-    //   sub-step 0: MFMAs on G0 | reads G1 (s, k 32..63)  | requests 12..15 of stage s+1
-    //   wait for own requests and reads, barrier: stage s+1 has landed, buffer s & 1 is free
-    //   sub-step 1: MFMAs on G1 | reads G0 (s+1, k 0..31) | requests 0..11 of stage s+2 (into buffer s & 1)
-#define MRL_SB __builtin_amdgcn_sched_barrier(0)
-    constexpr int kMfmas = kBlocks * kBlocks, kReads = 2 * kBlocks, kLoads = 2 * kLoadsPerWave;
-    static_assert(kMfmas == 64 && kReads == 16 && kLoads == 16, "the schedule below is written for these counts");
-    Frags G0, G1;
-    set_load_tile(load_tile);
-#pragma unroll
-    for (int i = 0; i < kLoads; ++i) issue_one(0, i);
-    stage_issued();
-    __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0): stage 0 has landed
-    __syncthreads();
-#pragma unroll
-    for (int r = 0; r < kReads; ++r) read1(G0, smem, 0, r);
-#pragma unroll
-    for (int i = 0; i < 12; ++i) issue_one(1, i);
-    int stage_idx = 0;
-    for (int mine = 0; mine < my_tiles; ++mine) {
-        zero_acc();
-        pin_acc();
-        for (int kstep = 0; kstep < n_ksteps; ++kstep, ++stage_idx) {
-            const int buf = stage_idx & 1;
-            const unsigned char* stage = smem + buf * kStageBytes;
-            const unsigned char* other = smem + (buf ^ 1) * kStageBytes;
-            MRL_SB;
-            if (kATrans || kBTrans) __builtin_amdgcn_s_waitcnt(0xC07F);      // lgkmcnt(0): G0 has arrived
-            MRL_SB;
-#pragma unroll
-            for (int i = 0; i < kMfmas; ++i) {
-                mfma1(G0, i);
-                MRL_SB;
-                if (i % 3 == 0 && i / 3 < kReads) {
-                    read1(G1, stage, 1, i / 3);
-                    MRL_SB;
-                }
-                if (i % 6 == 1 && i / 6 < 4) {
-                    issue_one(buf ^ 1, 12 + i / 6);
-                    MRL_SB;
-                }
-            }
-            stage_issued();
-            __builtin_amdgcn_s_waitcnt(0x0070);        // vmcnt(0) lgkmcnt(0)
-            asm volatile("s_barrier" ::: "memory");
-            MRL_SB;
-#pragma unroll
-            for (int i = 0; i < kMfmas; ++i) {
-                mfma1(G1, i);
-                MRL_SB;
-                if (i % 3 == 0 && i / 3 < kReads) {
-                    read1(G0, other, 0, i / 3);
-                    MRL_SB;
-                }
-                if (i % 5 == 1 && i / 5 < 12) {
-                    issue_one(buf, i / 5);
-                    MRL_SB;
-                }
-            }
-        }
-        pin_acc();
-        store_tile(first_tile + (int64_t)mine * tile_stride);
-    }
-    __builtin_amdgcn_s_waitcnt(0x0F70);                // nothing is in flight into LDS when the workgroup ends
-#undef MRL_SB
+    mfma_tile_loop<kATrans, kBTrans>(smem, A, lda, M, B, ldb, N, K, seq, store_tile);
 }
 
 int persistent_grid() {
