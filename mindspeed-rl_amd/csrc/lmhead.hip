@@ -19,6 +19,7 @@
 
 #include <atomic>
 
+#include "lmhead_tile.h"
 #include "mrl_internal.h"
 #include "vocab_common.h"
 
@@ -201,47 +202,29 @@ __global__ __launch_bounds__(kThreads, (kTB <= 2 ? 2 : 1)) void lmhead_fwd_kerne
 }
 
 // ------------------------------------------------------------------------------------------
-// Second generation of the tile loop: a 512-thread workgroup (2 x 4 wavefronts, one workgroup per
-// CU) owns 256 vocabulary rows x 256 tokens, so each wavefront keeps the 128 x 64 sub-tile of the
-// kernel above but every staged byte feeds twice the MFMA work.  Operands go from global memory
-// straight into LDS (global_load_lds_dwordx4: no staging registers, no ds_write), into one of two
-// stage buffers, so the loads of k-step s+1 run during the MFMAs of k-step s and a k-step costs
-// ONE barrier.  A direct load puts lane i of a wavefront at LDS byte base + 16 i, which rules out
-// padded rows; instead the 16-byte chunks are XOR-swizzled inside each 256-byte pair of rows:
-//   physical slot (0..15) = logical slot ^ (pair index & 15),  logical slot = (row & 1) * 8 + chunk
-// The 16 lanes that a ds_read_b128 serves together read 16 consecutive rows at one chunk, i.e. 8
-// pairs x 2 rows -> 16 different slots -> all 64 banks, no conflict.  The loop runs over the
-// flattened (vocabulary tile, k-step) sequence, so the first loads of the next tile are in flight
-// during the softmax statistics of the current one.
-constexpr int kThreads2 = 512;
-constexpr int BT2 = 256;                         // tokens per workgroup
-constexpr int kOperandBytes = 256 * BK * 2;      // one operand of one stage: 256 rows x 128 bytes
-constexpr int kStageBytes = 2 * kOperandBytes;   // A (weights) then B (hidden)
-constexpr int kLdsBytes2 = 2 * kStageBytes;      // two stages
+// Second generation: the shared tile loop of the lm_head products (lmhead_tile.h: 256 x 256 tiles, one
+// wavefront per SIMD with a 128 x 128 sub-tile on v_mfma_f32_16x16x32_bf16, operands straight into two
+// LDS stages) with the online softmax statistics as what is done with a finished tile.  A workgroup
+// owns 256 tokens and walks the vocabulary tiles of its group; the loop runs over the flattened
+// (vocabulary tile, k-step) sequence, so the first loads of the next tile are in flight during the
+// statistics of the current one.
+struct VocabGroupTiles {
+    int tile_begin, n_tiles, token_tile;
+    __device__ __forceinline__ void coords(int j, int& tm, int& tn) const {
+        tm = tile_begin + j;
+        tn = token_tile;
+    }
+};
 
-// Global element offset (row * hdim + column, without the k-step) of the chunk that lane `lane`
-// of wavefront `wave` brings in with its load j (0..3) of an operand whose tile has `rows_valid`
-// rows left (rows beyond are clamped to the last valid one and masked later).
-__device__ __forceinline__ int stage_src_offset(int wave, int lane, int j, int hdim, int rows_valid) {
-    const int phys_row = (wave * 4 + j) * 8 + (lane >> 3);
-    const int pair = phys_row >> 1;
-    const int slot = ((phys_row & 1) << 3) | (lane & 7);
-    const int logical = slot ^ (pair & 15);
-    int row = 2 * pair + (logical >> 3);
-    if (row >= rows_valid) row = rows_valid - 1;
-    return row * hdim + (logical & 7) * 8;
-}
-
-__global__ __launch_bounds__(kThreads2, 1) void lmhead_fwd_kernel_v2(
+__global__ __launch_bounds__(mrl_tile::kThreads, 1) void lmhead_fwd_kernel_v2(
     const uint16_t* __restrict__ hidden, const uint16_t* __restrict__ weight, int64_t n_tokens, int vocab, int hdim,
     int n_groups, int tiles_per_group, float k_scale, float* __restrict__ partial) {
+    using namespace mrl_tile;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    __shared__ Stats comb[4][2][32];             // [token wavefront][token block][lane % 32]
-    constexpr int kTB = 2;
+    __shared__ Stats comb[2][kBlocks][16];       // [token wavefront][token block][lane % 16]
 
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int wv = wave >> 2, wt = wave & 3;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wv = wave >> 1, wt = wave & 1;
     // Workgroups are dealt round-robin to the 8 XCDs and one round of 256 fills the chip.  The 32
     // workgroups that share an XCD (and its L2) in a round are 4 token tiles x 8 vocabulary groups:
     // the 8 that stream the same hidden block and the 4 that stream the same weight tiles run side
@@ -250,191 +233,74 @@ __global__ __launch_bounds__(kThreads2, 1) void lmhead_fwd_kernel_v2(
     const int xcd = blockIdx.x & 7, slot = (blockIdx.x >> 3) & 31, round = blockIdx.x >> 8;
     const int group = slot & 7;
     const int64_t ttile = (int64_t)(round * 8 + xcd) * 4 + (slot >> 3);
-    const int64_t t0 = ttile * BT2;
+    const int64_t t0 = ttile * BN;
     if (t0 >= n_tokens) return;                 // padding of the last round
-    const int n_vtiles = (vocab + BV - 1) / BV;
-    const int tile_begin = group * tiles_per_group;
-    const int tile_end = min(tile_begin + tiles_per_group, n_vtiles);
-    const int n_ksteps = hdim / BK;
+    const int n_vtiles = (vocab + BM - 1) / BM;
+    VocabGroupTiles seq;
+    seq.tile_begin = group * tiles_per_group;
+    seq.n_tiles = max(0, min(seq.tile_begin + tiles_per_group, n_vtiles) - seq.tile_begin);
+    seq.token_tile = (int)ttile;
 
-    // sources of this lane's four chunks per operand and stage
-    const uint16_t* b_base = hidden + t0 * hdim;
-    const int tokens_valid = (int)min((int64_t)BT2, n_tokens - t0);
-    int b_off[4], a_off[4];
+    // a lane holds one token of each of its wavefront's 8 token blocks
+    Stats st[kBlocks];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) b_off[j] = stage_src_offset(wave, lane, j, hdim, tokens_valid);
+    for (int tb = 0; tb < kBlocks; ++tb) st[tb] = {kMaxInit, 0.f, 0.f};
 
-    // Buffer (MUBUF) form of the LDS load on purpose: the global_load_lds form is a FLAT instruction
-    // that touches two address spaces, and while one is pending the compiler turns every LDS wait
-    // into lgkmcnt(0), which would undo the fragment pipeline below.
-    const mrl::rsrc_t w_rsrc = mrl::make_rsrc(weight, 0xffffffffu);
-    const mrl::rsrc_t h_rsrc = mrl::make_rsrc(b_base, 0xffffffffu);
-    auto issue = [&](int tile, int kstep, int buf) {
-        const uint32_t a_tile = (uint32_t)(((int64_t)tile * BV * hdim + kstep * BK) * 2);
-        const uint32_t b_tile = (uint32_t)(kstep * BK * 2);
-        unsigned char* dst = smem + buf * kStageBytes + (wave * 4) * 1024;
+    // online softmax statistics of a tile: per token block a lane holds 8 x 4 vocabulary rows
+    auto tile_stats = [&](Accumulators& acc, int tm, int /*tn*/) {
+        const int v0 = tm * BM + wv * 128 + 4 * (lane >> 4);       // + 16 vb + r
+        const bool ragged = (tm * BM + BM > vocab);
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (void __attribute__((address_space(3)))*)(dst + j * 1024), 16,
-                                                 a_off[j] * 2, a_tile, 0, 0);
+        for (int tb = 0; tb < kBlocks; ++tb) {
+            if (ragged) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(h_rsrc,
-                                                 (void __attribute__((address_space(3)))*)(dst + kOperandBytes + j * 1024),
-                                                 16, b_off[j] * 2, b_tile, 0, 0);
-    };
-    auto set_a_rows = [&](int tile) {
-        const int rows_valid = min(BV, vocab - tile * BV);
+                for (int vb = 0; vb < kBlocks; ++vb)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) a_off[j] = stage_src_offset(wave, lane, j, hdim, rows_valid);
-    };
-
-    // fragment addresses: row (lane & 31) of a 32-row block, chunk 2 ks + (lane >> 5)
-    const int frag_pair = (lane & 31) >> 1;
-    const int frag_slot = (((lane & 1) << 3) | (lane >> 5)) ^ frag_pair;          // ^ (2 ks) per k sub-step
-    const int a_frag = (wv * 64) * 256 + frag_pair * 256;                          // + vb * 16 * 256
-    const int b_frag = kOperandBytes + (wt * 32) * 256 + frag_pair * 256;          // + tb * 16 * 256
-
-    Stats st[kTB];
-#pragma unroll
-    for (int tb = 0; tb < kTB; ++tb) st[tb] = {kMaxInit, 0.f, 0.f};
-
-    // The (tile, k-step) stages are numbered 0 .. n_stages-1; stage s lives in buffer s & 1.
-    const int n_stages = (tile_end > tile_begin ? tile_end - tile_begin : 0) * n_ksteps;
-    int next_tile = tile_begin, next_k = 0;      // the stage that is requested next
-    auto issue_next = [&](int buf) {
-        if (next_k == 0) set_a_rows(next_tile);
-        issue(next_tile, next_k, buf);
-        if (++next_k == n_ksteps) {
-            next_k = 0;
-            ++next_tile;
-        }
-    };
-    struct Frags {
-        bf16x8 a[4], b[kTB];
-    };
-    auto read_frags = [&](Frags& f, const unsigned char* stage, int ks) {
-        const int slot_bytes = (frag_slot ^ (2 * ks)) * 16;
-#pragma unroll
-        for (int vb = 0; vb < 4; ++vb)
-            f.a[vb] = *reinterpret_cast<const bf16x8*>(stage + a_frag + vb * 16 * 256 + slot_bytes);
-#pragma unroll
-        for (int tb = 0; tb < kTB; ++tb)
-            f.b[tb] = *reinterpret_cast<const bf16x8*>(stage + b_frag + tb * 16 * 256 + slot_bytes);
-    };
-    floatx16 acc[4][kTB];
-    auto zero_acc = [&]() {
-#pragma unroll
-        for (int vb = 0; vb < 4; ++vb)
-#pragma unroll
-            for (int tb = 0; tb < kTB; ++tb)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) acc[vb][tb][i] = 0.f;
-    };
-    auto mma = [&](const Frags& f) {
-#pragma unroll
-        for (int vb = 0; vb < 4; ++vb)
-#pragma unroll
-            for (int tb = 0; tb < kTB; ++tb)
-                acc[vb][tb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[vb], f.b[tb], acc[vb][tb], 0, 0, 0);
-    };
-
-    if (n_stages > 0) {
-        Frags f0, f1;
-        issue_next(0);
-        __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0): stage 0 has landed
-        __syncthreads();
-        if (n_stages > 1) issue_next(1);
-        read_frags(f0, smem, 0);
-        zero_acc();
-        int tile = tile_begin, kstep = 0;
-        for (int stage_idx = 0; stage_idx < n_stages; ++stage_idx) {
-            const int buf = stage_idx & 1;
-            const unsigned char* stage = smem + buf * kStageBytes;
-            // software pipeline: the fragments of sub-step ks+1 are requested before the MFMAs of ks
-            read_frags(f1, stage, 1);
-            __builtin_amdgcn_sched_barrier(0);
-            mma(f0);
-            __builtin_amdgcn_sched_barrier(0);
-            read_frags(f0, stage, 2);
-            __builtin_amdgcn_sched_barrier(0);
-            mma(f1);
-            __builtin_amdgcn_sched_barrier(0);
-            read_frags(f1, stage, 3);
-            __builtin_amdgcn_sched_barrier(0);
-            mma(f0);
-            __builtin_amdgcn_sched_barrier(0);
-            // The last fragments of this stage are in registers and the next stage has landed: after
-            // the barrier this buffer may be overwritten, and the first fragments of the next stage are
-            // requested before the last MFMAs of this one are issued.  The barrier and the read are
-            // unconditional (after the last stage the read fetches unused bytes of the other buffer): a
-            // branch around them would make the wait before the MFMAs cover the new request as well.
-            __builtin_amdgcn_s_waitcnt(0x0070);            // vmcnt(0) lgkmcnt(0)
-            __syncthreads();
-            read_frags(f0, smem + (buf ^ 1) * kStageBytes, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            mma(f1);
-            __builtin_amdgcn_sched_barrier(0);
-            // the stage after next goes into the buffer that the barrier has just freed; requested
-            // after the MFMAs so that its address arithmetic does not hold them up (measured: 6 % faster
-            // than right after the barrier; spreading the requests over the next stage was slower)
-            if (stage_idx + 2 < n_stages) issue_next(buf);
-            __builtin_amdgcn_sched_barrier(0);
-            if (++kstep == n_ksteps) {
-                // online softmax statistics of this tile: a lane holds 64 vocabulary rows of each token column
-                const int v0 = tile * BV;
-                const bool ragged = (v0 + BV > vocab);
-#pragma unroll
-                for (int tb = 0; tb < kTB; ++tb) {
-                    if (ragged) {
-#pragma unroll
-                        for (int vb = 0; vb < 4; ++vb)
-#pragma unroll
-                            for (int i = 0; i < 16; ++i) {
-                                const int v = v0 + wv * 128 + vb * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
-                                if (v >= vocab) acc[vb][tb][i] = kMaxInit;
-                            }
-                    }
-                    float vmax = st[tb].m;
-#pragma unroll
-                    for (int vb = 0; vb < 4; ++vb)
-#pragma unroll
-                        for (int i = 0; i < 16; ++i) vmax = fmaxf(vmax, acc[vb][tb][i]);
-                    grow_max<true>(st[tb], vmax, k_scale);
-                    // no valid vocabulary row seen yet by this lane: see the first-generation kernel
-                    const float mk = st[tb].m > kMaxInit ? st[tb].m * k_scale : __builtin_inff();
-#pragma unroll
-                    for (int vb = 0; vb < 4; ++vb)
-#pragma unroll
-                        for (int i = 0; i < 16; ++i) add_one<true>(st[tb], acc[vb][tb][i], k_scale, mk);
-                }
-                zero_acc();
-                kstep = 0;
-                ++tile;
+                    for (int r = 0; r < 4; ++r)
+                        if (v0 + 16 * vb + r >= vocab) acc[vb][tb][r] = kMaxInit;
             }
+            float vmax = st[tb].m;
+#pragma unroll
+            for (int vb = 0; vb < kBlocks; ++vb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) vmax = fmaxf(vmax, acc[vb][tb][r]);
+            grow_max<true>(st[tb], vmax, k_scale);
+            // A lane that has seen no valid vocabulary row yet (the first tile of its group is ragged and
+            // ends above its rows) still holds the start value as its maximum: z * k - m * k of the masked
+            // entries would then be the rounding residual of two numbers of magnitude 1e30 instead of
+            // zero.  With an infinite m * k their exponentials are exactly 0.
+            const float mk = st[tb].m > kMaxInit ? st[tb].m * k_scale : __builtin_inff();
+#pragma unroll
+            for (int vb = 0; vb < kBlocks; ++vb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) add_one<true>(st[tb], acc[vb][tb][r], k_scale, mk);
+        }
+    };
+    mfma_tile_loop<false, false>(smem, weight, hdim, vocab, hidden, hdim, (int)n_tokens, hdim, seq, tile_stats);
+
+    // combine the four lane quarters (same token, other vocabulary rows), then the two vocabulary wavefronts
+#pragma unroll
+    for (int tb = 0; tb < kBlocks; ++tb) {
+#pragma unroll
+        for (int off = 16; off <= 32; off <<= 1) {
+            Stats o;
+            o.m = __shfl_xor(st[tb].m, off, 64);
+            o.s = __shfl_xor(st[tb].s, off, 64);
+            o.u = __shfl_xor(st[tb].u, off, 64);
+            st[tb] = merge<true>(st[tb], o, k_scale);
         }
     }
-
-    // combine the two lane halves (same token, other vocabulary rows), then the two vocabulary wavefronts
+    __syncthreads();
+    if (wv == 1 && lane < 16) {
 #pragma unroll
-    for (int tb = 0; tb < kTB; ++tb) {
-        Stats o;
-        o.m = __shfl_xor(st[tb].m, 32, 64);
-        o.s = __shfl_xor(st[tb].s, 32, 64);
-        o.u = __shfl_xor(st[tb].u, 32, 64);
-        st[tb] = merge<true>(st[tb], o, k_scale);
+        for (int tb = 0; tb < kBlocks; ++tb) comb[wt][tb][lane] = st[tb];
     }
     __syncthreads();
-    if (wv == 1 && lane < 32) {
+    if (wv == 0 && lane < 16) {
 #pragma unroll
-        for (int tb = 0; tb < kTB; ++tb) comb[wt][tb][lane] = st[tb];
-    }
-    __syncthreads();
-    if (wv == 0 && lane < 32) {
-#pragma unroll
-        for (int tb = 0; tb < kTB; ++tb) {
+        for (int tb = 0; tb < kBlocks; ++tb) {
             const Stats r = merge<true>(st[tb], comb[wt][tb][lane], k_scale);
-            const int64_t t = t0 + wt * 64 + tb * 32 + lane;
+            const int64_t t = t0 + wt * 128 + tb * 16 + lane;
             if (t < n_tokens) {
                 float* p = partial + ((int64_t)group * n_tokens + t) * 4;
                 p[0] = r.m;
@@ -514,14 +380,16 @@ static int lmhead_forward(const char* fn, const void* hidden, const void* weight
     const int n_vtiles = (int)((vocab + BV - 1) / BV);
     const int tiles_per_group = (n_vtiles + n_groups - 1) / n_groups;
     // a group without tiles (tiny vocabularies) still writes its neutral partials
-    // the second-generation loop addresses the weights with 32-bit byte offsets
-    if (lmhead_v2_enabled() && vocab * hidden_dim * 2 < (1LL << 32)) {
+    if (lmhead_v2_enabled()) {
         // 256-token tiles, operands straight into two LDS stages (128 KiB of dynamic LDS)
+        constexpr int kLdsBytes2 = mrl_tile::kLdsStages, kThreads2 = mrl_tile::kThreads;
         static const hipError_t attr = hipFuncSetAttribute((const void*)lmhead_fwd_kernel_v2,
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes2);
         MRL_REQUIRE(attr == hipSuccess, MRL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", fn, kLdsBytes2,
                     hipGetErrorString(attr));
-        const int64_t n_ttiles = (n_tokens + BT2 - 1) / BT2;
+        MRL_REQUIRE(256 * hidden_dim * 2 < (1LL << 31) && n_tokens <= 0x7fffffffLL, MRL_ERR_UNSUPPORTED,
+                    "%s: size out of range", fn);
+        const int64_t n_ttiles = (n_tokens + mrl_tile::BN - 1) / mrl_tile::BN;
         const int64_t n_rounds = (n_ttiles + 31) / 32;       // 32 token tiles x 8 groups per round of 256 workgroups
         MRL_REQUIRE(n_rounds * 256 <= 0x7fffffffLL, MRL_ERR_UNSUPPORTED, "%s: grid too large", fn);
         static_assert(MRL_LMHEAD_GROUPS == 8, "the workgroup mapping assumes 8 vocabulary groups");
