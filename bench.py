@@ -50,7 +50,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS) + ["c3fwd", "c3"],
                     help="c3fwd: the fused lm_head + log-prob forward of configs[3] (bf16 MFMA, logits never stored); "
-                         "c3: configs[3] forward + backward from the hidden states (chunked GEMM -> fused sweep -> GEMMs)")
+                         "c3: configs[3] forward + backward from the hidden states (per chunk: logits product -> fused sweep -> dHidden and dW products)")
     ap.add_argument("--tokens", type=int, default=163840, help="rows of the c3fwd workload")
     ap.add_argument("--entropy-coeff", type=float, default=0.001,
                     help="non-zero so that the forward computes entropy and the backward its gradient")
@@ -374,7 +374,7 @@ def run_lmhead_train(args):
                                "%d rows at a time" % (total, args.chunk_rows), "response_tokens": tokens, "accumulate": "f32",
                    "products": "hand-written gfx950 MFMA kernels (gemm_nt_kernel: logits, dHidden, dW)",
                    "sweep": "fused_sweep_persistent_kernel in place"},
-        "roofline": {"kernel": "whole step (3 matrix products per chunk + fused sweeps + transposed copies)",
+        "roofline": {"kernel": "whole step (gemm_kernel x 3 per chunk + fused_sweep_persistent_kernel)",
                      "bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "flops_per_step": flops,
                      "fused_sweeps_ms_per_step": sweep_ms, "logits_products_ms_per_step": logits_ms,
