@@ -372,7 +372,7 @@ def run_lmhead_train(args):
         "data": "synthetic",
         "config": {"workload": "configs[3]: hidden [%d,3584] x W [152064,3584], GRPO loss as configs[1], logits only for "
                                "%d rows at a time" % (total, args.chunk_rows), "response_tokens": tokens, "accumulate": "f32",
-                   "products": "hand-written gfx950 MFMA kernels (gemm_nt_kernel: logits, dHidden, dW)",
+                   "products": "hand-written gfx950 MFMA kernels (gemm_kernel: logits, dHidden, dW)",
                    "sweep": "fused_sweep_persistent_kernel in place"},
         "roofline": {"kernel": "whole step (gemm_kernel x 3 per chunk + fused_sweep_persistent_kernel)",
                      "bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
