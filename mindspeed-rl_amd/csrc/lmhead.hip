@@ -276,7 +276,7 @@ __global__ __launch_bounds__(mrl_tile::kThreads, 1) void lmhead_fwd_kernel_v2(
                 for (int r = 0; r < 4; ++r) add_one<true>(st[tb], acc[vb][tb][r], k_scale, mk);
         }
     };
-    mfma_tile_loop<false, false>(smem, weight, hdim, vocab, hidden, hdim, (int)n_tokens, hdim, seq, tile_stats);
+    mfma_tile_loop<false, false, 4>(smem, weight, hdim, vocab, hidden, hdim, (int)n_tokens, hdim, seq, tile_stats);
 
     // combine the four lane quarters (same token, other vocabulary rows), then the two vocabulary wavefronts
 #pragma unroll

@@ -155,7 +155,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const uint16_t* __res
         }
     };
 
-    mfma_tile_loop<kATrans, kBTrans>(smem, A, lda, M, B, ldb, N, K, seq, store_tile);
+    mfma_tile_loop<kATrans, kBTrans, 0>(smem, A, lda, M, B, ldb, N, K, seq, store_tile);
 }
 
 int persistent_grid() {

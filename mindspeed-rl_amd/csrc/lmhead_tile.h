@@ -80,8 +80,9 @@ typedef floatx4 Accumulators[kBlocks][kBlocks];
 // wt * 128 .. + 127 of B (n); acc[vb][tb] is the 16 x 16 block at m = 16 vb, n = 16 tb of it, of which a
 // lane holds column n = lane & 15 and rows m = 4 (lane >> 4) .. + 3.  Rows of a ragged last tile beyond
 // M or N hold products of clamped operand rows: the epilogue must skip them.  K % 64 == 0 unless an
-// operand is k-major.  Every thread of the workgroup must call this (it contains barriers).
-template <bool kATrans, bool kBTrans, typename Seq, typename Epilogue>
+// operand is k-major.  kEarly (0..4): how many of a stage's 16 requests go out early, see the schedule
+// below.  Every thread of the workgroup must call this (it contains barriers).
+template <bool kATrans, bool kBTrans, int kEarly, typename Seq, typename Epilogue>
 __device__ __forceinline__ void mfma_tile_loop(unsigned char* smem, const uint16_t* __restrict__ A, int64_t lda, int M,
                                                const uint16_t* __restrict__ B, int64_t ldb, int N, int K, const Seq& seq,
                                                Epilogue&& epilogue) {
@@ -115,11 +116,11 @@ __device__ __forceinline__ void mfma_tile_loop(unsigned char* smem, const uint16
         seq.coords(j, load_tm, load_tn);
         const int rows_a = min(BM, M - load_tm * BM), rows_b = min(BN, N - load_tn * BN);
 #pragma unroll
-        for (int j = 0; j < kLoadsPerWave; ++j) {
-            a_off[j] = (int)((kATrans ? stage_src_offset_kmajor(wave, lane, j, lda, rows_a)
-                                      : stage_src_offset(wave, lane, j, lda, rows_a)) * 2);
-            b_off[j] = (int)((kBTrans ? stage_src_offset_kmajor(wave, lane, j, ldb, rows_b)
-                                      : stage_src_offset(wave, lane, j, ldb, rows_b)) * 2);
+        for (int i = 0; i < kLoadsPerWave; ++i) {
+            a_off[i] = (int)((kATrans ? stage_src_offset_kmajor(wave, lane, i, lda, rows_a)
+                                      : stage_src_offset(wave, lane, i, lda, rows_a)) * 2);
+            b_off[i] = (int)((kBTrans ? stage_src_offset_kmajor(wave, lane, i, ldb, rows_b)
+                                      : stage_src_offset(wave, lane, i, ldb, rows_b)) * 2);
         }
         // one descriptor per tile: byte offsets inside a tile stay below 2^32 for any operand size
         if (!kATrans) a_rsrc = mrl::make_rsrc(A + (int64_t)load_tm * BM * lda, 0xffffffffu);
@@ -232,15 +233,21 @@ __device__ __forceinline__ void mfma_tile_loop(unsigned char* smem, const uint16
     // stream (an MFMA holds the matrix pipe for 16 cycles, other instructions issue meanwhile).  A
     // stage s (buffer s & 1) is two sub-steps of 64 MFMAs, each on a fragment set that was read during
     // the sub-step before:
-    //   sub-step 0: MFMAs on G0 | reads G1 (s, k 32..63)
+    //   sub-step 0: MFMAs on G0 | reads G1 (s, k 32..63)  | the last kEarly requests of stage s+1
     //   wait for own requests and reads, barrier: stage s+1 has landed, buffer s & 1 is free
-    //   sub-step 1: MFMAs on G1 | reads G0 (s+1, k 0..31) | the 16 requests of stage s+2 (into buffer s & 1)
-    // The requests go out one every 4 MFMAs, all of them in sub-step 1: each then has a whole sub-step
-    // (1 us) before the barrier that needs it.  Measured on the logits product: 4 of them moved into
-    // sub-step 0 cost 4 %, 8 cost 11 %; two or three times as dense right after the barrier 1 - 7 %.
+    //   sub-step 1: MFMAs on G1 | reads G0 (s+1, k 0..31) | the first 16 - kEarly requests of stage s+2
+    //                                                        (into buffer s & 1)
+    // How the 16 requests of a stage are best placed depends on the caller's tile order, measured at
+    // 32 768 x 152 064 x 3584: the plain products (panels of tiles) want all of them in sub-step 1, one
+    // every 4 MFMAs, so that each has a whole sub-step (1 us) before the barrier that needs it (4 of them
+    // in sub-step 0: -4 %, 8: -11 %; twice or three times as dense right after the barrier: -1 .. -7 %);
+    // the fused forward (a workgroup walks the vocabulary with one block of tokens) wants 4 of them in
+    // sub-step 0 (0: -15 %, 2: -3 %, 8: -9 %).
 #define MRL_SB __builtin_amdgcn_sched_barrier(0)
     constexpr int kMfmas = kBlocks * kBlocks, kReads = 2 * kBlocks, kLoads = 2 * kLoadsPerWave;
     static_assert(kMfmas == 64 && kReads == 16 && kLoads == 16, "the schedule below is written for these counts");
+    static_assert(kEarly >= 0 && kEarly <= 4, "at most 4 early requests");
+    constexpr int kLate = kLoads - kEarly, kLateEvery = kEarly == 0 ? 4 : 5;
     Frags G0, G1;
     set_load_tile(0);
 #pragma unroll
@@ -251,8 +258,8 @@ __device__ __forceinline__ void mfma_tile_loop(unsigned char* smem, const uint16
 #pragma unroll
     for (int r = 0; r < kReads; ++r) read1(G0, smem, 0, r);
 #pragma unroll
-    for (int i = 0; i < kLoads; ++i) issue_one(1, i);
-    stage_issued();
+    for (int i = 0; i < kLate; ++i) issue_one(1, i);
+    if (kEarly == 0) stage_issued();
     int stage_idx = 0;
     for (int mine = 0; mine < n_tiles; ++mine) {
         zero_acc();
@@ -272,7 +279,12 @@ __device__ __forceinline__ void mfma_tile_loop(unsigned char* smem, const uint16
                     read1(G1, stage, 1, i / 3);
                     MRL_SB;
                 }
+                if (kEarly > 0 && i % 6 == 1 && i / 6 < kEarly) {
+                    issue_one(buf ^ 1, kLate + i / 6);
+                    MRL_SB;
+                }
             }
+            if (kEarly > 0) stage_issued();
             __builtin_amdgcn_s_waitcnt(0x0070);        // vmcnt(0) lgkmcnt(0)
             asm volatile("s_barrier" ::: "memory");
             MRL_SB;
@@ -284,12 +296,12 @@ __device__ __forceinline__ void mfma_tile_loop(unsigned char* smem, const uint16
                     read1(G0, other, 0, i / 3);
                     MRL_SB;
                 }
-                if (i % 4 == 3) {
-                    issue_one(buf, i / 4);
+                if (i % kLateEvery == kLateEvery - (kEarly == 0 ? 1 : 4) && i / kLateEvery < kLate) {
+                    issue_one(buf, i / kLateEvery);
                     MRL_SB;
                 }
             }
-            stage_issued();
+            if (kEarly == 0) stage_issued();
         }
         pin_acc();
         int tm, tn;
