@@ -7,6 +7,7 @@ The observed errors are far smaller; tighter bounds are asserted where the arith
 """
 import math
 import os
+import random
 
 import numpy as np
 import pytest
@@ -1466,6 +1467,44 @@ def test_lmhead_products_through_the_c_abi(dev, tokens, vocab, hdim):
     assert lib.mrl_lmhead_logprob_bwd(hd.data_ptr(), wd.data_ptr(), dzd.data_ptr(), v_pad - 8, tokens, vocab, hdim,
                                       dh.data_ptr(), dw.data_ptr(), stream) == -1
     assert b"dlogits_row_stride" in lib.mrl_last_error()
+
+
+def test_lmhead_products_random_shapes(dev):
+    """40 seeded shapes of the three lm_head products (tokens 1 .. 2500, vocabularies that are multiples of 8
+    up to 3000, hidden sizes that are multiples of 64 up to 768: ragged tiles along every dimension, k-steps
+    that end inside a tile, single-tile and many-tile grids) against fp32 products on the device; memory
+    behind every operand holds NaN."""
+    rnd = random.Random(20251)
+    lib = _lib.load()
+    stream = _lib.stream(dev)
+    for case in range(40):
+        tokens = rnd.choice([1, 7, 63, 64, 65, 255, 256, 257, 511, 1000, rnd.randint(1, 2500)])
+        vocab = 8 * rnd.choice([1, 7, 8, 9, 31, 32, 33, 100, rnd.randint(1, 375)])
+        hdim = 64 * rnd.choice([1, 2, 3, 4, 7, 12])
+        g = torch.Generator(device=dev).manual_seed(case)
+        v_pad = (vocab + 63) // 64 * 64
+        hbuf = torch.full((tokens + 64, hdim), float("nan"), dtype=torch.bfloat16, device=dev)
+        wbuf = torch.full((vocab + 64, hdim), float("nan"), dtype=torch.bfloat16, device=dev)
+        dzbuf = torch.full((tokens + 64, v_pad), float("nan"), dtype=torch.bfloat16, device=dev)
+        hbuf[:tokens] = torch.randn(tokens, hdim, generator=g, device=dev).to(torch.bfloat16)
+        wbuf[:vocab] = (torch.randn(vocab, hdim, generator=g, device=dev) * (2.0 / hdim ** 0.5)).to(torch.bfloat16)
+        dzbuf[:tokens] = 0
+        dzbuf[:tokens, :vocab] = (torch.randn(tokens, vocab, generator=g, device=dev) * 0.01).to(torch.bfloat16)
+        h, w, dz = hbuf[:tokens], wbuf[:vocab], dzbuf[:tokens]
+        what = "case %d: tokens=%d vocab=%d hidden=%d" % (case, tokens, vocab, hdim)
+        z = torch.full((tokens, v_pad), 7.0, dtype=torch.bfloat16, device=dev)
+        _lib.call("mrl_lmhead_logits", h.data_ptr(), w.data_ptr(), tokens, vocab, hdim, z.data_ptr(), v_pad, stream)
+        want = h.float() @ w.float().t()
+        assert (z[:, :vocab].float() - want).abs().max().item() <= 2 ** -8 * want.abs().max().item() + 1e-6, what
+        assert (z[:, vocab:] == 7.0).all().item(), what
+        dh = torch.full((tokens, hdim), 5.0, dtype=torch.bfloat16, device=dev)
+        dw = torch.ones(vocab, hdim, dtype=torch.float32, device=dev)
+        _lib.call("mrl_lmhead_logprob_bwd", h.data_ptr(), w.data_ptr(), dz.data_ptr(), v_pad, tokens, vocab, hdim,
+                  dh.data_ptr(), dw.data_ptr(), stream)
+        want_dh = dz[:, :vocab].float() @ w.float()
+        want_dw = 1.0 + dz[:, :vocab].float().t() @ h.float()
+        assert (dh.float() - want_dh).abs().max().item() <= 2 ** -7 * want_dh.abs().max().item() + 1e-9, what
+        assert (dw - want_dw).abs().max().item() <= 1e-5 * (want_dw - 1.0).abs().max().item() + 1e-7, what
 
 
 def test_copy_kernel_moves_bytes(dev):
