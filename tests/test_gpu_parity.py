@@ -1785,8 +1785,8 @@ def test_full_size_lmhead_forward(dev):
 
 def test_full_size_lmhead_training_step(dev):
     """configs[3]'s training step at its full size (128 sequences, ~164 k tokens, H = 3584, V = 152 064):
-    the step with two different chunkings (32 768 rows, and 20 000 rows, which is no multiple of a tile)
-    gives the same loss and the same dHidden bit for bit and the same dWeight up to how fp32 sums group;
+    the step run twice gives bit-identical results; with two different chunkings (32 768 rows, and 20 000
+    rows, which is no multiple of a tile) it gives the same loss and the same dHidden bit for bit and the same dWeight up to how fp32 sums group;
     <dWeight, W> = <dHidden, hidden> (both equal sum dlogits * logits: an identity between the two
     backward products that needs no dlogits); and the rows of one whole sequence against the oracle's
     loss gradient (CPU, fed the device's bf16 logits of those rows, scaled by its share of the tokens)
@@ -1832,6 +1832,10 @@ def test_full_size_lmhead_training_step(dev):
         return loss.item(), out.cpu(), dh[0], dw
 
     l1, o1, dh1, dw1 = step(32768)
+    l1b, o1b, dh1b, dw1b = step(32768)
+    # nothing in the step depends on timing: no atomics, dWeight accumulated in stream order
+    assert l1b == l1 and torch.equal(o1b, o1) and torch.equal(dh1b, dh1) and torch.equal(dw1b, dw1)
+    del dh1b, dw1b
     l2, o2, dh2, dw2 = step(20000)
     assert l1 == l2 and torch.equal(o1, o2)
     assert torch.equal(dh1, dh2)
