@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define MRL_VERSION 201
+#define MRL_VERSION 300
 
 enum mrl_status {
     MRL_OK = 0,
@@ -271,7 +271,8 @@ int mrl_policy_loss_bwd(const float* log_prob, const float* old_log_prob,
  * (grpo_actor_loss_func.py:127-144, dapo_actor_loss_func.py:129-152) and all their backwards.
  *
  * Call order: mrl_fused_loss_prepare -> mrl_fused_logprob_loss -> mrl_fused_loss_reduce, and
- * mrl_scale_rows when autograd later delivers an upstream gradient.
+ * mrl_scale_rows_note when autograd later delivers an upstream gradient: four launches for the
+ * forward and backward of the whole path when the mask is given by the response lengths.
  */
 
 /* Largest vocabulary the row-in-registers kernels hold for a logits dtype (0 = bad dtype): one
@@ -281,8 +282,9 @@ int mrl_policy_loss_bwd(const float* log_prob, const float* old_log_prob,
 int64_t mrl_fused_max_vocab(int logits_dtype);
 
 /* Bytes of workspace mrl_fused_logprob_loss wants for this shape (16-byte aligned device memory):
- * 16 for rows that one workgroup holds (the row counter), 16 + 32 * n_rows for wider rows (plus one
- * 16-byte record per half row); 0 if the fused sweep does not take the shape at all. */
+ * 16 for rows that one workgroup holds (the row counter of the persistent workgroups), 16 + 32 *
+ * n_rows for wider rows (plus one 16-byte record per half row); 0 if the fused sweep does not take
+ * the shape at all. */
 int64_t mrl_fused_workspace_bytes(int logits_dtype, int64_t n_rows, int64_t vocab);
 
 /* Step 1.  Maps the [batch, width] loss operands onto logits rows.
@@ -295,7 +297,14 @@ int64_t mrl_fused_workspace_bytes(int logits_dtype, int64_t n_rows, int64_t voca
  * Outputs: row_start int64 [batch], row_count int32 [batch], seq_mask_sum float [batch] (sum of
  * each mask row), row_ops float [n_rows * 8] = {old, ref, adv, mask, w_pg, 1/(N+1e-8), 0, 0} per
  * logits row, mask = 0 for rows outside every window; N = sum of the whole mask; w_pg is
- * 1/(N+1e-8) (seq_mean 0) or 1/(batch * seq_mask_sum[i]) (seq_mean 1).  prompt_length >= 1. */
+ * 1/(N+1e-8) (seq_mean 0) or 1/(batch * seq_mask_sum[i]) (seq_mean 1).  prompt_length >= 1.
+ * The same launch prepares the sweep that follows on `stream`: sweep_workspace (nullable, a multiple
+ * of 8 bytes) is zeroed, which is what mrl_fused_logprob_loss asks of a workspace handed to it as
+ * `workspace_cleared`, and scale_out (nullable, two floats, 8-byte aligned) receives
+ * {scale_host * *scale_in, 0}: the scale the sweep is to write into its gradients (scale_in, a
+ * nullable DEVICE scalar, NULL = 1: what mrl_scale_rows_note learned at the previous backward) next
+ * to the zeroed counter that mrl_scale_rows_note keeps there.  With the mask given by the response
+ * lengths (mask NULL) and at most 2048 sequences all of this is ONE launch. */
 int mrl_fused_loss_prepare(int layout, int64_t batch, int64_t width, int64_t n_rows,
                            const int32_t* seqlens, const int32_t* cu_seqlens_padded,
                            int64_t padded_seq_len, const void* prompt_length, int prompt_dtype,
@@ -303,7 +312,8 @@ int mrl_fused_loss_prepare(int layout, int64_t batch, int64_t width, int64_t n_r
                            const float* old_log_prob, const float* ref_log_prob,
                            const float* advantages, const void* mask, int mask_dtype, int seq_mean,
                            int64_t* row_start, int32_t* row_count, float* seq_mask_sum,
-                           float* row_ops, void* stream);
+                           float* row_ops, void* sweep_workspace, int64_t sweep_workspace_bytes,
+                           const float* scale_in, float scale_host, float* scale_out, void* stream);
 
 /* Step 2.  The sweep.  Per row with a non-zero mask: logp, entropy (if `entropy` is given) as in
  * mrl_vocab_logprob_fwd; the token's loss terms as in mrl_policy_loss_fwd; then
@@ -318,26 +328,40 @@ int mrl_fused_loss_prepare(int layout, int64_t batch, int64_t width, int64_t n_r
  * has_old = 0 means old_log_prob = log_prob.detach() (ratio 1).  workspace:
  * mrl_fused_workspace_bytes(dtype, n_rows, vocab) bytes of device memory owned by the caller: the
  * counter from which the persistent workgroups take their next row and, for rows wider than one
- * workgroup holds, the records through which the two halves of a row exchange their statistics
- * (both reset by this call on `stream`; a workspace must not be shared by sweeps that can be in
- * flight at the same time, and a captured graph keeps using the address it was captured with).
- * NULL is allowed for rows that one workgroup holds: they are then walked with a fixed stride,
- * about a twentieth slower on large batches.  Needs 16-byte aligned rows, vocab % (16/elem) == 0 and
- * vocab <= mrl_fused_max_vocab(dtype), and wide rows (above half of that) cannot be swept in place;
- * else MRL_ERR_UNSUPPORTED (use the split fwd/bwd entry points then).  The wait of a workgroup for
- * the other half of its row is bounded: past the bound it computes that half's statistics itself
- * from memory. */
+ * workgroup holds, the records through which the two halves of a row exchange their statistics.
+ * Both must be zero when the sweep starts: with workspace_cleared != 0 the caller vouches for that
+ * (mrl_fused_loss_prepare clears it in passing), else this call clears it on `stream` first.  A
+ * workspace must not be shared by sweeps that can be in flight at the same time, and a captured
+ * graph keeps using the address it was captured with.  NULL is allowed for rows that one workgroup
+ * holds: every row then gets a workgroup of its own, which costs large batches about a quarter more
+ * time.  Needs 16-byte aligned rows, vocab % (16/elem) == 0 and
+ * vocab <= mrl_fused_max_vocab(dtype); else MRL_ERR_UNSUPPORTED (use the split fwd/bwd entry points
+ * then).  The wait of a workgroup for the other half of its row is bounded
+ * (mrl_set_wide_spin_limit): past the bound it computes that half's statistics itself from memory,
+ * with the same result to the last bit; in place that is safe because a workgroup overwrites its
+ * half only after its record has reached memory, and a reader that finds the record after all
+ * discards what it read. */
 int mrl_fused_logprob_loss(const void* logits, int logits_dtype, int64_t n_rows, int64_t vocab,
                            int64_t row_stride, const void* labels, int labels_dtype,
                            float inv_temperature, const float* row_ops, int has_old,
                            float clip_lo, float clip_hi, int kl_penalty, float kl_coef,
                            float entropy_coeff, float grad_scale, const float* grad_scale_dev,
                            void* dlogits, int64_t dlogits_row_stride, float* logp, float* entropy,
-                           float* row_terms, void* workspace, int64_t workspace_bytes, void* stream);
+                           float* row_terms, void* workspace, int64_t workspace_bytes,
+                           int workspace_cleared, void* stream);
+
+/* Polls a workgroup spends waiting for the record of the other half of a wide row before it reads
+ * that half itself (default 2^18; 0 = never wait, which exercises the fallback; negative restores
+ * the default).  Process-wide, read at every launch; returns the previous value.  No counterpart
+ * in the reference. */
+int64_t mrl_set_wide_spin_limit(int64_t polls);
 
 /* Step 3.  Sums row_terms per sequence (tokens with a non-zero mask but no logits row enter with
  * log_prob = entropy = 0, as in the split path) and finalizes out[8] / row_sums exactly like
- * mrl_policy_loss_fwd. */
+ * mrl_policy_loss_fwd.  done_counter (nullable): four zeroed bytes of device memory (word 1 of a
+ * cleared sweep workspace serves); with it the whole step is one launch - the workgroup that
+ * finishes last combines the sequences - and the counter is zero again afterwards.  loss_out
+ * (nullable): receives out[0] once more, for a caller that wants the loss in storage of its own. */
 int mrl_fused_loss_reduce(const float* row_terms, const int64_t* row_start,
                           const int32_t* row_count, int64_t batch, int64_t width,
                           const float* old_log_prob, const float* ref_log_prob,
@@ -345,7 +369,7 @@ int mrl_fused_loss_reduce(const float* row_terms, const int64_t* row_start,
                           const void* response_length, int response_dtype, float clip_lo,
                           float clip_hi, int kl_penalty, float kl_coef, float entropy_coeff,
                           int seq_mean, float loss_scale, float* row_sums, float* out,
-                          void* stream);
+                          uint32_t* done_counter, float* loss_out, void* stream);
 
 /* x[r, :] *= (*upstream / *applied) in place, unless that ratio is exactly 1 (then the kernel
  * exits without touching memory).  upstream and applied are DEVICE scalars: the gradient autograd
@@ -362,6 +386,15 @@ int mrl_scale_rows(void* x, int dtype, int64_t n_rows, int64_t vocab, int64_t ro
  * mrl_fused_logprob_loss reads through grad_scale_dev; *rescales (nullable) is incremented when
  * upstream differed from applied, i.e. when the rescale moved memory.  All DEVICE pointers. */
 int mrl_grad_scale_note(const float* upstream, float* applied, float* learned, uint32_t* rescales,
+                        void* stream);
+
+/* mrl_scale_rows followed by mrl_grad_scale_note for ONE buffer in ONE launch.  applied: two
+ * floats, 8-byte aligned: {the scale x carries, a counter that is zero between calls} - the pair
+ * mrl_fused_loss_prepare writes to scale_out.  An upstream gradient of 0, Inf or NaN is applied like
+ * any other (autograd's product) and recorded as the scale x now carries; it cannot be undone, so a
+ * later backward over the same buffer yields NaN rather than a wrong finite value. */
+int mrl_scale_rows_note(void* x, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                        const float* upstream, float* applied, float* learned, uint32_t* rescales,
                         void* stream);
 
 /* ------------------------------------------------------------------------------------------

@@ -1,20 +1,19 @@
-// Fused lm_head + log-prob for gfx950: streams hidden x W_vocab^T tiles through bf16 MFMA and
+// Fused lm_head + log-prob for gfx950: streams W_vocab x hidden^T tiles through bf16 MFMA and
 // keeps an online log-sum-exp per token, so the [T, V] logits are never written to memory.
 //
 //   logits[t, v] = sum_k hidden[t, k] * W[v, k]        (bf16 operands, fp32 accumulate)
 //   lse, logp[label], entropy exactly as the vocabulary sweep computes them, on the fp32 logits
 //
-// Mapping.  The product is computed TRANSPOSED, S^T = W_tile x hidden_tile^T with
-// v_mfma_f32_32x32x16_bf16: vocabulary rows are the MFMA's M, tokens its N.  In the 32x32 result
-// layout a lane then owns ONE token column and 16 vocabulary rows, so the softmax statistics of a
-// token accumulate inside a lane; only the two lane halves and the two vocabulary wavefronts have
-// to be combined once, at the very end.  A workgroup (256 threads = 2x2 wavefronts) owns 128 tokens
-// and walks over the 256-row vocabulary tiles of its vocabulary group; each wavefront computes a
-// 128 (vocab) x 64 (token) sub-tile = 4x2 MFMA blocks per 16-wide k-step, operands staged through
-// LDS (rows padded to 144 bytes), the next k-step's global loads in flight during the MFMAs.
-// Vocabulary groups (gridDim = token tiles x groups, group = blockIdx % groups so that the
-// workgroups of one XCD read the same W rows) leave per-group partial statistics that a small
-// second kernel merges, together with the label logit (one fp32 dot product per token).
+// Mapping.  The product runs on the shared tile loop of lmhead_tile.h (256 x 256 tiles, one
+// wavefront per SIMD with a 128 x 128 sub-tile of v_mfma_f32_16x16x32_bf16 blocks, operands straight
+// from global memory into two LDS stages) with the vocabulary as the MFMA's M and the tokens as its
+// N: in the 16x16 result layout a lane then owns ONE token column of each block and 4 vocabulary
+// rows, so the softmax statistics of a token accumulate inside a lane; only the four lane quarters
+// and the two vocabulary wavefronts have to be combined once, at the very end.  A workgroup owns
+// 256 tokens and walks the 256-row vocabulary tiles of its vocabulary group; the groups (8, dealt so
+// that the workgroups of one XCD share hidden blocks and weight tiles in its L2) leave per-group
+// partial statistics that a small second kernel merges, together with the label logit (one fp32 dot
+// product per token).
 #include <stdlib.h>
 
 #include <atomic>
@@ -33,181 +32,9 @@ namespace {
 
 using namespace mrl_vocab;
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-
-constexpr int kThreads = 256;
-constexpr int BV = 256;            // vocabulary rows per macro tile
-// tokens per macro tile = 64 * kTB: each of the two token wavefronts owns kTB 32-token MFMA blocks
-constexpr int BK = 64;             // k elements per LDS stage
-constexpr int kLdsStride = BK + 8; // bf16 elements per LDS row: 144 bytes, breaks the bank pattern
-constexpr int kChunksPerRow = BK / 8;                          // 16-byte chunks per row and stage
-constexpr int kALoads = BV * kChunksPerRow / kThreads;         // 8 chunks per thread
-
-template <int kTB>
-__global__ __launch_bounds__(kThreads, (kTB <= 2 ? 2 : 1)) void lmhead_fwd_kernel(
-    const uint16_t* __restrict__ hidden, const uint16_t* __restrict__ weight, int64_t n_tokens, int vocab, int hdim,
-    int n_groups, int tiles_per_group, float k_scale, float* __restrict__ partial) {
-    __shared__ __attribute__((aligned(16))) uint16_t As[BV * kLdsStride];
-    constexpr int BT = 64 * kTB;
-    constexpr int kBLoads = BT * kChunksPerRow / kThreads;
-    __shared__ __attribute__((aligned(16))) uint16_t Bs[BT * kLdsStride];
-    __shared__ Stats comb[2][kTB][32];   // [token half][token block][lane % 32]
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int wv = wave >> 1, wt = wave & 1;
-    const int group = blockIdx.x % n_groups;
-    const int64_t t0 = (int64_t)(blockIdx.x / n_groups) * BT;
-    const int n_vtiles = (vocab + BV - 1) / BV;
-    const int tile_begin = group * tiles_per_group;
-    const int tile_end = min(tile_begin + tiles_per_group, n_vtiles);
-
-    // global -> LDS staging: chunk c = tid + i*256 covers row c/8, 16-byte column c%8
-    const int ld_row = tid >> 3, ld_col = tid & 7;
-    // token rows of this workgroup as 32-bit element offsets from the tile base, clamped so that
-    // tail rows read valid memory (they are masked on output)
-    const uint16_t* b_base = hidden + t0 * hdim;
-    int b_off[kBLoads];
-#pragma unroll
-    for (int i = 0; i < kBLoads; ++i) {
-        int64_t r = ld_row + 32 * i;
-        if (t0 + r >= n_tokens) r = n_tokens - 1 - t0;
-        b_off[i] = (int)r * hdim + ld_col * 8;
-    }
-
-    Stats st[kTB];
-#pragma unroll
-    for (int tb = 0; tb < kTB; ++tb) st[tb] = {kMaxInit, 0.f, 0.f};
-
-    for (int tile = tile_begin; tile < tile_end; ++tile) {
-        const int v0 = tile * BV;
-        const uint16_t* a_base = weight + (int64_t)v0 * hdim;
-        int a_off[kALoads];
-#pragma unroll
-        for (int i = 0; i < kALoads; ++i) {
-            int r = ld_row + 32 * i;
-            if (v0 + r >= vocab) r = vocab - 1 - v0;
-            a_off[i] = r * hdim + ld_col * 8;
-        }
-        floatx16 acc[4][kTB];
-#pragma unroll
-        for (int vb = 0; vb < 4; ++vb)
-#pragma unroll
-            for (int tb = 0; tb < kTB; ++tb)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) acc[vb][tb][i] = 0.f;
-
-        u32x4 a_reg[kALoads], b_reg[kBLoads];
-#pragma unroll
-        for (int i = 0; i < kALoads; ++i) a_reg[i] = *reinterpret_cast<const u32x4*>(a_base + a_off[i]);
-#pragma unroll
-        for (int i = 0; i < kBLoads; ++i) b_reg[i] = *reinterpret_cast<const u32x4*>(b_base + b_off[i]);
-
-        const int n_ksteps = hdim / BK;
-        for (int kstep = 0; kstep < n_ksteps; ++kstep) {
-            __syncthreads();                               // the previous stage has been consumed
-#pragma unroll
-            for (int i = 0; i < kALoads; ++i)
-                *reinterpret_cast<u32x4*>(&As[(ld_row + 32 * i) * kLdsStride + ld_col * 8]) = a_reg[i];
-#pragma unroll
-            for (int i = 0; i < kBLoads; ++i)
-                *reinterpret_cast<u32x4*>(&Bs[(ld_row + 32 * i) * kLdsStride + ld_col * 8]) = b_reg[i];
-            __syncthreads();
-            if (kstep + 1 < n_ksteps) {                    // next stage's loads fly during the MFMAs
-                const int off = (kstep + 1) * BK;
-#pragma unroll
-                for (int i = 0; i < kALoads; ++i) a_reg[i] = *reinterpret_cast<const u32x4*>(a_base + off + a_off[i]);
-#pragma unroll
-                for (int i = 0; i < kBLoads; ++i) b_reg[i] = *reinterpret_cast<const u32x4*>(b_base + off + b_off[i]);
-            }
-#pragma unroll
-            for (int ks = 0; ks < BK / 16; ++ks) {
-                const int koff = ks * 16 + (lane >> 5) * 8;
-                bf16x8 af[4], bfr[kTB];
-#pragma unroll
-                for (int vb = 0; vb < 4; ++vb)
-                    af[vb] = *reinterpret_cast<const bf16x8*>(&As[(wv * 128 + vb * 32 + (lane & 31)) * kLdsStride + koff]);
-#pragma unroll
-                for (int tb = 0; tb < kTB; ++tb)
-                    bfr[tb] = *reinterpret_cast<const bf16x8*>(&Bs[(wt * 32 * kTB + tb * 32 + (lane & 31)) * kLdsStride + koff]);
-#pragma unroll
-                for (int vb = 0; vb < 4; ++vb)
-#pragma unroll
-                    for (int tb = 0; tb < kTB; ++tb)
-                        acc[vb][tb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[vb], bfr[tb], acc[vb][tb], 0, 0, 0);
-            }
-        }
-
-        // online softmax statistics of this tile: a lane holds 64 vocabulary rows of each token column
-        const bool ragged = (v0 + BV > vocab);
-#pragma unroll
-        for (int tb = 0; tb < kTB; ++tb) {
-            if (ragged) {
-#pragma unroll
-                for (int vb = 0; vb < 4; ++vb)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const int v = v0 + wv * 128 + vb * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
-                        if (v >= vocab) acc[vb][tb][i] = kMaxInit;
-                    }
-            }
-            float vmax = st[tb].m;
-#pragma unroll
-            for (int vb = 0; vb < 4; ++vb)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) vmax = fmaxf(vmax, acc[vb][tb][i]);
-            grow_max<true>(st[tb], vmax, k_scale);
-            // A lane that has seen no valid vocabulary row yet (the first tile of its group is ragged and
-            // ends above its rows) still holds the start value as its maximum: z * k - m * k of the masked
-            // entries would then be the rounding residual of two numbers of magnitude 1e30 instead of
-            // zero.  With an infinite m * k their exponentials are exactly 0.
-            const float mk = st[tb].m > kMaxInit ? st[tb].m * k_scale : __builtin_inff();
-#pragma unroll
-            for (int vb = 0; vb < 4; ++vb)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) add_one<true>(st[tb], acc[vb][tb][i], k_scale, mk);
-        }
-    }
-
-    // combine the two lane halves (same token, other vocabulary rows), then the two vocabulary wavefronts
-#pragma unroll
-    for (int tb = 0; tb < kTB; ++tb) {
-        Stats o;
-        o.m = __shfl_xor(st[tb].m, 32, 64);
-        o.s = __shfl_xor(st[tb].s, 32, 64);
-        o.u = __shfl_xor(st[tb].u, 32, 64);
-        st[tb] = merge<true>(st[tb], o, k_scale);
-    }
-    __syncthreads();
-    if (wv == 1 && lane < 32) {
-#pragma unroll
-        for (int tb = 0; tb < kTB; ++tb) comb[wt][tb][lane] = st[tb];
-    }
-    __syncthreads();
-    if (wv == 0 && lane < 32) {
-#pragma unroll
-        for (int tb = 0; tb < kTB; ++tb) {
-            const Stats r = merge<true>(st[tb], comb[wt][tb][lane], k_scale);
-            const int64_t t = t0 + wt * 32 * kTB + tb * 32 + lane;
-            if (t < n_tokens) {
-                float* p = partial + ((int64_t)group * n_tokens + t) * 4;
-                p[0] = r.m;
-                p[1] = r.s;
-                p[2] = r.u;
-                p[3] = 0.f;
-            }
-        }
-    }
-}
-
-// ------------------------------------------------------------------------------------------
-// Second generation: the shared tile loop of the lm_head products (lmhead_tile.h: 256 x 256 tiles, one
-// wavefront per SIMD with a 128 x 128 sub-tile on v_mfma_f32_16x16x32_bf16, operands straight into two
-// LDS stages) with the online softmax statistics as what is done with a finished tile.  A workgroup
-// owns 256 tokens and walks the vocabulary tiles of its group; the loop runs over the flattened
-// (vocabulary tile, k-step) sequence, so the first loads of the next tile are in flight during the
-// statistics of the current one.
+// The tiles of one workgroup: the vocabulary tiles of its group against its block of tokens.  The
+// tile loop runs over the flattened (vocabulary tile, k-step) sequence, so the first loads of the
+// next tile are in flight during the statistics of the current one.
 struct VocabGroupTiles {
     int tile_begin, n_tiles, token_tile;
     __device__ __forceinline__ void coords(int j, int& tm, int& tn) const {
@@ -216,7 +43,7 @@ struct VocabGroupTiles {
     }
 };
 
-__global__ __launch_bounds__(mrl_tile::kThreads, 1) void lmhead_fwd_kernel_v2(
+__global__ __launch_bounds__(mrl_tile::kThreads, 1) void lmhead_fwd_kernel(
     const uint16_t* __restrict__ hidden, const uint16_t* __restrict__ weight, int64_t n_tokens, int vocab, int hdim,
     int n_groups, int tiles_per_group, float k_scale, float* __restrict__ partial) {
     using namespace mrl_tile;
@@ -355,15 +182,6 @@ __global__ __launch_bounds__(256) void lmhead_finish_kernel(
     }
 }
 
-// MRL_LMHEAD_V2=0 selects the first-generation tile loop (a tuning / debugging switch).
-bool lmhead_v2_enabled() {
-    static const bool on = [] {
-        const char* e = getenv("MRL_LMHEAD_V2");
-        return !(e && e[0] == '0');
-    }();
-    return on;
-}
-
 }  // namespace
 
 extern "C" int64_t mrl_lmhead_workspace_bytes(int64_t n_tokens, int64_t vocab) {
@@ -377,34 +195,26 @@ static int lmhead_forward(const char* fn, const void* hidden, const void* weight
                           int64_t hidden_dim, const void* labels, int labels_dtype, float inv_temperature, float* logp,
                           float* entropy, float* lse, float* partial, hipStream_t s) {
     const int n_groups = MRL_LMHEAD_GROUPS;
-    const int n_vtiles = (int)((vocab + BV - 1) / BV);
-    const int tiles_per_group = (n_vtiles + n_groups - 1) / n_groups;
+    const int n_vtiles = (int)((vocab + mrl_tile::BM - 1) / mrl_tile::BM);
     // a group without tiles (tiny vocabularies) still writes its neutral partials
-    if (lmhead_v2_enabled()) {
-        // 256-token tiles, operands straight into two LDS stages (128 KiB of dynamic LDS)
-        constexpr int kLdsBytes2 = mrl_tile::kLdsStages, kThreads2 = mrl_tile::kThreads;
-        static const hipError_t attr = hipFuncSetAttribute((const void*)lmhead_fwd_kernel_v2,
-                                                           hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes2);
-        MRL_REQUIRE(attr == hipSuccess, MRL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", fn, kLdsBytes2,
-                    hipGetErrorString(attr));
-        MRL_REQUIRE(256 * hidden_dim * 2 < (1LL << 31) && n_tokens <= 0x7fffffffLL, MRL_ERR_UNSUPPORTED,
-                    "%s: size out of range", fn);
-        const int64_t n_ttiles = (n_tokens + mrl_tile::BN - 1) / mrl_tile::BN;
-        const int64_t n_rounds = (n_ttiles + 31) / 32;       // 32 token tiles x 8 groups per round of 256 workgroups
-        MRL_REQUIRE(n_rounds * 256 <= 0x7fffffffLL, MRL_ERR_UNSUPPORTED, "%s: grid too large", fn);
-        static_assert(MRL_LMHEAD_GROUPS == 8, "the workgroup mapping assumes 8 vocabulary groups");
-        hipLaunchKernelGGL(lmhead_fwd_kernel_v2, dim3((unsigned)(n_rounds * 256)), dim3(kThreads2), kLdsBytes2, s,
-                           (const uint16_t*)hidden, (const uint16_t*)weight, n_tokens, (int)vocab, (int)hidden_dim,
-                           n_groups, tiles_per_group, inv_temperature * kLog2e, partial);
-    } else {
-        // 128-token tiles (4x2 MFMA blocks per wavefront, two workgroups per CU), operands staged through registers
-        constexpr int kTokenBlocks = 2;
-        const int64_t n_ttiles = (n_tokens + 64 * kTokenBlocks - 1) / (64 * kTokenBlocks);
-        MRL_REQUIRE(n_ttiles * n_groups <= 0x7fffffffLL, MRL_ERR_UNSUPPORTED, "%s: grid too large", fn);
-        hipLaunchKernelGGL(lmhead_fwd_kernel<kTokenBlocks>, dim3((unsigned)(n_ttiles * n_groups)), dim3(kThreads), 0, s,
-                           (const uint16_t*)hidden, (const uint16_t*)weight, n_tokens, (int)vocab, (int)hidden_dim,
-                           n_groups, tiles_per_group, inv_temperature * kLog2e, partial);
-    }
+    const int tiles_per_group = (n_vtiles + n_groups - 1) / n_groups;
+    // 256-token tiles, operands straight into two LDS stages (128 KiB of dynamic LDS).  Function
+    // attributes belong to a device, so the reservation is made with every launch, on whichever
+    // device is current.
+    constexpr int kLdsBytes = mrl_tile::kLdsStages;
+    const hipError_t attr = hipFuncSetAttribute((const void*)lmhead_fwd_kernel,
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    MRL_REQUIRE(attr == hipSuccess, MRL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", fn, kLdsBytes,
+                hipGetErrorString(attr));
+    MRL_REQUIRE(256 * hidden_dim * 2 < (1LL << 31) && n_tokens <= 0x7fffffffLL, MRL_ERR_UNSUPPORTED,
+                "%s: size out of range", fn);
+    const int64_t n_ttiles = (n_tokens + mrl_tile::BN - 1) / mrl_tile::BN;
+    const int64_t n_rounds = (n_ttiles + 31) / 32;       // 32 token tiles x 8 groups per round of 256 workgroups
+    MRL_REQUIRE(n_rounds * 256 <= 0x7fffffffLL, MRL_ERR_UNSUPPORTED, "%s: grid too large", fn);
+    static_assert(MRL_LMHEAD_GROUPS == 8, "the workgroup mapping assumes 8 vocabulary groups");
+    hipLaunchKernelGGL(lmhead_fwd_kernel, dim3((unsigned)(n_rounds * 256)), dim3(mrl_tile::kThreads), kLdsBytes, s,
+                       (const uint16_t*)hidden, (const uint16_t*)weight, n_tokens, (int)vocab, (int)hidden_dim,
+                       n_groups, tiles_per_group, inv_temperature * kLog2e, partial);
     int rc = mrl::check_launch(fn);
     if (rc != MRL_OK) return rc;
     const dim3 fgrid((unsigned)((n_tokens + 3) / 4)), fblock(256);
@@ -424,8 +234,8 @@ static int lmhead_forward(const char* fn, const void* hidden, const void* weight
     MRL_REQUIRE(n_tokens >= 0 && vocab > 0 && hidden_dim > 0, MRL_ERR_INVALID_ARG,                                     \
                 "%s: n_tokens=%lld vocab=%lld hidden_dim=%lld", fn, (long long)n_tokens, (long long)vocab,             \
                 (long long)hidden_dim);                                                                                \
-    MRL_REQUIRE(hidden_dim % BK == 0, MRL_ERR_UNSUPPORTED, "%s: hidden_dim=%lld must be a multiple of %d", fn,         \
-                (long long)hidden_dim, BK);                                                                            \
+    MRL_REQUIRE(hidden_dim % mrl_tile::BK == 0, MRL_ERR_UNSUPPORTED, "%s: hidden_dim=%lld must be a multiple of %d", fn, \
+                (long long)hidden_dim, mrl_tile::BK);                                                                          \
     MRL_REQUIRE(vocab <= (1LL << 30) && hidden_dim <= (1LL << 20), MRL_ERR_UNSUPPORTED, "%s: size out of range", fn);  \
     MRL_REQUIRE(mrl::int_dtype_bytes(labels_dtype) != 0, MRL_ERR_UNSUPPORTED, "%s: labels dtype %d (want I32 or I64)", \
                 fn, labels_dtype);                                                                                     \

@@ -175,8 +175,9 @@ namespace mrl {
 template <bool kAccumulate, bool kATrans, bool kBTrans>
 static int launch_gemm(const char* fn, int grid, const void* a, int64_t lda, int64_t m, const void* b, int64_t ldb, int64_t n,
                        int64_t k, void* out, int64_t ldo, hipStream_t stream) {
-    static const hipError_t attr = hipFuncSetAttribute((const void*)gemm_kernel<kAccumulate, kATrans, kBTrans>,
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    // function attributes belong to a device: reserved with every launch, on whichever device is current
+    const hipError_t attr = hipFuncSetAttribute((const void*)gemm_kernel<kAccumulate, kATrans, kBTrans>,
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
     MRL_REQUIRE(attr == hipSuccess, MRL_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS", fn, kLdsBytes);
     hipLaunchKernelGGL((gemm_kernel<kAccumulate, kATrans, kBTrans>), dim3((unsigned)grid), dim3(kThreads), kLdsBytes, stream,
                        (const uint16_t*)a, lda, (int)m, (const uint16_t*)b, ldb, (int)n, (int)k, out, ldo);

@@ -22,6 +22,7 @@ struct FusedArgs {
     float clip_lo, clip_hi; int kl_penalty; float kl_coef, entropy_coeff, grad_scale;
     const float* grad_scale_dev;    // nullable device scalar that multiplies grad_scale
     void* workspace;                // nullable for narrow rows: row counter (+ half-row records)
+    bool workspace_cleared;         // the caller has zeroed it on this stream
     bool wide;                      // rows cut in two halves held by two workgroups
     int64_t half_elems;             // entries of the first half
     void* dlogits; int64_t d_stride;

@@ -9,12 +9,12 @@
 // that way) and all accesses are range-checked buffer accesses, so the unrolled bodies contain no
 // branch (see mrl_internal.h for why that matters).
 //
-// fused_sweep_kernel launches one workgroup per row; fused_sweep_persistent_kernel (the default
-// for large batches) launches one workgroup per CU that takes rows in ticket order and requests
-// its next row while it writes the current one.  bwd_chunk_kernel is the split path's backward
+// fused_sweep_kernel launches one workgroup per row (small batches, or no workspace);
+// fused_sweep_persistent_kernel launches one workgroup per CU that takes rows in ticket order and
+// requests its next row while it writes the current one.  bwd_chunk_kernel is the split path's backward
 // (upstream gradients and the log-sum-exp are inputs, so there is no statistics pass and nothing
 // has to stay on chip): a plain stream of one vector per thread.
-#include <stdlib.h>
+#include <atomic>
 
 #include "mrl_internal.h"
 #include "policy_terms.h"
@@ -357,10 +357,13 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_kernel(
 // the next unclaimed one.  With a fixed stride (row r, r + grid, ...) the workgroups drift apart and
 // the rows in flight spread over a wide stretch of memory; with tickets the rows in flight are always
 // the most recent `grid` consecutive ones, which the HBM system serves about a tenth faster.
-// The counter is four bytes of device memory that the caller owns (one per sweep that can be in
-// flight at a time); the launch resets it with ticket_reset_kernel on the same stream.
-__global__ void ticket_reset_kernel(unsigned int* counter, unsigned int first) {
-    if (threadIdx.x == 0) *counter = first;
+// The counter is the first four bytes of the caller's workspace and starts at ZERO: workgroup b
+// begins with unit b, and ticket t (the value the fetch-and-add returns) stands for unit
+// t + gridDim.x.  So "reset" means "clear": the workspace is zeroed by whoever prepares the sweep
+// (the prepare kernel of the loss, or clear_words_kernel below).
+__global__ void clear_words_kernel(unsigned long long* p, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0ull;
 }
 
 // Thread 0 passes its ticket to the workgroup through LDS.  The fences order LDS accesses only and
@@ -380,23 +383,32 @@ __device__ __forceinline__ uint32_t broadcast_ticket(uint32_t mine, uint32_t* sl
 // ------------------------------------------------------------------------------ wide rows
 // A row that does not fit the registers of one CU is cut into two halves that two workgroups hold at
 // the same time (units 2 r and 2 r + 1 of the ticket order, so the halves of a row are taken by
-// workgroups that ask for work one after the other).  Each workgroup publishes the statistics of
-// its half - 16 bytes in the caller's workspace, written and read with device-scope atomics only,
-// so that no cache has to be flushed - and picks up the other half's before it computes the row's
-// gradient.  A workgroup publishes BEFORE it waits, and nothing it does before publishing depends on
-// another workgroup, so waits cannot form a cycle; the wait is bounded all the same: when the limit
-// is reached the workgroup reads the other half from memory and computes its statistics itself.
-// That fallback is why wide rows are not swept in place: the other half must still hold logits.
+// workgroups that ask for work one after the other).  Each workgroup publishes a record of its half
+// - its statistics and, if the label lies in it, the logit at the label: 16 bytes in the caller's
+// workspace, written and read with device-scope atomics only, so that no cache has to be flushed -
+// and picks up the other half's before it computes the row's gradient.  A workgroup publishes BEFORE
+// it waits, and nothing it does before publishing depends on another workgroup, so waits cannot form
+// a cycle; the wait is bounded all the same: when the limit is reached the workgroup reads the other
+// half from memory and computes its statistics itself, with the partner's assignment of vectors to
+// threads and the same order of operations, so the result is the partner's to the last bit.
+//
+// In place (dlogits over the logits) the other half may be overwritten by its owner at any time
+// AFTER the owner has published: a workgroup waits until its record has reached memory before any of
+// its threads stores a gradient.  A workgroup that had to read the other half therefore looks at the
+// record once more afterwards: if it is there now, the record is used and what was read is thrown
+// away; if it still is not, the owner had not begun to write, and everything read was logits.
 struct HalfRecord {
     unsigned long long ms;      // (m, s): never 0, s >= 1 or NaN
-    unsigned long long u1;      // (u, 1)
+    unsigned long long uz;      // (u, logit at the label if it lies in this half, else 1): never 0
 };
 
 __device__ __forceinline__ unsigned long long pack2f(float lo, float hi) {
     return (unsigned long long)__float_as_uint(lo) | ((unsigned long long)__float_as_uint(hi) << 32);
 }
 
-// Statistics of a stretch of a row streamed from memory by the whole workgroup (the fallback above).
+// Statistics of a stretch of a row streamed from memory by the whole workgroup (the fallback above):
+// thread t takes vectors t, t + 1024, ... in this order, as thread_stats does with the vectors a
+// thread holds, and the reduction is the same.
 template <int DT, bool kEntropy>
 __device__ __forceinline__ Stats stream_stats(const typename Elem<DT>::T* base, int n_vec, float k, Stats* lds) {
     using E = Elem<DT>;
@@ -418,54 +430,84 @@ __device__ __forceinline__ Stats stream_stats(const typename Elem<DT>::T* base, 
     return block_reduce_1024<kEntropy>(st, k, lds);
 }
 
-// Publishes `mine` as half `half` of a row, waits (bounded) for the other half and returns the
-// statistics of the whole row, merged in the order (first half, second half) by both workgroups.
-// rec: the row's two records.  other_base / other_vec: where the other half's logits lie.
+// What thread 0 found in the other half's record.
+struct Inbox {
+    Stats st;
+    uint32_t zy_bits;           // fp32 bits of the logit at the label, if the other half holds it
+    uint32_t arrived;
+};
+
+__device__ __forceinline__ bool read_record(const HalfRecord* rec, unsigned long long& a, unsigned long long& b) {
+    if (a == 0) a = __hip_atomic_load(&rec->ms, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (b == 0) b = __hip_atomic_load(&rec->uz, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return a != 0 && b != 0;
+}
+
+__device__ __forceinline__ void fill_inbox(Inbox* in, unsigned long long a, unsigned long long b, bool ok) {
+    in->st.m = __uint_as_float((uint32_t)a);
+    in->st.s = __uint_as_float((uint32_t)(a >> 32));
+    in->st.u = __uint_as_float((uint32_t)b);
+    in->zy_bits = (uint32_t)(b >> 32);
+    in->arrived = ok ? 1u : 0u;
+}
+
+// Publishes `mine` (and z_y, the logit at the label, if this half holds it) as half `half` of a row,
+// waits (bounded) for the other half and returns the statistics of the whole row, merged in the order
+// (first half, second half) by both workgroups; z_y becomes the other half's where that half holds
+// the label (zy_there).  rec: the row's two records.  other_base / other_vec: where the other half's
+// logits lie; zy_ptr: where the logit at the label lies.
 template <int DT, bool kEntropy>
 __device__ __forceinline__ Stats exchange_halves(const Stats& mine, int half, HalfRecord* rec, uint32_t spin_limit,
                                                  const typename Elem<DT>::T* other_base, int other_vec, float k,
-                                                 Stats* lds, Stats* inbox, uint32_t* arrived) {
+                                                 Stats* lds, Inbox* inbox, bool zy_here, bool zy_there,
+                                                 const typename Elem<DT>::T* zy_ptr, float& z_y) {
+    using E = Elem<DT>;
     if (threadIdx.x == 0) {
+        // +0 would make an empty word of (u, z_y) = (0, 0): -0 is the same logit
+        const uint32_t zy_word = zy_here ? (__float_as_uint(z_y) == 0u ? 0x80000000u : __float_as_uint(z_y)) : 1u;
         __hip_atomic_store(&rec[half].ms, pack2f(mine.m, mine.s), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (kEntropy)
-            __hip_atomic_store(&rec[half].u1, pack2f(mine.u, __uint_as_float(1u)), __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
-        // at most spin_limit polls; with a limit of 0 the record is not looked at at all, so that the
-        // fallback can be exercised deterministically
-        unsigned long long a = 0, b = kEntropy ? 0ull : 1ull;
-        for (uint32_t polls = 0; polls < spin_limit; ++polls) {
-            if (a == 0) a = __hip_atomic_load(&rec[half ^ 1].ms, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (kEntropy && b == 0)
-                b = __hip_atomic_load(&rec[half ^ 1].u1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (a != 0 && b != 0) break;
-            __builtin_amdgcn_s_sleep(4);
+        __hip_atomic_store(&rec[half].uz, pack2f(kEntropy ? mine.u : 0.f, __uint_as_float(zy_word)), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+        // at most spin_limit polls; with a limit of 0 the record is not looked at here at all, so that
+        // the fallback can be exercised deterministically
+        unsigned long long a = 0, b = 0;
+        bool ok = false;
+        for (uint32_t polls = 0; polls < spin_limit && !ok; ++polls) {
+            ok = read_record(&rec[half ^ 1], a, b);
+            if (!ok) __builtin_amdgcn_s_sleep(4);
         }
-        const bool ok = a != 0 && b != 0;
-        inbox->m = __uint_as_float((uint32_t)a);
-        inbox->s = __uint_as_float((uint32_t)(a >> 32));
-        inbox->u = kEntropy ? __uint_as_float((uint32_t)b) : 0.f;
-        *arrived = ok ? 1u : 0u;
+        fill_inbox(inbox, a, b, ok);
+        // the record has reached memory before any thread of this workgroup stores a gradient
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
     __syncthreads();
-    Stats other = *inbox;
-    if (*arrived == 0u) other = stream_stats<DT, kEntropy>(other_base, other_vec, k, lds);   // uniform branch
+    Stats other = inbox->st;
+    if (inbox->arrived == 0u) {                                  // uniform branch
+        other = stream_stats<DT, kEntropy>(other_base, other_vec, k, lds);
+        if (threadIdx.x == 0) {
+            // the logit at the label from the other half, then - once it has arrived - the record again
+            uint32_t zy_mem = zy_there ? __float_as_uint(E::load(zy_ptr)) : 0u;
+            asm volatile("s_waitcnt vmcnt(0)" : "+v"(zy_mem)::"memory");
+            unsigned long long a = 0, b = 0;
+            const bool ok = read_record(&rec[half ^ 1], a, b);
+            fill_inbox(inbox, a, b, ok);
+            if (!ok) inbox->zy_bits = zy_mem;
+        }
+        __syncthreads();
+        if (inbox->arrived != 0u) other = inbox->st;
+    }
+    if (zy_there) z_y = __uint_as_float(inbox->zy_bits);
     return half == 0 ? merge<kEntropy>(mine, other, k) : merge<kEntropy>(other, mine, k);
-}
-
-__global__ void clear_words_kernel(unsigned long long* p, int64_t n) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) p[i] = 0ull;
 }
 
 // Persistent variant of the fused sweep: one workgroup per CU walks rows and, as it turns the
 // registers of a row into dlogits, refills them with its NEXT row, so the statistics pass of the next
 // row starts on its first vectors while the last are still arriving - the register file never has to
-// hold two rows.
-// kTicket: the next row is the next unclaimed one (see "row tickets" above), taken while the row is
-// being written; otherwise row r is followed by r + grid.
+// hold two rows.  The next row is the next unclaimed one (see "row tickets" above), taken while the
+// row is being written.
 // kWide: the units of work are half rows (see "wide rows" above): unit 2 r is the first
 // half_elems entries of row r, unit 2 r + 1 the rest; n_rows then counts units.
-template <int DT, int NV, bool kEntropy, bool kTicket, bool kWide>
+template <int DT, int NV, bool kEntropy, bool kWide>
 __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
     const typename Elem<DT>::T* logits, int64_t row_stride, int vocab, int64_t n_rows,
     const void* __restrict__ labels, int labels_dtype, float inv_t, const float* __restrict__ row_ops, int has_old,
@@ -479,8 +521,7 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
     // two slots used in turn: thread 0 may write the ticket of the following row while a slow
     // wavefront has yet to read this one's (one barrier per row separates a slot's reuse)
     __shared__ uint32_t next_row[2];
-    __shared__ Stats inbox;                 // the other half's statistics (wide rows)
-    __shared__ uint32_t arrived;
+    __shared__ Inbox inbox;                 // the other half's record (wide rows)
 
     const int tid = threadIdx.x;
     // bytes and vectors of a unit: the whole row, or its first / second half
@@ -490,7 +531,7 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
     const int64_t step = gridDim.x;
     if (grad_scale_dev) grad_scale *= *grad_scale_dev;
     // the counter as a 4-byte buffer: only the lane with offset 0 (thread 0) is inside it
-    const mrl::rsrc_t ticket = mrl::make_rsrc(kTicket ? (const void*)row_ticket : (const void*)dlogits, kTicket ? 4u : 0u);
+    const mrl::rsrc_t ticket = mrl::make_rsrc(row_ticket, 4u);
 
     // What a workgroup needs to know of the row it fetches next.  A row that is not a response token
     // is never read: its descriptor gets zero bytes, so the (unconditional) loads return zeros
@@ -556,19 +597,21 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
         const int64_t y_here = y - my_first;
         const bool y_mine = y_ok && (!kWide || (y_here >= 0 && y_here < (int64_t)(unit_bytes[half] / sizeof(T))));
         Next nx;
-        if (!kTicket) nx = plan(r + step);
         uint32_t zy_next = 0;
 
         bool wrote = false;                 // dlogits of row r written and the next row requested
         if (m != 0.f) {
-            const float z_y = E::from_bits(zy_bits);
+            float z_y = E::from_bits(zy_bits);
             const Stats st = thread_stats<DT, NV, kEntropy>(v, n_vec, k);
             Stats tot = block_reduce_1024<kEntropy>(st, k, lds);
             if (kWide) {
+                // the logit at the label as this unit loaded it counts only if the label lies in this
+                // half: the other half may already hold gradients when dlogits overwrite the logits
                 const int other_first = half ? 0 : half_elems;
-                tot = exchange_halves<DT, kEntropy>(tot, half, half_records + row * 2, spin_limit,
-                                                    logits + row * row_stride + other_first,
-                                                    (int)(unit_bytes[half ^ 1] / 16u), k, lds, &inbox, &arrived);
+                const T* whole = logits + row * row_stride;
+                tot = exchange_halves<DT, kEntropy>(tot, half, half_records + row * 2, spin_limit, whole + other_first,
+                                                    (int)(unit_bytes[half ^ 1] / 16u), k, lds, &inbox, y_mine,
+                                                    y_ok && !y_mine, whole + (y_ok ? y : 0), z_y);
             }
             float lse;
             const RowScalars s = row_scalars<kEntropy>(tot, k, inv_t, y_ok, z_y, ops, has_old, p, grad_scale, m, lse);
@@ -577,10 +620,9 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
                 const RowGrad g = row_grad<kEntropy>(s, k, inv_t, lse);
                 // the ticket is asked for ahead of the stores and picked up behind the first H of
                 // them: it is older than every store, so waiting for it does not wait for them
-                uint32_t mine = 0;
-                if (kTicket) mine = mrl::buf_atomic_add_u32(ticket, lane_offset(), 1u);
+                const uint32_t mine = mrl::buf_atomic_add_u32(ticket, lane_offset(), 1u);
                 grad_part<DT, kEntropy, 0, H>(v, g, dst);
-                if (kTicket) nx = plan((int64_t)broadcast_ticket(mine, &next_row[parity]));
+                nx = plan((int64_t)broadcast_ticket(mine, &next_row[parity]) + step);
                 load_part<0, H>(v, nx.row);
                 grad_part<DT, kEntropy, H, NV>(v, g, dst);
                 store_label_grad<DT, kEntropy>(dst, g, y_mine, y_here, z_y);
@@ -592,10 +634,9 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
             write_masked_row_outputs(row, logp, entropy, row_terms);
         }
         if (!wrote) {                       // no gradient for this row: zeros, same order of operations
-            uint32_t mine = 0;
-            if (kTicket) mine = mrl::buf_atomic_add_u32(ticket, lane_offset(), 1u);
+            const uint32_t mine = mrl::buf_atomic_add_u32(ticket, lane_offset(), 1u);
             zero_part<0, H>(dst);
-            if (kTicket) nx = plan((int64_t)broadcast_ticket(mine, &next_row[parity]));
+            nx = plan((int64_t)broadcast_ticket(mine, &next_row[parity]) + step);
             load_part<0, H>(v, nx.row);
             zero_part<H, NV>(dst);
             mrl::buf_store_b32(0u, mrl::make_rsrc(dlogits, 0u), 0u);
@@ -690,6 +731,44 @@ __global__ __launch_bounds__(256) void scale_rows_kernel(typename Elem<DT>::T* x
     }
 }
 
+// One backward of one buffer in a single launch: the conditional rescale above, then the book-keeping
+// of grad_scale_note_kernel by whichever workgroup finishes last (a counter next to the scale tells;
+// every workgroup has read the scale before it counts itself, so the last one may overwrite it).
+template <int DT>
+__global__ __launch_bounds__(256) void scale_rows_note_kernel(typename Elem<DT>::T* x, int64_t row_stride, int vocab,
+                                                              int64_t n_rows, const float* __restrict__ upstream,
+                                                              float* applied, float* learned, uint32_t* rescales) {
+    using E = Elem<DT>;
+    constexpr int kVec = E::kVec;
+    const float u = *upstream;
+    const float was = applied[0];
+    const float ratio = u / was;
+    if (ratio != 1.f) {
+        const int n_vec = vocab / kVec;
+        for (int64_t r = blockIdx.x; r < n_rows; r += gridDim.x) {
+            u32x4* vec = reinterpret_cast<u32x4*>(x + r * row_stride);
+            for (int idx = threadIdx.x; idx < n_vec; idx += 256) {
+                float z[kVec];
+                E::unpack(vec[idx], z);
+#pragma unroll
+                for (int i = 0; i < kVec; ++i) z[i] *= ratio;
+                vec[idx] = E::pack(z);
+            }
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t* done = reinterpret_cast<uint32_t*>(applied) + 1;
+        const uint32_t before = __hip_atomic_fetch_add(done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (before == gridDim.x - 1) {
+            if (rescales && ratio != 1.f) *rescales += 1u;
+            applied[0] = u;
+            *done = 0u;
+            if (learned && u != 0.f && __builtin_isfinite(u)) *learned = u;
+        }
+    }
+}
+
 // Book-keeping behind one or more scale_rows_kernel launches: the buffers now carry `upstream`.
 __global__ void grad_scale_note_kernel(const float* __restrict__ upstream, float* applied, float* learned,
                                        uint32_t* rescales) {
@@ -721,26 +800,15 @@ int cu_count() {
     return n;
 }
 
-// MRL_SWEEP_PERSISTENT=0 selects the one-workgroup-per-row launch (a tuning / debugging switch).
-bool persistent_enabled() {
-    static const bool on = [] {
-        const char* e = getenv("MRL_SWEEP_PERSISTENT");
-        return !(e && e[0] == '0');
-    }();
-    return on;
-}
-
 // Upper bound of the polls a workgroup spends waiting for the other half of a wide row before it
-// computes that half's statistics itself; MRL_WIDE_SPIN_LIMIT overrides it (0: never look, always compute).
-uint32_t wide_spin_limit() {
-    static const uint32_t limit = [] {
-        const char* e = getenv("MRL_WIDE_SPIN_LIMIT");
-        return e ? (uint32_t)strtoul(e, nullptr, 10) : (1u << 18);
-    }();
-    return limit;
-}
+// computes that half's statistics itself (mrl_set_wide_spin_limit; 0: never look, always compute).
+constexpr uint32_t kDefaultSpinLimit = 1u << 18;
+std::atomic<uint32_t> g_wide_spin_limit{kDefaultSpinLimit};
 
 constexpr int64_t kWorkspaceHeader = 16;    // the row counter, padded to the alignment of the records
+
+// Rows that go to the persistent workgroups; fewer get one workgroup each.
+inline bool wants_persistent(int64_t n_rows, int cus) { return cus > 0 && n_rows > 2 * (int64_t)cus; }
 
 template <int DT, int NV>
 int launch_fused(const mrl::FusedArgs& a) {
@@ -748,41 +816,33 @@ int launch_fused(const mrl::FusedArgs& a) {
     const dim3 block(kBlock);
     const Params p = {a.clip_lo, a.clip_hi, a.kl_coef, a.entropy_coeff, 1.f, a.kl_penalty, 0};
     unsigned int* counter = reinterpret_cast<unsigned int*>(a.workspace);
-    const bool tk = counter != nullptr;
-#define MRL_FUSEDP_LAUNCH(ENT, TK, WIDE, UNITS, HALF, REC)                                                         \
-    hipLaunchKernelGGL((fused_sweep_persistent_kernel<DT, NV, ENT, TK, WIDE>), pgrid, block, 0, a.stream,           \
-                       (const T*)a.logits, a.row_stride, (int)a.vocab, UNITS, a.labels, a.labels_dtype, a.inv_t,    \
-                       a.row_ops, a.has_old, p, a.grad_scale, a.grad_scale_dev, (T*)a.dlogits, a.d_stride, a.logp,  \
-                       a.entropy, a.row_terms, counter, HALF, REC, wide_spin_limit())
-    if (a.wide) {
-        // half rows: the persistent kernel for every batch size, an even number of workgroups
-        int cus = cu_count();
+    const int cus = cu_count();
+    const bool persistent = a.wide || (counter != nullptr && wants_persistent(a.n_rows, cus));
+    if (persistent) {
         if (cus < 2) return mrl::fail(MRL_ERR_LAUNCH, "mrl_fused_logprob_loss: cannot query the device");
-        const int64_t units = 2 * a.n_rows;
-        const unsigned grid = (unsigned)((int64_t)(cus & ~1) < units ? (cus & ~1) : units);
-        const dim3 pgrid(grid);
+        // half rows: an even number of workgroups, so that the halves of a row start side by side
+        const int64_t units = a.wide ? 2 * a.n_rows : a.n_rows;
+        const int64_t want = a.wide ? (cus & ~1) : cus;
+        const dim3 pgrid((unsigned)(want < units ? want : units));
         HalfRecord* rec = reinterpret_cast<HalfRecord*>(reinterpret_cast<char*>(a.workspace) + kWorkspaceHeader);
-        const int64_t words = a.n_rows * 4;
-        hipLaunchKernelGGL(clear_words_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, a.stream,
-                           reinterpret_cast<unsigned long long*>(rec), words);
-        hipLaunchKernelGGL(ticket_reset_kernel, dim3(1), dim3(64), 0, a.stream, counter, grid);
-        const int half = (int)a.half_elems;
-        if (a.with_entropy) MRL_FUSEDP_LAUNCH(true, true, true, units, half, rec);
-        else MRL_FUSEDP_LAUNCH(false, true, true, units, half, rec);
-        return mrl::check_launch("mrl_fused_logprob_loss");
-    }
-    const int cus = persistent_enabled() ? cu_count() : 0;
-    if (cus > 0 && a.n_rows > 2 * (int64_t)cus) {
-        const dim3 pgrid((unsigned)cus);
-        // the workgroups start on rows 0 .. grid-1; the counter hands out the rows behind them
-        if (tk) hipLaunchKernelGGL(ticket_reset_kernel, dim3(1), dim3(64), 0, a.stream, counter, (unsigned)cus);
-        if (a.with_entropy && tk) MRL_FUSEDP_LAUNCH(true, true, false, a.n_rows, 0, nullptr);
-        else if (a.with_entropy) MRL_FUSEDP_LAUNCH(true, false, false, a.n_rows, 0, nullptr);
-        else if (tk) MRL_FUSEDP_LAUNCH(false, true, false, a.n_rows, 0, nullptr);
-        else MRL_FUSEDP_LAUNCH(false, false, false, a.n_rows, 0, nullptr);
-        return mrl::check_launch("mrl_fused_logprob_loss");
-    }
+        if (!a.workspace_cleared) {
+            const int64_t words = (kWorkspaceHeader + (a.wide ? a.n_rows * 2 * (int64_t)sizeof(HalfRecord) : 0)) / 8;
+            hipLaunchKernelGGL(clear_words_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, a.stream,
+                               reinterpret_cast<unsigned long long*>(a.workspace), words);
+        }
+        const uint32_t spin = g_wide_spin_limit.load(std::memory_order_relaxed);
+#define MRL_FUSEDP_LAUNCH(ENT, WIDE)                                                                               \
+    hipLaunchKernelGGL((fused_sweep_persistent_kernel<DT, NV, ENT, WIDE>), pgrid, block, 0, a.stream,               \
+                       (const T*)a.logits, a.row_stride, (int)a.vocab, units, a.labels, a.labels_dtype, a.inv_t,    \
+                       a.row_ops, a.has_old, p, a.grad_scale, a.grad_scale_dev, (T*)a.dlogits, a.d_stride, a.logp,  \
+                       a.entropy, a.row_terms, counter, (int)a.half_elems, rec, spin)
+        if (a.wide && a.with_entropy) MRL_FUSEDP_LAUNCH(true, true);
+        else if (a.wide) MRL_FUSEDP_LAUNCH(false, true);
+        else if (a.with_entropy) MRL_FUSEDP_LAUNCH(true, false);
+        else MRL_FUSEDP_LAUNCH(false, false);
 #undef MRL_FUSEDP_LAUNCH
+        return mrl::check_launch("mrl_fused_logprob_loss");
+    }
     const dim3 grid((unsigned)a.n_rows);
 #define MRL_FUSED_LAUNCH(ENT)                                                                                  \
     hipLaunchKernelGGL((fused_sweep_kernel<DT, NV, ENT>), grid, block, 0, a.stream, (const T*)a.logits,        \
@@ -868,10 +928,8 @@ bool row_sweep_supported(int dtype, int64_t vocab, const void* in, int64_t in_st
     const int64_t per_vec = 16 / eb;
     if (vocab % per_vec != 0) return false;
     const int64_t n_vec = vocab / per_vec;
-    if (pick_nv(n_vec) == 0) {
-        // two halves held by two workgroups: not in place (see "wide rows")
-        if (pick_nv((n_vec + 1) / 2) == 0 || in == out) return false;
-    }
+    // wider rows: two halves held by two workgroups (see "wide rows")
+    if (pick_nv(n_vec) == 0 && pick_nv((n_vec + 1) / 2) == 0) return false;
     if (!aligned(in, 16) || !aligned(out, 16)) return false;
     if (n_rows > 1 && ((in_stride * eb) % 16 != 0 || (out_stride * eb) % 16 != 0)) return false;
     return true;
@@ -894,15 +952,21 @@ extern "C" int64_t mrl_fused_workspace_bytes(int logits_dtype, int64_t n_rows, i
     return kWorkspaceHeader + n_rows * (int64_t)sizeof(HalfRecord) * 2;
 }
 
+extern "C" int64_t mrl_set_wide_spin_limit(int64_t polls) {
+    const uint32_t next = polls < 0 ? kDefaultSpinLimit : (uint32_t)(polls > 0xffffffffLL ? 0xffffffffLL : polls);
+    return (int64_t)g_wide_spin_limit.exchange(next, std::memory_order_relaxed);
+}
+
 extern "C" int mrl_fused_logprob_loss(const void* logits, int logits_dtype, int64_t n_rows, int64_t vocab,
                                       int64_t row_stride, const void* labels, int labels_dtype,
                                       float inv_temperature, const float* row_ops, int has_old, float clip_lo,
                                       float clip_hi, int kl_penalty, float kl_coef, float entropy_coeff,
                                       float grad_scale, const float* grad_scale_dev, void* dlogits,
                                       int64_t dlogits_row_stride, float* logp, float* entropy, float* row_terms,
-                                      void* workspace, int64_t workspace_bytes, void* stream) {
+                                      void* workspace, int64_t workspace_bytes, int workspace_cleared,
+                                      void* stream) {
     const char* fn = "mrl_fused_logprob_loss";
-    MRL_REQUIRE(n_rows >= 0 && vocab > 0 && n_rows <= 0x7fffffffLL, MRL_ERR_INVALID_ARG, "%s: n_rows=%lld vocab=%lld",
+    MRL_REQUIRE(n_rows >= 0 && vocab > 0 && n_rows <= 0x3fffffffLL, MRL_ERR_INVALID_ARG, "%s: n_rows=%lld vocab=%lld",
                 fn, (long long)n_rows, (long long)vocab);
     const int eb = mrl::float_dtype_bytes(logits_dtype);
     MRL_REQUIRE(eb != 0, MRL_ERR_UNSUPPORTED, "%s: logits dtype %d (want F32, BF16 or F16)", fn, logits_dtype);
@@ -920,8 +984,7 @@ extern "C" int mrl_fused_logprob_loss(const void* logits, int logits_dtype, int6
                 "%s: workspace must be 16-byte and grad_scale_dev 4-byte aligned", fn);
     MRL_REQUIRE(mrl::row_sweep_supported(logits_dtype, vocab, logits, row_stride, dlogits, dlogits_row_stride, n_rows),
                 MRL_ERR_UNSUPPORTED,
-                "%s: needs 16-byte aligned rows, vocab %% %d == 0 and vocab <= %lld for this dtype (got vocab=%lld); rows "
-                "above half of that are not swept in place", fn,
+                "%s: needs 16-byte aligned rows, vocab %% %d == 0 and vocab <= %lld for this dtype (got vocab=%lld)", fn,
                 16 / eb, (long long)mrl_fused_max_vocab(logits_dtype), (long long)vocab);
     if (dlogits != logits) {
         const char* x = (const char*)logits;
@@ -936,7 +999,7 @@ extern "C" int mrl_fused_logprob_loss(const void* logits, int logits_dtype, int6
     a.labels = labels; a.labels_dtype = labels_dtype; a.inv_t = inv_temperature; a.row_ops = row_ops;
     a.has_old = has_old; a.clip_lo = clip_lo; a.clip_hi = clip_hi; a.kl_penalty = kl_penalty; a.kl_coef = kl_coef;
     a.entropy_coeff = entropy_coeff; a.grad_scale = grad_scale; a.grad_scale_dev = grad_scale_dev;
-    a.workspace = workspace; a.dlogits = dlogits; a.d_stride = dlogits_row_stride;
+    a.workspace = workspace; a.workspace_cleared = workspace_cleared != 0; a.dlogits = dlogits; a.d_stride = dlogits_row_stride;
     a.logp = logp; a.entropy = entropy; a.row_terms = row_terms; a.with_entropy = (entropy != nullptr);
     a.stream = mrl::as_stream(stream);
     const int64_t n_vec = vocab / (16 / eb);
@@ -948,7 +1011,7 @@ extern "C" int mrl_fused_logprob_loss(const void* logits, int logits_dtype, int6
         nv = pick_nv((n_vec + 1) / 2);
     }
     if (workspace != nullptr || a.wide) {
-        const int64_t need = mrl_fused_workspace_bytes(logits_dtype, n_rows, vocab);
+        const int64_t need = a.wide ? mrl_fused_workspace_bytes(logits_dtype, n_rows, vocab) : kWorkspaceHeader;
         MRL_REQUIRE(workspace != nullptr && workspace_bytes >= need, MRL_ERR_INVALID_ARG,
                     "%s: workspace of %lld bytes, need %lld (rows of this width are cut in two halves that exchange "
                     "their statistics through it)", fn, (long long)(workspace ? workspace_bytes : 0), (long long)need);
@@ -1002,5 +1065,39 @@ extern "C" int mrl_grad_scale_note(const float* upstream, float* applied, float*
                 MRL_ERR_MISALIGNED, "%s: pointers must be 4-byte aligned", fn);
     hipLaunchKernelGGL(grad_scale_note_kernel, dim3(1), dim3(64), 0, mrl::as_stream(stream), upstream, applied, learned,
                        rescales);
+    return mrl::check_launch(fn);
+}
+
+extern "C" int mrl_scale_rows_note(void* x, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                                   const float* upstream, float* applied, float* learned, uint32_t* rescales,
+                                   void* stream) {
+    const char* fn = "mrl_scale_rows_note";
+    const int eb = mrl::float_dtype_bytes(dtype);
+    MRL_REQUIRE(eb != 0, MRL_ERR_UNSUPPORTED, "%s: dtype %d (want F32, BF16 or F16)", fn, dtype);
+    MRL_REQUIRE(n_rows > 0 && n_rows <= 0x7fffffffLL && vocab > 0 && row_stride >= vocab, MRL_ERR_INVALID_ARG,
+                "%s: n_rows=%lld vocab=%lld row_stride=%lld", fn, (long long)n_rows, (long long)vocab,
+                (long long)row_stride);
+    MRL_REQUIRE(x && upstream && applied, MRL_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+    MRL_REQUIRE(mrl::aligned(upstream, 4) && mrl::aligned(applied, 8) && mrl::aligned(learned, 4) &&
+                    mrl::aligned(rescales, 4),
+                MRL_ERR_MISALIGNED, "%s: applied must be 8-byte, the other scalars 4-byte aligned", fn);
+    MRL_REQUIRE(vocab % (16 / eb) == 0 && mrl::aligned(x, 16) && (n_rows == 1 || (row_stride * eb) % 16 == 0),
+                MRL_ERR_UNSUPPORTED, "%s: needs 16-byte aligned rows", fn);
+    hipStream_t s = mrl::as_stream(stream);
+    const dim3 grid((unsigned)(n_rows < 1024 ? n_rows : 1024)), block(256);
+    switch (dtype) {
+        case MRL_F32:
+            hipLaunchKernelGGL(scale_rows_note_kernel<MRL_F32>, grid, block, 0, s, (float*)x, row_stride, (int)vocab,
+                               n_rows, upstream, applied, learned, rescales);
+            break;
+        case MRL_BF16:
+            hipLaunchKernelGGL(scale_rows_note_kernel<MRL_BF16>, grid, block, 0, s, (uint16_t*)x, row_stride,
+                               (int)vocab, n_rows, upstream, applied, learned, rescales);
+            break;
+        default:
+            hipLaunchKernelGGL(scale_rows_note_kernel<MRL_F16>, grid, block, 0, s, (uint16_t*)x, row_stride,
+                               (int)vocab, n_rows, upstream, applied, learned, rescales);
+            break;
+    }
     return mrl::check_launch(fn);
 }

@@ -323,16 +323,6 @@ int launch_bwd(const void* logits, int64_t n_rows, int vocab, int64_t row_stride
     return mrl::check_launch("mrl_vocab_logprob_bwd");
 }
 
-// MRL_BWD_CHUNK=0 keeps the one-workgroup-per-row backward kernel for every shape (a tuning /
-// debugging switch).
-bool bwd_chunks_enabled() {
-    static const bool on = [] {
-        const char* e = getenv("MRL_BWD_CHUNK");
-        return !(e && e[0] == '0');
-    }();
-    return on;
-}
-
 int check_common(const char* fn, const void* logits, int logits_dtype, int64_t n_rows, int64_t vocab,
                  int64_t row_stride, const void* labels, int labels_dtype, float inv_t) {
     MRL_REQUIRE(n_rows >= 0 && vocab > 0, MRL_ERR_INVALID_ARG, "%s: n_rows=%lld vocab=%lld", fn,
@@ -436,7 +426,7 @@ extern "C" int mrl_vocab_logprob_bwd(const void* logits, int logits_dtype, int64
     hipStream_t s = mrl::as_stream(stream);
     const int v = (int)vocab;
     // rows from 16 KiB on, same dtype in and out: the streaming kernel (one vector per thread)
-    if (dlogits_dtype == logits_dtype && bwd_chunks_enabled() &&
+    if (dlogits_dtype == logits_dtype &&
         mrl::bwd_chunks_supported(logits_dtype, vocab, logits, row_stride, dlogits, dlogits_row_stride, n_rows)) {
         const mrl::BwdArgs a = {logits, logits_dtype, n_rows, vocab, row_stride, labels, labels_dtype, inv_temperature,
                                 lse, entropy, g_logp, g_entropy, dlogits, dlogits_row_stride, s};

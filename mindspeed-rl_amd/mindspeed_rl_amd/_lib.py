@@ -50,14 +50,16 @@ SIGNATURES = {
                             _f32, _vp, _vp, _vp, _vp, _vp, _vp],
     "mrl_fused_max_vocab": [_int],
     "mrl_fused_loss_prepare": [_int, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _int, _vp, _int, _vp, _vp, _vp, _vp, _int,
-                               _int, _vp, _vp, _vp, _vp, _vp],
+                               _int, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _f32, _vp, _vp],
     "mrl_fused_workspace_bytes": [_int, _i64, _i64],
     "mrl_fused_logprob_loss": [_vp, _int, _i64, _i64, _i64, _vp, _int, _f32, _vp, _int, _f32, _f32, _int, _f32, _f32,
-                               _f32, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp],
+                               _f32, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _int, _vp],
+    "mrl_set_wide_spin_limit": [_i64],
     "mrl_fused_loss_reduce": [_vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _int, _vp, _int, _f32, _f32, _int, _f32,
-                              _f32, _int, _f32, _vp, _vp, _vp],
+                              _f32, _int, _f32, _vp, _vp, _vp, _vp, _vp],
     "mrl_scale_rows": [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp],
     "mrl_grad_scale_note": [_vp, _vp, _vp, _vp, _vp],
+    "mrl_scale_rows_note": [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp],
     "mrl_lmhead_workspace_bytes": [_i64, _i64],
     "mrl_lmhead_logprob_fwd": [_vp, _vp, _i64, _i64, _i64, _vp, _int, _f32, _vp, _vp, _vp, _vp, _i64, _vp],
     "mrl_lmhead_logits": [_vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp],
@@ -75,7 +77,8 @@ SIGNATURES = {
     "mrl_bandwidth_probe": [_int, _vp, _vp, _i64, _i64, _vp],
 }
 _RESTYPES = {"mrl_last_error": ctypes.c_char_p, "mrl_fused_workspace_bytes": ctypes.c_int64, "mrl_fused_max_vocab": ctypes.c_int64,
-             "mrl_lmhead_workspace_bytes": ctypes.c_int64, "mrl_lmhead_static_max_tokens": ctypes.c_int64}
+             "mrl_lmhead_workspace_bytes": ctypes.c_int64, "mrl_lmhead_static_max_tokens": ctypes.c_int64,
+             "mrl_set_wide_spin_limit": ctypes.c_int64}
 
 _lib = None
 

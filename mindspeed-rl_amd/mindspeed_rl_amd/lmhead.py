@@ -103,9 +103,8 @@ class _FusedLmHeadLoss(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, hidden, weight, labels, batch, cfg):
-        from .loss import _expected_scale, _mask_args, _sweep_workspace
+        from .loss import _FusedOperands
         dev = _lib.require_device(hidden, weight, labels)
-        lib = _lib.load()
         hdim = hidden.shape[-1]
         h2d = hidden.detach().reshape(-1, hdim).contiguous()
         w = weight.detach().contiguous()
@@ -115,42 +114,14 @@ class _FusedLmHeadLoss(torch.autograd.Function):
             lab = lab.to(torch.int64)
         lab = lab.contiguous()
         n_seq, width = batch["responses"].shape[0], batch["responses"].shape[-1]
-
-        def f32(t):
-            return None if t is None else t.to(dev).to(torch.float32).contiguous()
-
-        def idx(t):
-            if t.dtype not in (torch.int32, torch.int64):
-                t = t.to(torch.int64)
-            return t.to(dev).reshape(-1).contiguous()
-
-        old, ref, adv = f32(batch.get("old_log_prob")), f32(cfg["ref_log_prob"]), f32(batch.get("advantages"))
-        mask_t, _ = _mask_args(cfg["mask"], batch["response_length"], dev)
-        prompt, resp = idx(batch["prompt_length"]), idx(batch["response_length"])
-        if cfg["packed"]:
-            layout, padded_s = 0, 0
-            seqlens = cfg["seqlens"].to(dev).to(torch.int32).contiguous()
-            cu = cfg["cu"].to(dev).to(torch.int32).contiguous()
-        else:
-            layout, padded_s = 1, hidden.shape[1]
-            seqlens = cu = None
-        row_start = torch.empty(n_seq, dtype=torch.int64, device=dev)
-        row_count = torch.empty(n_seq, dtype=torch.int32, device=dev)
-        seq_msum = torch.empty(n_seq, dtype=torch.float32, device=dev)
-        row_ops = torch.empty(n_rows * 8, dtype=torch.float32, device=dev)
-        row_terms = torch.empty(n_rows * 8, dtype=torch.float32, device=dev)
-        row_sums = torch.empty(max(n_seq, 1) * 8, dtype=torch.float32, device=dev)
-        out = torch.empty(8, dtype=torch.float32, device=dev)
+        layout, padded_s = (0, 0) if cfg["packed"] else (1, hidden.shape[1])
+        chunk_cap = max(1, min(int(cfg["chunk_rows"]), max(n_rows, 1)))
+        ops = _FusedOperands(dev, batch, cfg, n_rows, n_seq, width, layout, padded_s, _lib.BF16, vocab, chunk_cap)
         want_ent = cfg["entropy_coeff"] != 0
-        ent = torch.empty(n_rows, dtype=torch.float32, device=dev) if want_ent else None
+        ent = torch.empty(max(n_rows, 1), dtype=torch.float32, device=dev) if want_ent else None
         stream = _lib.stream(dev)
-        mdt = _lib.dtype_code(mask_t) if mask_t is not None else _lib.F32
-        pdt, rdt = _lib.dtype_code(prompt), _lib.dtype_code(resp)
-        _lib.call("mrl_fused_loss_prepare", layout, n_seq, width, n_rows, _lib.ptr(seqlens), _lib.ptr(cu), padded_s,
-                  _lib.ptr(prompt), pdt, _lib.ptr(resp), rdt, _lib.ptr(old), _lib.ptr(ref), _lib.ptr(adv),
-                  _lib.ptr(mask_t), mdt, cfg["seq_mean"], _lib.ptr(row_start), _lib.ptr(row_count),
-                  _lib.ptr(seq_msum), _lib.ptr(row_ops), stream)
-        grad_scale, scale_dev, applied = _expected_scale(cfg, dev)
+        ops.prepare(stream)
+        row_ops = ops.rows[:max(n_rows, 1) * 8]
         # Rows whose mask is zero (prompts, padding, masked tokens) add nothing to the loss, to dWeight or
         # to their own dHidden: when they are more than a twentieth of the rows, the live rows are gathered
         # and only they go through the products.  The row count sizes the products, so it is read back (one
@@ -161,14 +132,15 @@ class _FusedLmHeadLoss(torch.autograd.Function):
             if live.numel() * 20 > n_rows * 19:
                 live = None
         all_rows, h_all = n_rows, h2d
+        p_ops, p_terms = ops.p_ops, ops.p_terms
         if live is not None:
             n_rows = live.numel()
             h2d = h_all.index_select(0, live)
             lab = lab.index_select(0, live)
             row_ops = row_ops.view(all_rows, 8).index_select(0, live).reshape(-1)
-            terms_all, row_terms = row_terms, torch.empty(max(n_rows, 1) * 8, dtype=torch.float32, device=dev)
-            ent = torch.empty(max(n_rows, 1), dtype=torch.float32, device=dev) if want_ent else None
-        chunk = max(1, min(int(cfg["chunk_rows"]), n_rows))
+            row_terms = torch.empty(max(n_rows, 1) * 8, dtype=torch.float32, device=dev)
+            p_ops, p_terms = row_ops.data_ptr(), row_terms.data_ptr()
+        chunk = max(1, min(chunk_cap, n_rows))
         # the chunk of logits: rows padded to whole k-steps of the dHidden product; the padding columns
         # are zeroed once and never written (they meet rows of the weight that read as zero)
         v_pad = _round_up(vocab, 64)
@@ -178,38 +150,35 @@ class _FusedLmHeadLoss(torch.autograd.Function):
             logits = torch.empty((chunk, v_pad), dtype=h2d.dtype, device=dev)
         d_hidden = torch.empty_like(h2d)
         d_weight32 = torch.zeros((vocab, hdim), dtype=torch.float32, device=dev)
-        sweep_bytes = lib.mrl_fused_workspace_bytes(_lib.dtype_code(logits), chunk, vocab)
-        sweep_ws = torch.empty(max(sweep_bytes, 16), dtype=torch.uint8, device=dev)
         esz = h2d.element_size()
         for c0 in range(0, n_rows, chunk):
             rows = min(n_rows, c0 + chunk) - c0
             h_c = h2d.data_ptr() + c0 * hdim * esz
             _timed("mrl_lmhead_logits", rows, dev, h_c, _lib.ptr(w), rows, vocab, hdim, _lib.ptr(logits), v_pad, stream)
+            # the first sweep finds the workspace cleared by the prepare step, the others clear it themselves
             vocab_ops._timed_call(
                 "mrl_fused_logprob_loss", rows, dev, _lib.ptr(logits), _lib.dtype_code(logits), rows, vocab, v_pad,
                 lab.data_ptr() + c0 * lab.element_size(), _lib.dtype_code(lab), cfg["inv_temperature"],
-                row_ops.data_ptr() + c0 * 32, 0 if old is None else 1, cfg["clip_lo"], cfg["clip_hi"], cfg["kl_penalty"],
-                cfg["kl_coef"], cfg["entropy_coeff"], grad_scale, _lib.ptr(scale_dev), _lib.ptr(logits), v_pad, None,
-                (ent.data_ptr() + c0 * 4) if want_ent else None, row_terms.data_ptr() + c0 * 32, _lib.ptr(sweep_ws),
-                sweep_bytes, stream)
+                p_ops + c0 * 32, 0 if ops.old is None else 1, cfg["clip_lo"], cfg["clip_hi"], cfg["kl_penalty"],
+                cfg["kl_coef"], cfg["entropy_coeff"], cfg["loss_scale"], _lib.ptr(ops.applied), _lib.ptr(logits), v_pad,
+                None, (ent.data_ptr() + c0 * 4) if want_ent else None, p_terms + c0 * 32, ops.workspace,
+                ops.ws_bytes, 1 if c0 == 0 else 0, stream)
             _timed("mrl_lmhead_logprob_bwd", rows, dev, h_c, _lib.ptr(w), _lib.ptr(logits), v_pad, rows, vocab, hdim,
                    d_hidden.data_ptr() + c0 * hdim * esz, _lib.ptr(d_weight32), stream)
         if live is not None:
-            compact_dh, compact_terms = d_hidden, row_terms
+            compact_dh = d_hidden
             d_hidden = torch.zeros_like(h_all)
             d_hidden.index_copy_(0, live, compact_dh)
-            row_terms = terms_all.zero_()
-            row_terms.view(all_rows, 8).index_copy_(0, live, compact_terms[:n_rows * 8].view(n_rows, 8))
-        _lib.call("mrl_fused_loss_reduce", _lib.ptr(row_terms), _lib.ptr(row_start), _lib.ptr(row_count), n_seq, width,
-                  _lib.ptr(old), _lib.ptr(ref), _lib.ptr(adv), _lib.ptr(mask_t), mdt, _lib.ptr(resp), rdt,
-                  cfg["clip_lo"], cfg["clip_hi"], cfg["kl_penalty"], cfg["kl_coef"], cfg["entropy_coeff"],
-                  cfg["seq_mean"], cfg["loss_scale"], _lib.ptr(row_sums), _lib.ptr(out), stream)
+            terms_all = ops.rows[all_rows * 8:all_rows * 16].zero_()
+            terms_all.view(all_rows, 8).index_copy_(0, live, row_terms[:n_rows * 8].view(n_rows, 8))
+        ops.reduce(stream)
+        applied = ops.applied
         d_weight = d_weight32.to(w.dtype)
         ctx.save_for_backward(d_hidden, d_weight, applied)
         ctx.meta = (tuple(hidden.shape), cfg.get("scale_state"))
         ctx.handed_out = False
-        ctx.mark_non_differentiable(out)
-        return out[0].clone(), out
+        ctx.mark_non_differentiable(ops.out)
+        return ops.loss, ops.out
 
     @staticmethod
     def backward(ctx, g_loss, _g_out):

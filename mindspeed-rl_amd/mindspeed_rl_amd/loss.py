@@ -142,13 +142,14 @@ def policy_loss(log_prob, entropy, old_log_prob, ref_log_prob, advantages, mask=
 def fused_supported(output, grad_inplace=False):
     """True if the row-in-registers kernel can take these logits: a floating dtype it knows,
     16-byte aligned dense rows and a vocabulary that fits the register files of one workgroup
-    (or of two, which is not available for an in-place gradient)."""
+    or of two.  (``grad_inplace`` is accepted for call compatibility: every supported shape can
+    also be swept in place.)"""
     if output.dtype not in (torch.float32, torch.bfloat16, torch.float16) or not output.is_cuda:
         return False
     vocab = output.shape[-1]
     per_vec = 16 // output.element_size()
     limit = _lib.load().mrl_fused_max_vocab(_lib.dtype_code(output))
-    if vocab % per_vec != 0 or vocab > (limit // 2 if grad_inplace else limit):
+    if vocab % per_vec != 0 or vocab > limit:
         return False
     return output.is_contiguous() and output.data_ptr() % 16 == 0
 
@@ -168,41 +169,23 @@ class GradScaleState:
         self.rescales = torch.zeros(1, dtype=torch.int32, device=device)
 
 
-def _sweep_workspace(flat):
-    """(tensor or None, bytes): the fused sweep's workspace for these ``[rows, V]`` logits, from
-    torch's allocator per call (a sweep in flight never shares it): the row counter of the
-    persistent workgroups and, for rows that two workgroups hold, the half-row records.
-    MRL_SWEEP_TICKET=0 withholds it where it is optional, which makes the sweep walk rows with a
-    fixed stride instead (a tuning switch)."""
-    n_bytes = _lib.load().mrl_fused_workspace_bytes(_lib.dtype_code(flat), flat.shape[0], flat.shape[1])
-    if n_bytes <= 16 and os.environ.get("MRL_SWEEP_TICKET", "1") == "0":
-        return None, 0
-    return torch.empty(max(n_bytes, 16), dtype=torch.uint8, device=flat.device), n_bytes
-
-
-def _note_upstream(upstream, applied, state, stream):
-    _lib.call("mrl_grad_scale_note", _lib.ptr(upstream), _lib.ptr(applied),
-              _lib.ptr(state.learned) if state is not None else None,
-              _lib.ptr(state.rescales) if state is not None else None, stream)
-
-
-def _expected_scale(cfg, dev):
-    """(host factor, device scalar or None, applied): the scale the sweep writes into its gradients.
-    An explicit ``expected_upstream`` wins; else the loss object's learned scale is read on the
-    device; else 1."""
+def _expected_scale(cfg):
+    """(device scalar or None, host factor): the scale the sweep writes into its gradients is their
+    product.  An explicit ``expected_upstream`` wins; else the loss object's learned scale is read
+    on the device; else 1."""
     state, explicit = cfg.get("scale_state"), cfg.get("expected_upstream")
     if explicit is None and state is not None:
-        applied = state.learned.clone()
-        return cfg["loss_scale"], applied, applied
-    expected = 1.0 if explicit is None else float(explicit)
-    return cfg["loss_scale"] * expected, None, torch.full((1,), expected, dtype=torch.float32, device=dev)
+        return state.learned, 1.0
+    return None, 1.0 if explicit is None else float(explicit)
 
 
 def _deliver_eager_grads(ctx, buffers, applied, state, g_loss):
-    """Backward of an eager-gradient op: ``buffers`` hold the gradients at scale ``applied`` (a
-    device scalar); returns them at the scale of ``g_loss``.  The first backward rescales the stored
-    buffers in place and hands them out; a later backward over a retained graph must not touch what
-    the first one handed out, so it scales copies."""
+    """Backward of an eager-gradient op: ``buffers`` hold the gradients at scale ``applied[0]`` (a
+    device scalar, followed by the counter of mrl_scale_rows_note); returns them at the scale of
+    ``g_loss``.  The first backward rescales the stored buffers in place and hands them out; a later
+    backward over a retained graph must not touch what the first one handed out, so it scales
+    copies.  An upstream gradient of 0, Inf or NaN cannot be undone: a later backward over the
+    same graph then yields NaN."""
     dev = buffers[0].device
     stream = _lib.stream(dev)
     upstream = g_loss.to(torch.float32).reshape(1).contiguous()
@@ -210,20 +193,111 @@ def _deliver_eager_grads(ctx, buffers, applied, state, g_loss):
     ctx.handed_out = True
     if not first:
         buffers = tuple(t.clone() for t in buffers)
-    for t in buffers:
-        flat = t.view(-1, t.shape[-1])
+        applied = applied.clone()
+    learned = _lib.ptr(state.learned) if state is not None else None
+    rescales = _lib.ptr(state.rescales) if state is not None else None
+    flats = [t.view(-1, t.shape[-1]) for t in buffers]
+    if len(flats) == 1 and flats[0].shape[0] > 0:
+        flat = flats[0]
+        _lib.call("mrl_scale_rows_note", _lib.ptr(flat), _lib.dtype_code(flat), flat.shape[0], flat.shape[1],
+                  flat.shape[1], _lib.ptr(upstream), _lib.ptr(applied), learned, rescales, stream)
+        return buffers
+    for flat in flats:
         _lib.call("mrl_scale_rows", _lib.ptr(flat), _lib.dtype_code(flat), flat.shape[0], flat.shape[1],
                   flat.shape[1], _lib.ptr(upstream), _lib.ptr(applied), stream)
     # the stored buffers now carry `upstream` (first backward) or still what they carried (copies)
-    _note_upstream(upstream, applied if first else applied.clone(), state, stream)
+    _lib.call("mrl_grad_scale_note", _lib.ptr(upstream), _lib.ptr(applied), learned, rescales, stream)
     return buffers
+
+
+def _align(n, to):
+    return (n + to - 1) // to * to
+
+
+class _FusedOperands:
+    """Device memory and normalised operands of one fused step, and its prepare / reduce launches.
+
+    Everything small lives in ONE allocation (window tables, per-sequence sums, the eight output
+    scalars, the gradient scale with its counter, the sweep's workspace) and the per-row operands and
+    terms in a second one; the kernels get addresses inside them."""
+
+    def __init__(self, dev, batch, cfg, n_rows, n_seq, width, layout, padded_s, sweep_dtype_code, vocab, sweep_rows):
+        lib = _lib.load()
+
+        def f32(t):
+            return None if t is None else t.to(dev).to(torch.float32).contiguous()
+
+        def idx(t):
+            if t is None:
+                return None
+            if t.dtype not in (torch.int32, torch.int64):
+                t = t.to(torch.int64)
+            return t.to(dev).reshape(-1).contiguous()
+
+        self.dev, self.cfg = dev, cfg
+        self.n_rows, self.n_seq, self.width, self.layout, self.padded_s = n_rows, n_seq, width, layout, padded_s
+        self.old, self.ref, self.adv = f32(batch.get("old_log_prob")), f32(cfg["ref_log_prob"]), f32(batch.get("advantages"))
+        self.mask_t, _ = _mask_args(cfg["mask"], batch["response_length"], dev)
+        self.prompt, self.resp = idx(batch["prompt_length"]), idx(batch["response_length"])
+        if layout == 0:
+            self.seqlens = cfg["seqlens"].to(dev).to(torch.int32).contiguous()
+            self.cu = cfg["cu"].to(dev).to(torch.int32).contiguous()
+        else:
+            self.seqlens = self.cu = None
+        self.mdt = _lib.dtype_code(self.mask_t) if self.mask_t is not None else _lib.F32
+        self.pdt, self.rdt = _lib.dtype_code(self.prompt), _lib.dtype_code(self.resp)
+        # the sweep's workspace is sized for the largest launch (a chunk, for the lm_head step)
+        # (at least its 16-byte header, whose second word the reduce step borrows as its counter)
+        self.ws_bytes = max(16, lib.mrl_fused_workspace_bytes(sweep_dtype_code, sweep_rows, vocab))
+        seqs = max(n_seq, 1)
+        o_out = 0                                   # float[8]
+        o_applied = 32                              # float[2]
+        o_ws = 48                                   # the sweep workspace, 16-byte aligned
+        o_start = _align(o_ws + self.ws_bytes, 16)  # int64[n_seq]
+        o_sums = o_start + 8 * seqs                 # float[n_seq * 8]
+        o_count = o_sums + 32 * seqs                # int32[n_seq]
+        o_msum = o_count + 4 * seqs                 # float[n_seq]
+        self.small = torch.empty(o_msum + 4 * seqs, dtype=torch.uint8, device=dev)
+        base = self.small.data_ptr()
+        self.out = self.small[o_out:o_out + 32].view(torch.float32)
+        self.applied = self.small[o_applied:o_applied + 8].view(torch.float32)
+        self.workspace = base + o_ws
+        self.p_start, self.p_sums, self.p_count, self.p_msum = base + o_start, base + o_sums, base + o_count, base + o_msum
+        self.rows = torch.empty(max(n_rows, 1) * 16, dtype=torch.float32, device=dev)
+        self.p_ops = self.rows.data_ptr()
+        self.p_terms = self.p_ops + max(n_rows, 1) * 32
+        self.loss = torch.empty((), dtype=torch.float32, device=dev)
+
+    def prepare(self, stream):
+        cfg = self.cfg
+        scale_dev, scale_host = _expected_scale(cfg)
+        _lib.call("mrl_fused_loss_prepare", self.layout, self.n_seq, self.width, self.n_rows, _lib.ptr(self.seqlens),
+                  _lib.ptr(self.cu), self.padded_s, _lib.ptr(self.prompt), self.pdt, _lib.ptr(self.resp), self.rdt,
+                  _lib.ptr(self.old), _lib.ptr(self.ref), _lib.ptr(self.adv), _lib.ptr(self.mask_t), self.mdt,
+                  cfg["seq_mean"], self.p_start, self.p_count, self.p_msum, self.p_ops,
+                  self.workspace if self.n_rows > 0 else None, self.ws_bytes if self.n_rows > 0 else 0,
+                  _lib.ptr(scale_dev), scale_host, _lib.ptr(self.applied) if self.n_rows > 0 else None, stream)
+        if self.n_rows == 0:
+            self.applied[0] = scale_host if scale_dev is None else scale_dev[0] * scale_host
+            self.applied[1] = 0.0
+
+    def reduce(self, stream, p_terms=None):
+        cfg = self.cfg
+        # word 1 of the cleared sweep workspace counts the workgroups of the reduce step
+        done = self.workspace + 4 if self.n_rows > 0 else None
+        _lib.call("mrl_fused_loss_reduce", self.p_terms if p_terms is None else p_terms, self.p_start, self.p_count,
+                  self.n_seq, self.width, _lib.ptr(self.old), _lib.ptr(self.ref), _lib.ptr(self.adv),
+                  _lib.ptr(self.mask_t), self.mdt, _lib.ptr(self.resp), self.rdt, cfg["clip_lo"], cfg["clip_hi"],
+                  cfg["kl_penalty"], cfg["kl_coef"], cfg["entropy_coeff"], cfg["seq_mean"], cfg["loss_scale"],
+                  self.p_sums, _lib.ptr(self.out), done, _lib.ptr(self.loss), stream)
 
 
 class _FusedLogprobLoss(torch.autograd.Function):
     """logits -> (loss, out[8]) with dlogits produced in the same sweep (one read, one write of
     the [T, V] tensor for forward + backward).  The backward only rescales the stored dlogits if
     the upstream gradient differs from the scale they already carry (kept in a device scalar, so
-    a second backward over a retained graph rescales by the ratio of the two upstream values)."""
+    a second backward over a retained graph rescales by the ratio of the two upstream values).
+    Three launches in the forward (prepare, sweep, reduce) and one in the backward."""
 
     @staticmethod
     def forward(ctx, output, labels, batch, cfg):
@@ -236,61 +310,25 @@ class _FusedLogprobLoss(torch.autograd.Function):
             lab = lab.to(torch.int64)
         lab = lab.contiguous()
         n_seq, width = batch["responses"].shape[0], batch["responses"].shape[-1]
-
-        def f32(t):
-            return None if t is None else t.to(dev).to(torch.float32).contiguous()
-
-        def idx(t):
-            if t is None:
-                return None
-            if t.dtype not in (torch.int32, torch.int64):
-                t = t.to(torch.int64)
-            return t.to(dev).reshape(-1).contiguous()
-
-        old, ref, adv = f32(batch.get("old_log_prob")), f32(cfg["ref_log_prob"]), f32(batch.get("advantages"))
-        mask_t, lens_t = _mask_args(cfg["mask"], batch["response_length"], dev)
-        prompt, resp = idx(batch["prompt_length"]), idx(batch["response_length"])
-        if cfg["packed"]:
-            layout, padded_s = 0, 0
-            seqlens = cfg["seqlens"].to(dev).to(torch.int32).contiguous()
-            cu = cfg["cu"].to(dev).to(torch.int32).contiguous()
-        else:
-            layout, padded_s = 1, output.shape[1]
-            seqlens = cu = None
-        row_start = torch.empty(n_seq, dtype=torch.int64, device=dev)
-        row_count = torch.empty(n_seq, dtype=torch.int32, device=dev)
-        seq_msum = torch.empty(n_seq, dtype=torch.float32, device=dev)
-        row_ops = torch.empty(n_rows * 8, dtype=torch.float32, device=dev)
-        row_terms = torch.empty(n_rows * 8, dtype=torch.float32, device=dev)
-        row_sums = torch.empty(max(n_seq, 1) * 8, dtype=torch.float32, device=dev)
-        out = torch.empty(8, dtype=torch.float32, device=dev)
+        layout, padded_s = (0, 0) if cfg["packed"] else (1, output.shape[1])
+        ops = _FusedOperands(dev, batch, cfg, n_rows, n_seq, width, layout, padded_s, _lib.dtype_code(flat), vocab,
+                             n_rows)
         ent = torch.empty(n_rows, dtype=torch.float32, device=dev) if cfg["entropy_coeff"] != 0 else None
         dlogits = flat if cfg["grad_inplace"] else torch.empty_like(flat)
         stream = _lib.stream(dev)
-        mdt = _lib.dtype_code(mask_t) if mask_t is not None else _lib.F32
-        pdt = _lib.dtype_code(prompt)
-        rdt = _lib.dtype_code(resp)
-        _lib.call("mrl_fused_loss_prepare", layout, n_seq, width, n_rows, _lib.ptr(seqlens), _lib.ptr(cu), padded_s,
-                  _lib.ptr(prompt), pdt, _lib.ptr(resp), rdt, _lib.ptr(old), _lib.ptr(ref), _lib.ptr(adv),
-                  _lib.ptr(mask_t), mdt, cfg["seq_mean"], _lib.ptr(row_start), _lib.ptr(row_count),
-                  _lib.ptr(seq_msum), _lib.ptr(row_ops), stream)
-        grad_scale, scale_dev, applied = _expected_scale(cfg, dev)
-        workspace, ws_bytes = _sweep_workspace(flat)
+        ops.prepare(stream)
         vocab_ops._timed_call("mrl_fused_logprob_loss", n_rows, dev, _lib.ptr(flat), _lib.dtype_code(flat), n_rows,
                               vocab, vocab, _lib.ptr(lab), _lib.dtype_code(lab), cfg["inv_temperature"],
-                              _lib.ptr(row_ops), 0 if old is None else 1, cfg["clip_lo"], cfg["clip_hi"],
-                              cfg["kl_penalty"], cfg["kl_coef"], cfg["entropy_coeff"], grad_scale,
-                              _lib.ptr(scale_dev), _lib.ptr(dlogits), vocab, None, _lib.ptr(ent), _lib.ptr(row_terms),
-                              _lib.ptr(workspace), ws_bytes, stream)
-        _lib.call("mrl_fused_loss_reduce", _lib.ptr(row_terms), _lib.ptr(row_start), _lib.ptr(row_count), n_seq, width,
-                  _lib.ptr(old), _lib.ptr(ref), _lib.ptr(adv), _lib.ptr(mask_t), mdt, _lib.ptr(resp), rdt,
-                  cfg["clip_lo"], cfg["clip_hi"], cfg["kl_penalty"], cfg["kl_coef"], cfg["entropy_coeff"],
-                  cfg["seq_mean"], cfg["loss_scale"], _lib.ptr(row_sums), _lib.ptr(out), stream)
-        ctx.save_for_backward(dlogits, applied)
+                              ops.p_ops, 0 if ops.old is None else 1, cfg["clip_lo"], cfg["clip_hi"],
+                              cfg["kl_penalty"], cfg["kl_coef"], cfg["entropy_coeff"], cfg["loss_scale"],
+                              _lib.ptr(ops.applied), _lib.ptr(dlogits), vocab, None, _lib.ptr(ent), ops.p_terms,
+                              ops.workspace, ops.ws_bytes, 1, stream)
+        ops.reduce(stream)
+        ctx.save_for_backward(dlogits, ops.applied)
         ctx.meta = (tuple(output.shape), cfg.get("scale_state"))
         ctx.handed_out = False
-        ctx.mark_non_differentiable(out)
-        return out[0].clone(), out
+        ctx.mark_non_differentiable(ops.out)
+        return ops.loss, ops.out
 
     @staticmethod
     def backward(ctx, g_loss, _g_out):

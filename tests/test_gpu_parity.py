@@ -1118,6 +1118,19 @@ def test_fused_sweep_vocab_sizes(dev, dtype, vocab):
         assert abs(got_stats[k] - want_stats[k]) <= TOL_LOSS_REL * abs(want_stats[k]) + 1e-6, k
     assert (dz.float().cpu() - dz_o).abs().max().item() < TOL_DLOGITS
     assert (dz.float().cpu() - dz_o).abs().max().item() <= 2 ** -8 * dz_o.abs().max().item() + 1e-9
+    # the gradient written over the logits, and - for rows that two workgroups hold - without ever waiting
+    # for the other half's record (every workgroup reads the other half itself): the same bits
+    lib = _lib.load()
+    for limit in (-1, 0):
+        lib.mrl_set_wide_spin_limit(limit)
+        try:
+            z2 = logits.to(dev).requires_grad_()
+            z_in = z2 * 1.0
+            got2, _ = f.compute_loss(z_in, _to_dev(b, dev), fused=True, grad_inplace=True, **_to_dev(kw, dev))
+            (dz2,) = torch.autograd.grad(got2, z2)
+        finally:
+            lib.mrl_set_wide_spin_limit(-1)
+        assert got2.item() == got.item() and torch.equal(dz2, dz), limit
 
 
 @pytest.mark.parametrize("dtype,vocab", [(torch.float32, 152064), (torch.bfloat16, 262144)])
@@ -1155,7 +1168,7 @@ def test_fused_sweep_wide_rows(dev, dtype, vocab):
         dz, ent, terms = out
         _lib.call("mrl_fused_logprob_loss", z.data_ptr(), _lib.dtype_code(z), rows, vocab, vocab, y.data_ptr(),
                   _lib.I64, 1.0, ops.data_ptr(), 1, 0.8, 1.2, 3, 0.01, 0.002, 1.0, None, dz.data_ptr(), vocab, None,
-                  ent.data_ptr(), terms.data_ptr(), ws.data_ptr(), ws_bytes, stream)
+                  ent.data_ptr(), terms.data_ptr(), ws.data_ptr(), ws_bytes, 0, stream)
 
     spaces = [torch.full((ws_bytes,), 0xCD, dtype=torch.uint8, device=dev) for _ in range(3)]
     want = []
@@ -1202,6 +1215,25 @@ def test_fused_sweep_wide_rows(dev, dtype, vocab):
     for got, ref in zip(outs, want):
         for a, b in zip(got, ref):
             assert torch.equal(a, b)
+    # in place (the gradients overwrite the logits while other workgroups still exchange statistics), and
+    # with a wait bound of zero polls: every workgroup then reads the other half of its row itself and
+    # looks for the record only afterwards - out of place and in place, the same bits as above
+    for limit, inplace in ((-1, True), (0, False), (0, True)):
+        lib.mrl_set_wide_spin_limit(limit)
+        try:
+            for case, ref in zip(cases, want):
+                z, y, ops = case
+                dz, ent, terms = outputs()
+                if inplace:
+                    dz.copy_(z)
+                    sweep((dz, y, ops), (dz, ent, terms), spaces[0], _lib.stream(dev))
+                else:
+                    sweep(case, (dz, ent, terms), spaces[0], _lib.stream(dev))
+                torch.cuda.synchronize()
+                for a, b in zip((dz, ent, terms), ref):
+                    assert torch.equal(a, b), (limit, inplace)
+        finally:
+            lib.mrl_set_wide_spin_limit(-1)
     # captured once, replayed next to an eager sweep
     g_out = outputs()
     graph = torch.cuda.CUDAGraph()
@@ -1539,7 +1571,7 @@ def _raw_fused_sweep(z, y, row_ops, dz, ent, terms, stream, ticket=None, scale_d
     rows, vocab = z.shape
     _lib.call("mrl_fused_logprob_loss", z.data_ptr(), _lib.dtype_code(z), rows, vocab, vocab, y.data_ptr(), _lib.I64,
               1.0, row_ops.data_ptr(), 1, 0.8, 1.2, 3, 0.01, 0.002, 1.0, _lib.ptr(scale_dev), dz.data_ptr(), vocab,
-              None, ent.data_ptr(), terms.data_ptr(), _lib.ptr(ticket), 0 if ticket is None else 16, stream)
+              None, ent.data_ptr(), terms.data_ptr(), _lib.ptr(ticket), 0 if ticket is None else 16, 0, stream)
 
 
 def _raw_fused_case(dev, seed, rows, vocab):
@@ -1558,10 +1590,10 @@ def _raw_fused_case(dev, seed, rows, vocab):
 
 def test_fused_sweep_on_two_streams_and_in_a_graph(dev):
     """The persistent sweep hands out rows through a counter that the caller owns and that a launch
-    resets on its own stream: two sweeps in flight on two streams (a counter each), a sweep without a
-    counter (fixed row stride) and a captured sweep replayed several times next to eager sweeps (the
-    reset is a kernel, so it is part of the graph, and the graph keeps its own counter) give the
-    results of a lone eager call, bit for bit - every row's result is independent of the order in
+    clears on its own stream: two sweeps in flight on two streams (a counter each), a sweep without a
+    counter (one workgroup per row) and a captured sweep replayed several times next to eager sweeps
+    (the clearing is a kernel, so it is part of the graph, and the graph keeps its own counter) give
+    the results of a lone eager call, bit for bit - every row's result is independent of the order in
     which rows are taken."""
     rows, vocab = 1500, 8200
     cases = [_raw_fused_case(dev, 50 + i, rows, vocab) for i in range(2)]
@@ -1573,10 +1605,10 @@ def test_fused_sweep_on_two_streams_and_in_a_graph(dev):
         torch.cuda.synchronize()
         want.append((dz, ent, terms))
         assert dz.float().abs().max().item() > 0 and not dz[ops[:, 3] == 0].any().item()
-        # every row was handed out exactly once: the counter ends at rows + workgroups
-        cus = torch.cuda.get_device_properties(dev).multi_processor_count
-        assert int(tickets[0][0].item()) == rows + cus
-    # no counter: rows are walked with a fixed stride
+        # every row was handed out exactly once: the workgroups start on the first rows, ticket t stands
+        # for row t + workgroups, and each workgroup draws one ticket too many
+        assert int(tickets[0][0].item()) == rows
+    # no counter: one workgroup per row
     z, y, ops = cases[0]
     plain = (torch.empty_like(z), torch.empty(rows, device=dev), torch.empty(rows, 8, device=dev))
     _raw_fused_sweep(z, y, ops, *plain, _lib.stream(dev), None)
@@ -1594,7 +1626,7 @@ def test_fused_sweep_on_two_streams_and_in_a_graph(dev):
     for got, ref in zip(outs, want):
         for a, b in zip(got, ref):
             assert torch.equal(a, b)
-    # many launches in a row on one stream may share one counter (each resets it behind the previous sweep)
+    # many launches in a row on one stream may share one counter (each clears it behind the previous sweep)
     for _ in range(300):
         _raw_fused_sweep(cases[0][0], cases[0][1], cases[0][2], *outs[0], _lib.stream(dev), tickets[0])
     torch.cuda.synchronize()
@@ -1909,7 +1941,7 @@ def _random_fused_case(i, rnd):
     ent = torch.zeros(rows, device=dev)
     lp = torch.zeros(rows, device=dev)
     terms = torch.zeros(rows, 8, device=dev)
-    # every other narrow case walks rows with a fixed stride (no workspace); wide rows need theirs
+    # every other narrow case gets no workspace (one workgroup per row whatever the batch); wide rows need theirs
     ws_bytes = _lib.load().mrl_fused_workspace_bytes(_lib.dtype_code(z), rows, vocab)
     assert ws_bytes >= 16
     workspace = torch.full((ws_bytes,), 0xAB, dtype=torch.uint8, device=dev) if (i % 2 == 0 or ws_bytes > 16) else None
@@ -1917,7 +1949,7 @@ def _random_fused_case(i, rnd):
     _lib.call("mrl_fused_logprob_loss", z.data_ptr(), _lib.dtype_code(z), rows, vocab, vocab, y.data_ptr(), _lib.I64,
               inv_t, ops.data_ptr(), 1, clip_lo, clip_hi, kl_kind, kl_coef, ent_c, 1.0, None, dz.data_ptr(), vocab,
               lp.data_ptr(), ent.data_ptr() if ent_c != 0 else None, terms.data_ptr(),
-              _lib.ptr(workspace), ws_bytes if workspace is not None else 0, _lib.stream(dev))
+              _lib.ptr(workspace), ws_bytes if workspace is not None else 0, 0, _lib.stream(dev))
     zr = (z.float() * inv_t).requires_grad_()
     logsm = torch.log_softmax(zr, -1)
     y_ok = (y >= 0) & (y < vocab)
@@ -2902,35 +2934,3 @@ def test_vocabulary_shards_merge_to_the_full_sweep(dev, dtype, bounds):
     assert not dz[5].any().item()
     # a label outside every shard: the oracle (Megatron's target mask) scores the row maximum there,
     # a sharded run scores 0 - documented difference, no rank owns such a label
-
-
-@pytest.mark.parametrize("switches,subset", [
-    ({"MRL_SWEEP_PERSISTENT": "0", "MRL_BWD_CHUNK": "0"},
-     "test_persistent_row_sweeps or test_fused_sweep_persistent or test_backward_fp32_full_vocab or "
-     "test_fused_sweep_random_shapes or test_split_sweeps_random_shapes or test_vocab_forward_backward_parity"),
-    ({"MRL_LMHEAD_V2": "0", "MRL_SWEEP_TICKET": "0"},
-     "test_lmhead_logprob_forward or test_lmhead_forward_random_shapes or test_fused_lmhead_policy_loss or "
-     "test_fused_sweep_persistent or test_persistent_row_sweeps"),
-    # no waiting at all for the other half of a wide row: every workgroup computes the other half's
-    # statistics itself from memory (the path a workgroup takes when its partner is late)
-    ({"MRL_WIDE_SPIN_LIMIT": "0"}, "test_fused_sweep_wide_rows or test_fused_sweep_vocab_sizes or "
-                                   "test_fused_sweep_random_shapes"),
-], ids=["per_row_sweep_and_loop_backward", "first_lmhead_loop_and_fixed_stride", "wide_rows_without_waiting"])
-def test_library_switches_in_child_processes(dev, switches, subset):
-    """The library reads its tuning switches once per process, so the kernels behind them (one workgroup
-    per row instead of persistent workgroups, the loop backward for every row length, the first
-    lm_head tile loop, the fixed row stride) cannot be reached from this process: a child process per
-    switch set runs the parity tests that cover those kernels at the sizes where the switch matters."""
-    import subprocess
-    import sys
-    env = dict(os.environ, **switches)
-    here = os.path.abspath(__file__)
-    assert "MRL_CHILD_OF_SWITCH_TEST" not in os.environ, "a child process must not start children of its own"
-    env["MRL_CHILD_OF_SWITCH_TEST"] = "1"
-    subset = "(%s) and not child_processes" % subset
-    proc = subprocess.run([sys.executable, "-m", "pytest", here, "-x", "-q", "-m", "gpu", "-k", subset,
-                           "-p", "no:cacheprovider"],
-                          env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=280)
-    tail = "\n".join(proc.stdout.splitlines()[-15:])
-    assert proc.returncode == 0, tail
-    assert " passed" in tail and "failed" not in tail, tail

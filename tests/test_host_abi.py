@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), "libmrl_hip.so lacks %s" % name
     # and the ctypes table binds exactly the declared set
     assert sorted(_lib.SIGNATURES) == declared
-    assert lib.mrl_version() == 201
+    assert lib.mrl_version() == 300
     assert lib.mrl_last_error() == b""
     assert os.path.dirname(_lib.library_path()).startswith(ROOT), "the library must live in-tree"
 
@@ -105,24 +105,34 @@ def test_argument_validation_launches_nothing():
     assert lib.mrl_fused_workspace_bytes(_lib.BF16, 100, 152064) == 16
     assert lib.mrl_fused_workspace_bytes(_lib.F32, 100, 152064) == 16 + 100 * 32
     assert lib.mrl_fused_workspace_bytes(_lib.BF16, 100, 311304) == 0
-    # a row that two workgroups hold needs the workspace, and cannot be swept in place
+    # a row that two workgroups hold needs the workspace
     rc = lib.mrl_fused_logprob_loss(p, _lib.F32, 2, 152064, 152064, p, _lib.I64, 1.0, p, 1, 0.8, 1.2, 4, 0.0, 0.0, 1.0,
-                                    None, p + (1 << 30), 152064, None, None, p, None, 0, None)
+                                    None, p + (1 << 30), 152064, None, None, p, None, 0, 0, None)
     assert rc == -1 and b"workspace" in lib.mrl_last_error()
     rc = lib.mrl_fused_logprob_loss(p, _lib.F32, 2, 152064, 152064, p, _lib.I64, 1.0, p, 1, 0.8, 1.2, 4, 0.0, 0.0, 1.0,
-                                    None, p, 152064, None, None, p, p, 1 << 20, None)
-    assert rc == -2 and b"in place" in lib.mrl_last_error()
+                                    None, p, 152064, None, None, p, p, 64, 0, None)
+    assert rc == -1 and b"workspace" in lib.mrl_last_error()                              # too small for two rows
     for vocab in (311304, 1003):
         rc = lib.mrl_fused_logprob_loss(p, _lib.BF16, 2, vocab, vocab, p, _lib.I64, 1.0, p, 1, 0.8, 1.2, 4, 0.0, 0.0,
-                                        1.0, None, p, vocab, None, None, p, None, 0, None)
+                                        1.0, None, p, vocab, None, None, p, None, 0, 0, None)
         assert rc == -2, vocab
     assert lib.mrl_fused_logprob_loss(p, _lib.BF16, 2, 64, 64, p, _lib.I64, 1.0, None, 1, 0.8, 1.2, 4, 0.0, 0.0, 1.0,
-                                      None, p, 64, None, None, p, None, 0, None) == -1    # no row operands
+                                      None, p, 64, None, None, p, None, 0, 0, None) == -1  # no row operands
     assert lib.mrl_fused_logprob_loss(p, _lib.BF16, 2, 64, 64, p, _lib.I64, 1.0, p, 1, 0.8, 1.2, 4, 0.0, 0.0, 1.0,
-                                      None, p, 64, None, None, p, p + 2, 16, None) == -3  # misaligned workspace
+                                      None, p, 64, None, None, p, p + 2, 16, 0, None) == -3  # misaligned workspace
     assert lib.mrl_scale_rows(p, _lib.I32, 2, 64, 64, p, p, None) == -2
     assert lib.mrl_scale_rows(p, _lib.BF16, 2, 64, 64, p, None, None) == -1                # no applied scale
     assert lib.mrl_grad_scale_note(p, None, None, None, None) == -1
+    assert lib.mrl_scale_rows_note(p, _lib.BF16, 2, 64, 64, p, None, None, None, None) == -1
+    assert lib.mrl_scale_rows_note(p, _lib.BF16, 2, 64, 64, p, p + 4, None, None, None) == -3   # scale + counter: 8 bytes
+    # the prepare step clears the sweep's workspace in whole 8-byte words
+    assert lib.mrl_fused_loss_prepare(0, 0, 4, 8, None, None, 0, None, 0, None, 0, None, None, None, None, 0, 0, None,
+                                      None, None, p, p, 12, None, 1.0, None, None) == -1
+    assert lib.mrl_fused_loss_prepare(0, 0, 4, 0, None, None, 0, None, 0, None, 0, None, None, None, None, 0, 0, None,
+                                      None, None, None, p, 16, None, 1.0, None, None) == -1     # nothing to prepare for
+    # the bound of the wide rows' wait: set, read back, restore
+    assert lib.mrl_set_wide_spin_limit(0) == 1 << 18 and lib.mrl_set_wide_spin_limit(-1) == 0
+    assert lib.mrl_set_wide_spin_limit(-1) == 1 << 18
     # fused lm_head: hidden size must be a multiple of the K tile, workspace must be large enough
     assert lib.mrl_lmhead_workspace_bytes(100, 1000) > 0
     assert lib.mrl_lmhead_logprob_fwd(p, p, 4, 1000, 100, p, _lib.I64, 1.0, p, None, None, p, 1 << 20, None) != 0
