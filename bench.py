@@ -1,19 +1,24 @@
 #!/usr/bin/env python3
 """Benchmark of the actor log-prob + GRPO loss hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c0|c2|c4chunk|c3|c3fwd]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|c1|c0|c2|c4|c4chunk|c3|c3fwd]
 
 One step = one pass of the path over one synthetic packed batch resident in HBM: the fused
 vocabulary sweep (log-prob + entropy + logsumexp), the unpack to [B, L], the fused policy loss
-with its five statistics (one device-to-host copy), and the backward down to dlogits.  Default
-workload is the Qwen2.5-7B-shaped GRPO actor step: 16 prompts x 8 responses, response lengths
+with its five statistics (one device-to-host copy), and the backward down to dlogits.  The
+headline workload is the Qwen2.5-7B-shaped GRPO actor step: 16 prompts x 8 responses, response lengths
 uniform in [512, 2048] (about 164k packed rows), vocabulary 152064, bf16 logits ~N(0, 3), labels
 drawn from softmax(logits), clip 0.2, k3 KL 0.001, token-mean loss.
 
 Prints ONE JSON line: tokens/s for the whole step, the roofline of the dominant kernel (the
-backward sweep) from HIP events recorded on the launch stream inside the timed region, and a CPU
+sweep) from HIP events recorded on the launch stream inside the timed region, and a CPU
 baseline: the oracle's restatement of the reference's torch op chain, timed on this host's cores
-on a bounded row sample of the same workload.
+on a bounded row sample of the same workload.  Without --workload (or with --workload all) the
+same line carries, under "other_workloads", a few steps of every other configuration: the
+CPU-sized batch (c0), the padded layout (c2), the whole long-response DAPO batch in token-budget
+micro-batches (c4), fp32 logits, an upstream gradient the loss object is not told (upstream0.25)
+and the lm_head forward and training step (c3fwd, c3); the headline keys stay those of the
+headline workload.
 """
 import argparse
 import json
@@ -48,9 +53,14 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS) + ["c3fwd", "c3"],
-                    help="c3fwd: the fused lm_head + log-prob forward of configs[3] (bf16 MFMA, logits never stored); "
+    ap.add_argument("--workload", default="all", choices=["all"] + sorted(WORKLOADS) + ["c4", "c3fwd", "c3"],
+                    help="all: the headline (c1) plus a few steps of every other workload under 'other_workloads'; "
+                         "c4: configs[4] whole - 8x16 long responses, dynamic-sampling filter, 64k-token micro-batches; "
+                         "c3fwd: the fused lm_head + log-prob forward of configs[3] (bf16 MFMA, logits never stored); "
                          "c3: configs[3] forward + backward from the hidden states (per chunk: logits product -> fused sweep -> dHidden and dW products)")
+    ap.add_argument("--token-budget", type=int, default=65536,
+                    help="c4 only: token budget of a micro-batch (configs[4]: 64k-token chunks)")
+    ap.add_argument("--other-steps", type=int, default=3, help="steps of each entry of other_workloads")
     ap.add_argument("--tokens", type=int, default=163840, help="rows of the c3fwd workload")
     ap.add_argument("--entropy-coeff", type=float, default=0.001,
                     help="non-zero so that the forward computes entropy and the backward its gradient")
@@ -231,7 +241,7 @@ def cpu_baseline(torch, w, rows_target, entropy_coeff, seed, mrl=None, dev=None,
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 
-def run_lmhead(args):
+def run_lmhead(args, steps=None, warmup=None):
     """configs[3], forward part: hidden [T, 3584] ~N(0,1), W [152064, 3584] ~N(0,0.02), bf16; one step =
     log-prob + entropy + logsumexp of every token without materialising the logits."""
     import torch
@@ -239,17 +249,19 @@ def run_lmhead(args):
     from mindspeed_rl_amd import lmhead
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    steps = args.steps if steps is None else steps
+    warmup = args.warmup if warmup is None else warmup
     tokens, vocab, hdim = args.tokens, 152064, 3584
     g = torch.Generator(device=dev).manual_seed(args.seed)
     hidden = torch.randn(tokens, hdim, generator=g, device=dev).to(torch.bfloat16)
     weight = (torch.randn(vocab, hdim, generator=g, device=dev) * 0.02).to(torch.bfloat16)
     labels = torch.randint(0, vocab, (tokens,), generator=g, device=dev)
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         mrl.lmhead_logprob(hidden, weight, labels)
     torch.cuda.synchronize()
     lmhead.kernel_events = []
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         lp, ent, lse = mrl.lmhead_logprob(hidden, weight, labels)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
@@ -262,20 +274,20 @@ def run_lmhead(args):
     err = (lp[:256] - ref.gather(-1, labels[:256, None]).squeeze(-1)).abs().max().item()
     result = {
         "metric": "tokens/sec for fused lm_head+logprob forward; MFMA TFLOP/s as % of bf16 dense peak",
-        "value": tokens / (elapsed / args.steps), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": elapsed * 1e3 / args.steps, "higher_is_better": True, "scaling": "weak",
+        "value": tokens / (elapsed / steps), "unit": "tokens/s", "n_gpus": 1, "steps": steps,
+        "warmup": warmup, "ms_per_step": elapsed * 1e3 / steps, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "configs[3] forward: hidden [%d,3584] x W [152064,3584]^T, online logsumexp, logits never "
                                "stored" % tokens, "accumulate": "f32"},
-        "roofline": {"kernel": "lmhead_fwd_kernel_v2 + lmhead_finish_kernel (mrl_lmhead_logprob_fwd)", "bound": "mfma",
+        "roofline": {"kernel": "lmhead_fwd_kernel + lmhead_finish_kernel (mrl_lmhead_logprob_fwd)", "bound": "mfma",
                      "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "flops_per_launch": flops, "avg_ms": ms},
         "max_abs_err_vs_fp32_gemm_256_rows": err,
     }
-    print(json.dumps(result), flush=True)
+    return result
 
 
-def run_lmhead_train(args):
+def run_lmhead_train(args, steps=None, warmup=None):
     """configs[3]: GRPO loss as in configs[1] but from hidden [T, 3584] and W [152064, 3584]; backward yields
     dHidden and dW.  Logits exist for --chunk-rows rows at a time."""
     import torch
@@ -283,6 +295,8 @@ def run_lmhead_train(args):
     from mindspeed_rl_amd import vocab_ops
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    steps = args.steps if steps is None else steps
+    warmup = args.warmup if warmup is None else warmup
     w = WORKLOADS["c1"]
     vocab, hdim = w["vocab"], 3584
     plen, rlen, rewards = make_lengths(torch, w, args.seed)
@@ -319,22 +333,22 @@ def run_lmhead_train(args):
         return loss, stats, dh, dw
 
     from mindspeed_rl_amd import lmhead
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     vocab_ops.kernel_events = []
     lmhead.kernel_events = []
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         loss, stats, dh, dw = step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     events, vocab_ops.kernel_events = vocab_ops.kernel_events, None
     gemm_events, lmhead.kernel_events = lmhead.kernel_events, None
-    sweep_ms = sum(s.elapsed_time(e) for (_, s, e, _) in events) / args.steps
-    logits_ms = sum(s.elapsed_time(e) for (n, s, e, _) in gemm_events if n == "mrl_lmhead_logits") / args.steps
-    bwd_ms = sum(s.elapsed_time(e) for (n, s, e, _) in gemm_events if n == "mrl_lmhead_logprob_bwd") / args.steps
-    ms = elapsed * 1e3 / args.steps
+    sweep_ms = sum(s.elapsed_time(e) for (_, s, e, _) in events) / steps
+    logits_ms = sum(s.elapsed_time(e) for (n, s, e, _) in gemm_events if n == "mrl_lmhead_logits") / steps
+    bwd_ms = sum(s.elapsed_time(e) for (n, s, e, _) in gemm_events if n == "mrl_lmhead_logprob_bwd") / steps
+    ms = elapsed * 1e3 / steps
     flops = 6.0 * total * vocab * hdim                       # forward GEMM + dHidden GEMM + dW GEMM
     tflops = flops / (ms * 1e-3) / 1e12
     del dh, dw
@@ -367,7 +381,7 @@ def run_lmhead_train(args):
     del z, w_hv, dh_c, dw32, h_t
     result = {
         "metric": "tokens/sec for fused lm_head + logprob + GRPO loss fwd+bwd (dHidden, dW); TFLOP/s as % of bf16 dense peak",
-        "value": tokens / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": tokens / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "configs[3]: hidden [%d,3584] x W [152064,3584], GRPO loss as configs[1], logits only for "
@@ -385,7 +399,7 @@ def run_lmhead_train(args):
             "hand_written_products_ms_per_step": logits_ms + bwd_ms},
         "loss": float(loss.detach()), "stats": stats[1:6],
     }
-    print(json.dumps(result), flush=True)
+    return result
 
 
 # HBM bytes per launch of the dominant kernel.  Not measured by this run: the figure comes from the
@@ -402,38 +416,43 @@ PROFILED_TRAFFIC = {
 }
 
 
-def _profiled_traffic(args, w, dominant):
+def _profiled_traffic(args, workload, w, path, dominant):
     """(bytes or None, where the figure comes from)."""
     if args.entropy_coeff != 0.001 or any(k.startswith("MRL_") for k in os.environ):
         return None, None
-    return PROFILED_TRAFFIC.get((args.workload, w["dtype"], args.path, dominant), (None, None))
+    return PROFILED_TRAFFIC.get((workload, w["dtype"], path, dominant), (None, None))
 
 
-def main():
-    args = parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build measures one GPU only (no collectives exist on this path); "
-              "run with --gpus 1", file=sys.stderr)
-        sys.exit(2)
+def _median(xs):
+    xs = sorted(xs)
+    return xs[len(xs) // 2] if len(xs) % 2 else 0.5 * (xs[len(xs) // 2 - 1] + xs[len(xs) // 2])
+
+
+def _release(torch):
+    import gc
+    gc.collect()
+    torch.cuda.empty_cache()
+
+
+def run_sweep(args, workload, dtype=None, upstream=1.0, path=None, steps=None, warmup=None, probes=True, cpu=True,
+              flush=False):
+    """One of the logits workloads (c1, c2, c0, c4chunk) through a loss object: K timed steps bracketed by
+    synchronisations, HIP events around every step (median) and around every vocabulary sweep.
+    flush: a 1 GiB buffer is rewritten between the steps, outside the per-step events, so that a working
+    set smaller than the last-level cache is read from HBM; the step time is then the median of the
+    per-step events."""
     import torch
     import mindspeed_rl_amd as mrl
     from mindspeed_rl_amd import _lib, vocab_ops
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(1)
-    _lib.load()
-    if args.workload == "c3fwd":
-        run_lmhead(args)
-        return
-    if args.workload == "c3":
-        run_lmhead_train(args)
-        return
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    w = dict(WORKLOADS[args.workload])
-    if args.dtype is not None and args.dtype != w["dtype"]:
-        w["dtype"] = args.dtype
-        w["desc"] += " [logits as %s]" % args.dtype
+    steps = args.steps if steps is None else steps
+    warmup = args.warmup if warmup is None else warmup
+    path = args.path if path is None else path
+    w = dict(WORKLOADS[workload])
+    if dtype is not None and dtype != w["dtype"]:
+        w["dtype"] = dtype
+        w["desc"] += " [logits as %s]" % dtype
     plen, rlen, rewards = make_lengths(torch, w, args.seed)
     logits, b, kw, total = build_device_batch(torch, mrl, w, plen, rlen, rewards, dev, args.seed)
     tokens = int(rlen.sum())
@@ -449,28 +468,42 @@ def main():
         f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.001),
                               "kl_penalty": "low_var_kl", "entropy_coeff": args.entropy_coeff})
 
+    # the root gradient autograd starts from, made once: torch would otherwise fill a ones tensor per step
+    root = torch.full((), float(upstream), dtype=torch.float32, device=dev)
+
     def step():
         z = logits.detach().requires_grad_()
-        loss, stats = f.compute_loss(z, b, fused=(args.path == "fused"), **kw)
-        (dz,) = torch.autograd.grad(loss if args.upstream == 1.0 else loss * args.upstream, z)
+        loss, stats = f.compute_loss(z, b, fused=(path == "fused"), **kw)
+        (dz,) = torch.autograd.grad(loss, z, grad_outputs=root)
         return loss, stats, dz
 
+    scrub = torch.empty(1 << 30, dtype=torch.uint8, device=dev) if flush else None
     rescales = f.grad_scale_state(dev).rescales
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     rescales_before = int(rescales.item())
     vocab_ops.kernel_events = []
     dz = None
+    step_events = []
+    stream = torch.cuda.current_stream(dev)
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         del dz                      # the previous gradient is released before the next one is allocated
+        if flush:
+            scrub.fill_(1)
+            torch.cuda.synchronize()
+        s_ev, e_ev = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s_ev.record(stream)
         loss, stats, dz = step()
+        e_ev.record(stream)
+        step_events.append((s_ev, e_ev))
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     events = vocab_ops.kernel_events
     vocab_ops.kernel_events = None
-    ms_per_step = elapsed * 1e3 / args.steps
+    step_ms = [s_ev.elapsed_time(e_ev) for s_ev, e_ev in step_events]
+    ms_per_step = _median(step_ms) if flush else elapsed * 1e3 / steps
 
     def avg_ms(name):
         ts = [s.elapsed_time(e) for (n, s, e, _) in events if n == name]
@@ -489,8 +522,8 @@ def main():
     # the kernel each entry point dispatches to for this shape (csrc/row_sweep.hip, csrc/vocab_logprob.hip)
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     wide = row_bytes > 19 * 1024 * 16                      # a row that two workgroups hold
-    persistent = wide or (os.environ.get("MRL_SWEEP_PERSISTENT", "1") != "0" and total > 2 * cus)
-    chunked = os.environ.get("MRL_BWD_CHUNK", "1") != "0" and row_bytes >= 16384 and row_bytes % 16 == 0
+    persistent = wide or total > 2 * cus
+    chunked = row_bytes >= 16384 and row_bytes % 16 == 0
     kernel_symbol = {"mrl_vocab_logprob_fwd": "vocab_fwd_kernel",
                      "mrl_vocab_logprob_bwd": "bwd_chunk_kernel" if chunked else "vocab_bwd_kernel",
                      "mrl_fused_logprob_loss": ("fused_sweep_persistent_kernel" + (" (half rows)" if wide else ""))
@@ -509,15 +542,15 @@ def main():
     # path needs only 2 of them, so the same step is also quoted against that 3-pass byte count
     three_pass_bytes = total * row_bytes + live_rows * 2 * row_bytes + dead_rows * row_bytes
     three_pass_gbps = three_pass_bytes / (ms_per_step * 1e-3) / 1e9
-    traffic, traffic_source = _profiled_traffic(args, w, dominant)
+    traffic, traffic_source = _profiled_traffic(args, workload, w, path, dominant)
 
     result = {
         "metric": "tokens/sec for logprob+GRPO loss fwd+bwd; achieved HBM GB/s as % of peak",
         "value": tokens / (ms_per_step * 1e-3),
         "unit": "tokens/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
+        "steps": steps,
+        "warmup": warmup,
         "ms_per_step": ms_per_step,
         "higher_is_better": True,
         "scaling": "weak",
@@ -528,9 +561,10 @@ def main():
             "workload": w["desc"], "responses": int(plen.shape[0]), "layout": w.get("layout", "packed"),
             "packed_rows": total, "response_tokens": tokens,
             "vocab": vocab, "accumulate": "f32", "loss_kind": w.get("loss", "grpo: clip 0.2, low_var_kl 0.001"),
-            "entropy_coeff": args.entropy_coeff, "loss": "token-mean", "path": args.path,
-            # the scalar the step multiplies the loss by before backward(); the loss object is not told
-            "upstream": args.upstream,
+            "entropy_coeff": args.entropy_coeff, "loss": "token-mean", "path": path,
+            # the scalar autograd starts the backward from; the loss object is not told
+            "upstream": upstream,
+            "caches_flushed_between_steps": bool(flush),
         },
         "roofline": {
             "kernel": "%s (%s)" % (kernels[dominant]["symbol"], dominant), "bound": "hbm",
@@ -539,18 +573,34 @@ def main():
             "traffic_source": {"measured_this_run": False, "from_committed_profile": traffic_source},
             "bytes_per_launch": kernels[dominant]["bytes_per_launch"], "avg_ms": kernels[dominant]["avg_ms"],
         },
+        "ms_per_step_median": _median(step_ms),
+        "ms_per_step_mean_wall": elapsed * 1e3 / steps,
         "kernels": kernels,
         "step_hbm": {"GBps": step_gbps, "frac": step_gbps / HBM_PEAK_GBPS, "algorithmic_bytes_per_step": step_bytes},
         # NOT a roofline fraction: the step's time applied to the bytes a 3-pass (read, read, write)
         # implementation would move, so that the fused and the split path can be compared on one denominator
         "comparison_on_three_pass_bytes": {"bytes": three_pass_bytes, "equivalent_GBps": three_pass_gbps},
-        "rescale_passes_in_timed_steps": int(rescales.item()) - rescales_before if args.path == "fused" else None,
+        "rescale_passes_in_timed_steps": int(rescales.item()) - rescales_before if path == "fused" else None,
         "stats": {k: float(v) for k, v in stats.items()},
         "loss": float(loss.detach()),
     }
-    # practical ceilings on this box: with the sweeps' access pattern (one workgroup per 152064-entry bf16
-    # row) and with the pattern the HBM system serves best (one vector per thread, small workgroups)
-    del dz
+    del dz, scrub, logits, b
+    _release(torch)
+    if probes:
+        result["measured_ceiling"] = bandwidth_ceilings(torch, _lib, dev)
+        # a read+write stream of R read bytes and W written bytes cannot beat R/read + W/write on this box
+        best_copy = max(result["measured_ceiling"]["copy_GBps"], result["measured_ceiling"]["stream_copy_GBps"])
+        for k in kernels.values():
+            k["frac_of_measured_copy"] = k["GBps"] / best_copy
+        result["roofline"]["frac_of_measured_copy_ceiling"] = kernels[dominant]["GBps"] / best_copy
+    if cpu:
+        result["cpu_baseline"] = cpu_baseline(torch, w, args.cpu_rows, args.entropy_coeff, args.seed, mrl, dev, path)
+    return result
+
+
+def bandwidth_ceilings(torch, _lib, dev):
+    """Practical ceilings on this box: with the sweeps' access pattern (one workgroup per 152064-entry bf16
+    row) and with the pattern the HBM system serves best (one vector per thread, small workgroups)."""
     probe_rows, probe_row_bytes = 32768, 304128
     nbytes = probe_rows * probe_row_bytes
     src = torch.empty(nbytes, dtype=torch.uint8, device=dev)
@@ -579,17 +629,224 @@ def main():
     e.record()
     torch.cuda.synchronize()
     ceilings["runtime_d2d_copy_GBps"] = 2 * nbytes * 5 / (s.elapsed_time(e) * 1e-3) / 1e9
-    del src, dst
-    result["measured_ceiling"] = ceilings
-    # a read+write stream of R read bytes and W written bytes cannot beat R/read + W/write on this box
-    best_copy = max(ceilings["copy_GBps"], ceilings["stream_copy_GBps"])
-    for k in kernels.values():
-        k["frac_of_measured_copy"] = k["GBps"] / best_copy
-    result["roofline"]["frac_of_measured_copy_ceiling"] = kernels[dominant]["GBps"] / best_copy
-    dz = None
-    del dz
-    if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(torch, w, args.cpu_rows, args.entropy_coeff, args.seed, mrl, dev, args.path)
+    return ceilings
+
+
+# ----------------------------------------------------------------------------------------- configs[4], whole
+C4 = dict(prompts=8, group=16, r_lo=8192, r_hi=32768, vocab=129280, sigma=3.0)
+
+
+def make_c4_batch(torch, mrl, dev, seed):
+    """The experience batch of configs[4] without its logits: 8 prompts x 16 responses, R ~ U[8192, 32768],
+    1-token prompts, rewards Bernoulli(p), p ~ Beta(1/2, 1/2) per prompt; the dynamic-sampling filter
+    (workers/dynamic_sampling.py:81-86 of the reference) drops the groups whose rewards are all equal
+    BEFORE anything else sees the batch; advantages are the group-normalised rewards of the kept groups.
+    The seed is advanced until at least one group is dropped and at least three are kept.
+    Returns (batch on the device, kept row indices, rows before the filter)."""
+    n_all = C4["prompts"] * C4["group"]
+    while True:
+        gen = torch.Generator().manual_seed(seed)
+        rlen = torch.randint(C4["r_lo"], C4["r_hi"] + 1, (n_all, 1), generator=gen, dtype=torch.int32)
+        # Beta(1/2, 1/2) is the arcsine law: sin^2(pi u / 2) of a uniform u
+        p = torch.sin(torch.rand(C4["prompts"], 1, generator=gen) * (3.141592653589793 / 2)) ** 2
+        rewards = torch.bernoulli(p.repeat(1, C4["group"]).reshape(n_all, 1), generator=gen)
+        keep = mrl.dynamic_sampling_keep(rewards.flatten().to(dev), C4["group"])
+        if 3 * C4["group"] <= len(keep) < n_all:
+            break
+        seed += 1000
+    rlen, rewards = rlen[keep], rewards[keep]
+    n_seq, resp_w = len(keep), int(rlen.max())
+    full = {
+        "responses": torch.zeros(n_seq, resp_w, dtype=torch.int32, device=dev),
+        "response_length": rlen.to(dev),
+        "prompt_length": torch.ones(n_seq, 1, dtype=torch.int32, device=dev),
+    }
+    rmask = mrl.generate_mask(full["responses"], full["response_length"])
+    full["advantages"], _ = mrl.compute_group_norm_advantage_return(rewards.to(dev), rmask, full["response_length"],
+                                                                    C4["group"])
+    return full, keep, n_all
+
+
+def c4_micro_batch_inputs(torch, mrl, mb, dev, gen, ref_fn):
+    """Logits, labels and old log-probs of one micro-batch, made on the device: packed [1, T, V] bf16
+    logits ~N(0, 3), uniform labels, old = current log-prob + N(0, 0.05).  Returns (logits, kwargs)."""
+    vocab = C4["vocab"]
+    seqlens = (mb["prompt_length"] + mb["response_length"]).flatten().to(torch.int32)
+    cu = torch.zeros(seqlens.numel() + 1, dtype=torch.int32, device=dev)
+    cu[1:] = torch.cumsum(seqlens, 0)
+    total = int(cu[-1].item())
+    logits = torch.empty(1, total, vocab, dtype=torch.bfloat16, device=dev)
+    for lo in range(0, total, 8192):
+        hi = min(total, lo + 8192)
+        logits[0, lo:hi] = torch.randn(hi - lo, vocab, generator=gen, device=dev, dtype=torch.bfloat16) * C4["sigma"]
+    mb["labels"] = torch.randint(0, vocab, (1, total), generator=gen, device=dev)
+    kw = dict(use_remove_padding=True, seqlens_in_batch=seqlens, cu_seqlens_padded=cu, seq_len=int(seqlens.max().item()))
+    with torch.no_grad():
+        lp0 = ref_fn.compute_loss(logits, mb, forward_only=True, **kw)
+    maskf = mrl.generate_mask(mb["responses"], mb["response_length"]).to(torch.float32)
+    mb["old_log_prob"] = (lp0 + torch.randn(lp0.shape, generator=gen, device=dev) * 0.05) * maskf
+    return logits, kw, total
+
+
+def run_c4(args, steps=None, warmup=None):
+    """configs[4] as the reference runs it (models/base/base_training_engine.py:160-208 with use_dynamic_bsz):
+    the filtered batch is cut into token-budget micro-batches by the Karmarkar-Karp partitioner, and every
+    micro-batch goes through ONE DAPO loss object with use_dynamic_bsz / actual_micro_batch_size and
+    (loss / n_micro).backward().  One step = all micro-batches of the batch; the logits of a micro-batch
+    (up to 17 GB) are generated on the device right before it and are not part of the timed regions."""
+    import torch
+    import mindspeed_rl_amd as mrl
+    from mindspeed_rl_amd import vocab_ops
+    from mindspeed_rl_amd import seqlen_balancing as bal
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    steps = args.steps if steps is None else steps
+    warmup = args.warmup if warmup is None else warmup
+    full, keep, n_all = make_c4_batch(torch, mrl, dev, args.seed)
+    n_seq = len(keep)
+    batches, parts = bal.split_batches_with_dynamic_bsz(full, args.token_budget, None)
+    n_micro = len(batches)
+    f = mrl.LossFuncFactory.get_instance("ray_dapo", "actor")
+    f.add_loss_meta_info({"clip_ratio": 0.2, "clip_higher_enable": True, "clip_ratio_low": 0.2,
+                          "clip_ratio_high": 0.28, "token_level_loss": True, "entropy_coeff": args.entropy_coeff})
+    ref_fn = mrl.LossFuncFactory.get_instance("ray_grpo", "reference")
+    gen = torch.Generator(device=dev).manual_seed(args.seed)
+    rescales = f.grad_scale_state(dev).rescales
+    vocab, row_bytes = C4["vocab"], C4["vocab"] * 2
+    tokens = int(full["response_length"].sum().item())
+
+    def one_pass(record):
+        """All micro-batches once; returns (seconds inside the timed regions, per-micro-batch records)."""
+        spent, rows_seen, micro = 0.0, 0, []
+        for mb in batches:
+            mb = dict(mb)
+            logits, kw, total = c4_micro_batch_inputs(torch, mrl, mb, dev, gen, ref_fn)
+            z = logits.requires_grad_()
+            torch.cuda.synchronize()
+            if record:
+                vocab_ops.kernel_events = []
+            t0 = time.perf_counter()
+            loss, stats = f.compute_loss(z, mb, use_dynamic_bsz=True, actual_micro_batch_size=n_seq / n_micro,
+                                         index=None, **kw)
+            (loss / n_micro).backward()
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            spent += dt
+            rows_seen += total
+            if record:
+                events, vocab_ops.kernel_events = vocab_ops.kernel_events, None
+                sweep_ms = sum(s.elapsed_time(e) for (n, s, e, _) in events if n == "mrl_fused_logprob_loss")
+                live = int(mb["response_length"].sum().item())
+                nbytes = live * 2 * row_bytes + (total - live) * row_bytes
+                micro.append({"sequences": int(mb["response_length"].numel()), "rows": total, "step_ms": dt * 1e3,
+                              "sweep_ms": sweep_ms, "sweep_GBps": nbytes / (sweep_ms * 1e-3) / 1e9,
+                              "sweep_bytes": nbytes, "loss": float(loss.detach())})
+            del z, logits, loss
+        return spent, rows_seen, micro
+
+    for _ in range(warmup):
+        one_pass(False)
+    torch.cuda.synchronize()
+    rescales_before = int(rescales.item())
+    spent, micro = 0.0, []
+    for _ in range(steps):
+        dt, rows_seen, m = one_pass(True)
+        spent += dt
+        micro += m
+    ms_per_step = spent * 1e3 / steps
+    sweep_ms = sum(m["sweep_ms"] for m in micro)
+    sweep_bytes = sum(m["sweep_bytes"] for m in micro)
+    gbps = sweep_bytes / (sweep_ms * 1e-3) / 1e9
+    per_micro = sorted(m["sweep_GBps"] for m in micro)
+    result = {
+        "metric": "tokens/sec for logprob+DAPO loss fwd+bwd; achieved HBM GB/s as % of peak",
+        "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "configs[4]: 8x16 responses, R~U[8192,32768], V=129280 bf16, DAPO clip-higher 0.2/0.28, no KL, "
+                        "token-level loss; dynamic-sampling filter, then Karmarkar-Karp micro-batches of at most %d "
+                        "tokens through one loss object, (loss / n_micro).backward()" % args.token_budget,
+            "responses_before_filter": n_all, "responses_kept": n_seq, "groups_dropped": (n_all - n_seq) // C4["group"],
+            "micro_batches": n_micro, "token_budget": args.token_budget, "packed_rows": rows_seen,
+            "response_tokens": tokens, "vocab": vocab, "accumulate": "f32", "entropy_coeff": args.entropy_coeff,
+            "timed": "compute_loss + backward of every micro-batch (its logits are generated before, untimed)",
+        },
+        "roofline": {
+            "kernel": "fused_sweep_persistent_kernel (mrl_fused_logprob_loss), all micro-batches", "bound": "hbm",
+            "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": None,
+            "bytes_per_launch": sweep_bytes / len(micro), "avg_ms": sweep_ms / len(micro),
+            "per_micro_batch_GBps": {"min": per_micro[0], "median": _median(per_micro), "max": per_micro[-1]},
+        },
+        "rescale_passes_in_timed_steps": int(rescales.item()) - rescales_before,
+        "rescale_passes_in_all": int(rescales.item()),
+        "micro_batch_rows": {"min": min(m["rows"] for m in micro), "max": max(m["rows"] for m in micro)},
+        "micro_batch_step_ms": {"min": min(m["step_ms"] for m in micro), "median": _median([m["step_ms"] for m in micro]),
+                                "max": max(m["step_ms"] for m in micro)},
+        "loss": sum(m["loss"] for m in micro[-n_micro:]) / n_micro,
+    }
+    del batches, full
+    _release(torch)
+    return result
+
+
+def _compact(r):
+    """What other_workloads keeps of a result line."""
+    roof = r["roofline"]
+    out = {"ms_per_step": r["ms_per_step"], "value": r["value"], "unit": r["unit"], "steps": r["steps"],
+           "workload": r["config"]["workload"],
+           "roofline": {"kernel": roof["kernel"], "bound": roof["bound"], "achieved": roof["achieved"],
+                        "unit": roof["unit"], "frac": roof["frac"], "avg_ms": roof.get("avg_ms")}}
+    for key in ("ms_per_step_median", "rescale_passes_in_timed_steps", "library_products_comparison", "micro_batch_rows",
+                "micro_batch_step_ms"):
+        if key in r:
+            out[key] = r[key]
+    for key in ("per_micro_batch_GBps", "fused_sweeps_ms_per_step", "logits_products_ms_per_step",
+                "backward_products_ms_per_step"):
+        if key in roof:
+            out["roofline"][key] = roof[key]
+    for key in ("micro_batches", "responses_kept", "groups_dropped", "caches_flushed_between_steps"):
+        if key in r["config"]:
+            out[key] = r["config"][key]
+    return out
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (no collectives exist on this path); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import mindspeed_rl_amd as mrl  # noqa: F401  (fails loudly if the library is not built)
+    from mindspeed_rl_amd import _lib
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    _lib.load()
+    cpu = not args.no_cpu_baseline
+    if args.workload == "c3fwd":
+        result = run_lmhead(args)
+    elif args.workload == "c3":
+        result = run_lmhead_train(args)
+    elif args.workload == "c4":
+        result = run_c4(args)
+    elif args.workload == "c0":
+        result = run_sweep(args, "c0", dtype=args.dtype, upstream=args.upstream, cpu=cpu, flush=True)
+    elif args.workload != "all":
+        result = run_sweep(args, args.workload, dtype=args.dtype, upstream=args.upstream, cpu=cpu)
+    else:
+        # the headline first and alone on the card, then a few steps of everything else
+        result = run_sweep(args, "c1", dtype=args.dtype, upstream=args.upstream, cpu=cpu)
+        k, others = args.other_steps, {}
+        others["c0"] = _compact(run_sweep(args, "c0", steps=max(k, 20), warmup=3, probes=False, cpu=False, flush=True))
+        others["c2"] = _compact(run_sweep(args, "c2", steps=k, warmup=1, probes=False, cpu=False))
+        others["c4"] = _compact(run_c4(args, steps=1, warmup=1))
+        others["f32"] = _compact(run_sweep(args, "c1", dtype="f32", steps=k, warmup=1, probes=False, cpu=False))
+        others["upstream0.25"] = _compact(run_sweep(args, "c1", upstream=0.25, steps=k, warmup=2, probes=False, cpu=False))
+        others["c3fwd"] = _compact(run_lmhead(args, steps=k, warmup=1))
+        others["c3"] = _compact(run_lmhead_train(args, steps=max(1, k - 1), warmup=1))
+        result["other_workloads"] = others
     print(json.dumps(result), flush=True)
 
 
