@@ -198,8 +198,8 @@ def fused_lmhead_policy_loss(hidden, weight, batch, *, packed, seqlens=None, cu_
     :func:`mindspeed_rl_amd.fused_logprob_policy_loss` (``labels, responses, response_length,
     prompt_length, advantages``, optional ``old_log_prob``).  Returns ``(loss, out)``; ``backward()``
     yields dHidden and dWeight.  Full ``[T, V]`` logits are never materialised: at most
-    ``chunk_rows x V`` exist at a time.  ``hidden_dim`` and ``V`` must make 16-byte rows and
-    ``V <= mrl_fused_max_vocab``.  With ``compact_rows`` (default) rows without a live response token
+    ``chunk_rows x V`` exist at a time.  ``hidden_dim`` must be a multiple of 64, ``V`` of 8 and at
+    most ``mrl_fused_max_vocab`` (311 296); fp16 operands are not taken.  With ``compact_rows`` (default) rows without a live response token
     skip the GEMMs when they are more than 5 % of all rows; finding them costs one host
     synchronisation per call."""
     if kl_penalty is None:

@@ -439,7 +439,15 @@ class StandardLogProbComputer(LogProbComputer):
         labels = batch["labels"]
         inv_t = float(kwargs.get("inv_temperature", 1.0))
         injected = vocab_ops.get_vocab_parallel()
-        if injected is not None and injected is not vocab_ops.vocab_parallel_cross_entropy:
+        weight = kwargs.get("lm_head_weight")
+        if weight is not None:
+            # `output` holds the hidden states: the rows of the response windows are projected and scored
+            # tile by tile on the matrix cores, no logits are written (forward only, no autograd)
+            from .lmhead import lmhead_logprob
+            active = self._rows_in_windows(output, batch, kwargs).view(labels.shape)
+            log_probs, entropy, _ = lmhead_logprob(output, weight, labels, inv_temperature=inv_t,
+                                                   want_entropy=not skip_entropy, row_active=active)
+        elif injected is not None and injected is not vocab_ops.vocab_parallel_cross_entropy:
             # a caller's own cross entropy (the reference's hook) scores the rows, as in the reference
             scaled = output if inv_t == 1.0 else output * inv_t
             log_probs = compute_log_probs(scaled, labels)
@@ -532,6 +540,22 @@ class BaseLossFunc(ABC):
         strategy only (a caller that installs another ``logprob_computer`` gets the split path)."""
         return type(self.logprob_computer) is StandardLogProbComputer and _use_fused(output, kwargs)
 
+    def _from_hidden(self, output, batch, kwargs, **loss_args):
+        """The training step when the caller hands over the hidden states and ``lm_head_weight=``
+        instead of logits (keyword arguments ``lm_head_chunk_rows``, ``lm_head_compact_rows``):
+        logits exist for one chunk of rows at a time, and ``backward()`` reaches the hidden states
+        and the weight.  Forward-only calls take the same keyword through ``compute_log_probs``."""
+        from .lmhead import fused_lmhead_policy_loss
+        if type(self.logprob_computer) is not StandardLogProbComputer:
+            raise NotImplementedError("lm_head_weight= needs the standard log-prob strategy")
+        return fused_lmhead_policy_loss(
+            output, kwargs["lm_head_weight"], batch, packed=kwargs.get("use_remove_padding", False),
+            seqlens=kwargs.get("seqlens_in_batch"), cu_seqlens=kwargs.get("cu_seqlens_padded"),
+            inv_temperature=float(kwargs.get("inv_temperature", 1.0)),
+            expected_upstream=kwargs.get("expected_grad_scale"), scale_state=self.grad_scale_state(output.device),
+            chunk_rows=int(kwargs.get("lm_head_chunk_rows", 32768)),
+            compact_rows=bool(kwargs.get("lm_head_compact_rows", True)), **loss_args)
+
     @staticmethod
     def _get_compute_log_probs_input(output: torch.Tensor, batch: Dict[str, torch.Tensor]):
         if "responses" not in batch:
@@ -602,6 +626,13 @@ class GRPOActorLossFunc(BaseLossFunc):
         if forward_only:
             log_probs, _ = super().compute_log_probs(output=output, batch=batch, **kwargs)
             return log_probs
+        if kwargs.get("lm_head_weight") is not None:
+            loss, out = self._from_hidden(
+                output, batch, kwargs, ref_log_prob=batch.get("ref_log_prob"), clip_low=self.clip_ratio,
+                clip_high=self.clip_ratio, kl_penalty=self.kl_penalty, kl_coef=self.kl_ctrl.value,
+                entropy_coeff=self.entropy_coeff, token_level_loss=True,
+                loss_scale=_dynamic_scale(batch, forward_only, kwargs))
+            return _finish(loss, out)
         if self._fused(output, kwargs):
             loss, out = fused_logprob_policy_loss(
                 output, batch, ref_log_prob=batch.get("ref_log_prob"), clip_low=self.clip_ratio,
@@ -669,6 +700,12 @@ class DAPOActorLossFunc(BaseLossFunc):
             self.clip_ratio_low = self.clip_ratio
             self.clip_ratio_high = self.clip_ratio
         mask = batch["response_mask"] if "response_mask" in batch else None
+        if kwargs.get("lm_head_weight") is not None:
+            loss, out = self._from_hidden(
+                output, batch, kwargs, mask=mask, clip_low=self.clip_ratio_low, clip_high=self.clip_ratio_high,
+                kl_penalty=None, entropy_coeff=self.entropy_coeff, token_level_loss=self.token_level_loss,
+                loss_scale=_dynamic_scale(batch, forward_only, kwargs))
+            return _finish(loss, out)
         if self._fused(output, kwargs):
             loss, out = fused_logprob_policy_loss(
                 output, batch, mask=mask, clip_low=self.clip_ratio_low, clip_high=self.clip_ratio_high,
@@ -733,7 +770,9 @@ class PPOActorLossFunc(BaseLossFunc):
         common = dict(clip_low=self.clip_ratio, clip_high=self.clip_ratio, kl_penalty=None,
                       entropy_coeff=self.entropy_coeff, token_level_loss=True,
                       loss_scale=_dynamic_scale(batch, forward_only, kwargs))
-        if self._fused(output, kwargs):
+        if kwargs.get("lm_head_weight") is not None:
+            loss, out = self._from_hidden(output, batch, kwargs, **common)
+        elif self._fused(output, kwargs):
             loss, out = fused_logprob_policy_loss(output, batch, **common,
                                                   **_fused_kwargs(kwargs, self.grad_scale_state(output.device)))
         else:

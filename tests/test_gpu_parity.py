@@ -1451,6 +1451,87 @@ def test_fused_lmhead_policy_loss(dev, chunk_rows):
     assert (dw.float().cpu() * 2 - dw_want).abs().max().item() <= 2 ** -7 * dw_want.abs().max().item()
 
 
+@pytest.mark.parametrize("algo", ["grpo", "dapo", "ppo"])
+def test_loss_objects_take_hidden_states_and_lm_head_weight(dev, algo):
+    """The lm_head path behind the reference's own call surface: the training engine binds everything but
+    the model output with functools.partial and Megatron calls loss_func(output), then back-propagates
+    loss / num_microbatches (models/base/base_training_engine.py:236-270).  With lm_head_weight= bound
+    as well, `output` is the hidden states: same loss and statistics as the oracle on the projected
+    logits, and backward() reaches the hidden states and the weight.  The oracle is fed the bf16 logits
+    of the pipeline's own first product (one bf16 rounding away from F.linear, asserted here), its
+    dlogits are rounded to bf16 like the pipeline's.  Forward-only calls (old / reference log-probs)
+    take the same keyword and score the fp32 logits without storing any."""
+    from functools import partial
+    gen = torch.Generator().manual_seed({"grpo": 41, "dapo": 42, "ppo": 43}[algo])
+    vocab, hdim, inv_t = 2048, 128, 1.0 / 0.8
+    _, b, kw, _, _ = _make_batch(gen, 2, 4, 5, 24, vocab, torch.bfloat16, 1.0, 2, prompt_hi=6)
+    total = b["labels"].shape[1]
+    h = torch.randn(1, total, hdim, generator=gen).to(torch.bfloat16)
+    w = (torch.randn(vocab, hdim, generator=gen) * (3.0 / hdim ** 0.5)).to(torch.bfloat16)
+    z32 = torch.nn.functional.linear(h[0].float(), w.float())
+    # old / reference log-probs around the current policy, as the rollout side would have stored them
+    rmask = o_pack.generate_mask(torch.zeros_like(b["advantages"]), b["response_length"])
+    lp0 = o_loss.logprob_computer((z32 * inv_t).view(1, total, vocab), b, True, **kw)[0]
+    b["old_log_prob"] = (lp0 + torch.randn(lp0.shape, generator=gen) * 0.05) * rmask
+    b["ref_log_prob"] = (lp0 + torch.randn(lp0.shape, generator=gen) * 0.05) * rmask
+    hd, wd = h.to(dev).requires_grad_(), w.to(dev).requires_grad_()
+    zd = torch.empty(total, vocab, dtype=torch.bfloat16, device=dev)
+    _lib.call("mrl_lmhead_logits", hd.data_ptr(), wd.data_ptr(), total, vocab, hdim, zd.data_ptr(), vocab, _lib.stream(dev))
+    logits = zd.cpu().float()
+    assert (logits - z32).abs().max().item() <= 2 ** -8 * z32.abs().max().item()
+    if algo == "grpo":
+        meta_o = dict(clip_ratio=0.2, kl_coef=0.01, kl_penalty="low_var_kl", entropy_coeff=0.002)
+        meta_d = {"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.01), "kl_penalty": "low_var_kl", "entropy_coeff": 0.002}
+        oracle_loss, key = o_loss.grpo_compute_loss, ("ray_grpo", "actor")
+    elif algo == "dapo":
+        meta_o = dict(clip_ratio=0.2, clip_higher_enable=True, clip_ratio_low=0.2, clip_ratio_high=0.28,
+                      token_level_loss=False, entropy_coeff=0.002)
+        meta_d = dict(meta_o)
+        oracle_loss, key = o_loss.dapo_compute_loss, ("ray_dapo", "actor")
+    else:
+        meta_o = dict(clip_ratio=0.2, entropy_coeff=0.002)
+        meta_d = {"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.0), "entropy_coeff": 0.002}
+        oracle_loss, key = o_loss.ppo_compute_loss, ("ray_ppo", "actor")
+    zo = logits.view(1, total, vocab).requires_grad_()
+    want, want_stats = oracle_loss(zo * inv_t, b, meta_o, **kw)
+    (dz,) = torch.autograd.grad(want, zo)
+    dz16 = dz[0].to(torch.bfloat16).float()
+    n_micro = 4
+    dh_want = (dz16 @ w.float()) / n_micro
+    dw_want = (dz16.t() @ h[0].float()) / n_micro
+
+    f = mrl.LossFuncFactory.get_instance(*key)
+    f.add_loss_meta_info(meta_d)
+    bd, kwd = _to_dev(b, dev), _to_dev(kw, dev)
+    # exactly the caller's steps: bind, call with the model output alone, scale, backward
+    loss_func = partial(f.compute_loss, batch=bd, forward_only=False, non_loss_data=True, lm_head_weight=wd,
+                        inv_temperature=inv_t, lm_head_chunk_rows=64, **kwd)
+    loss, stats = loss_func(hd)
+    assert loss.dim() == 0 and loss.requires_grad and all(isinstance(v, float) for v in stats.values())
+    (loss / n_micro).backward()
+    assert abs(loss.item() - want.item()) <= TOL_LOSS_REL * abs(want.item()) + 1e-7
+    assert set(stats) == set(want_stats)
+    for k, v in want_stats.items():
+        assert abs(stats[k] - v) <= TOL_LOSS_REL * abs(v) + 1e-6, k
+    assert hd.grad.shape == hd.shape and wd.grad.shape == wd.shape and hd.grad.dtype == torch.bfloat16
+    assert (hd.grad.float().cpu()[0] - dh_want).abs().max().item() <= 2 ** -7 * dh_want.abs().max().item()
+    assert (wd.grad.float().cpu() - dw_want).abs().max().item() <= 2 ** -7 * dw_want.abs().max().item()
+    # forward only, through the actor object and through the reference-policy object: [B, L] log-probs of
+    # the fp32 logits, nothing stored
+    want_lp = o_loss.logprob_computer((z32 * inv_t).view(1, total, vocab), b, True, **kw)[0]
+    ref_fn = mrl.LossFuncFactory.get_instance("ray_grpo", "reference")
+    for obj in (f, ref_fn):
+        with torch.no_grad():
+            lp = partial(obj.compute_loss, batch=bd, forward_only=True, lm_head_weight=wd.detach(),
+                         inv_temperature=inv_t, **kwd)(hd.detach())
+        assert lp.shape == want_lp.shape
+        assert (lp.cpu() - want_lp).abs().max().item() < 2e-4
+    lp_rows, ent_rows = f.compute_log_probs(hd.detach(), bd, skip_entropy=False, lm_head_weight=wd.detach(),
+                                            inv_temperature=inv_t, **kwd)
+    want_ent = o_loss.logprob_computer((z32 * inv_t).view(1, total, vocab), b, False, **kw)[1]
+    assert (ent_rows.cpu() - want_ent).abs().max().item() < 2e-4
+
+
 @pytest.mark.parametrize("tokens,vocab,hdim", [(517, 4352, 3584), (300, 1000, 128), (64, 4096 + 24, 256), (1, 8, 64),
                                                (777, 2048, 192), (4100, 520, 64)])
 def test_lmhead_products_through_the_c_abi(dev, tokens, vocab, hdim):
@@ -2781,6 +2862,111 @@ def test_dynamic_micro_batches_end_to_end(dev, algo):
         if fused:
             # upstream 1/n_micro is learned from the first backward: one rescale pass, not n_micro
             assert f.grad_scale_state(dev).rescales.item() == 1
+
+
+def test_config4_whole_batch_in_micro_batches(dev):
+    """configs[4] whole, as `bench.py --workload c4` runs it: 8 x 16 responses of 8 k - 32 k tokens, the
+    dynamic-sampling filter first, the kept sequences cut into micro-batches of at most 65 536 tokens by the
+    Karmarkar-Karp partitioner (the oracle's partitions must be the same), every micro-batch's logits
+    ([T <= 65 536, 129 280] bf16, up to 17 GB) generated on the device, ONE DAPO loss object with
+    use_dynamic_bsz / actual_micro_batch_size, (loss / n_micro).backward().  The oracle cannot follow at
+    this size, so every micro-batch is held to the size-independent properties: the fused sweep and the
+    split kernels (independent code) agree on loss, statistics and every dlogit; every dlogits row sums to
+    zero; rows without a response token are exactly zero; sampled rows match the oracle's log-prob and
+    entropy and lie in the span of the two gradient directions the closed form allows.  The upstream
+    gradient 1 / n_micro is learned once: one rescale pass in the whole batch."""
+    import bench
+    import gc
+    from mindspeed_rl_amd import seqlen_balancing as bal
+    from oracle import balancing as o_bal
+    gc.collect()
+    torch.cuda.empty_cache()
+    free, _ = torch.cuda.mem_get_info(dev)
+    if free < 80 * 2 ** 30:
+        pytest.skip("needs more free HBM")
+    full, keep, n_all = bench.make_c4_batch(torch, mrl, dev, 0)
+    group, vocab = bench.C4["group"], bench.C4["vocab"]
+    n_seq = len(keep)
+    assert n_all == 128 and n_seq % group == 0 and 3 * group <= n_seq < n_all
+    kept_groups = sorted(set(i // group for i in keep))
+    assert keep == [g * group + j for g in kept_groups for j in range(group)]
+    # every kept group mixes rewards, so its advantages have both signs; lengths are in range
+    adv0 = full["advantages"][:, 0].view(-1, group)
+    assert (adv0.max(1).values > 0).all().item() and (adv0.min(1).values < 0).all().item()
+    rl = full["response_length"].flatten()
+    assert rl.min().item() >= 8192 and rl.max().item() <= 32768
+    batches, parts = bal.split_batches_with_dynamic_bsz(full, 65536, None)
+    lengths = (full["prompt_length"] + full["response_length"]).flatten().tolist()
+    assert parts == o_bal.rearrange_micro_batches(lengths, 65536, dynamic_max_batch_size=None)
+    n_micro = len(parts)
+    assert sorted(i for part in parts for i in part) == list(range(n_seq))
+    assert n_micro >= (sum(lengths) + 65535) // 65536 and all(sum(lengths[i] for i in part) <= 65536 for part in parts)
+    f = mrl.LossFuncFactory.get_instance("ray_dapo", "actor")
+    f.add_loss_meta_info({"clip_ratio": 0.2, "clip_higher_enable": True, "clip_ratio_low": 0.2,
+                          "clip_ratio_high": 0.28, "token_level_loss": True, "entropy_coeff": 0.001})
+    ref_fn = mrl.LossFuncFactory.get_instance("ray_grpo", "reference")
+    gen = torch.Generator(device=dev).manual_seed(0)
+    cpu_gen = torch.Generator().manual_seed(4)
+    total_loss, rows_seen, checked = 0.0, 0, 0
+    for k, (mb, part) in enumerate(zip(batches, parts)):
+        mb = dict(mb)
+        logits, kw, total = bench.c4_micro_batch_inputs(torch, mrl, mb, dev, gen, ref_fn)
+        rows_seen += total
+        flat, flat_labels = logits.view(-1, vocab), mb["labels"].reshape(-1)
+        cu = kw["cu_seqlens_padded"].cpu().tolist()
+        live = torch.zeros(total, dtype=torch.bool)
+        for i, r in enumerate(mb["response_length"].flatten().tolist()):
+            live[cu[i]:cu[i] + r] = True                     # 1-token prompts: the first R_i rows of a sequence
+        live_d = live.to(dev)
+        live_idx = torch.nonzero(live).flatten()
+        pick = torch.cat([live_idx[torch.randint(0, live_idx.numel(), (6,), generator=cpu_gen)],
+                          torch.nonzero(~live).flatten()[:2]])
+        pick_d = pick.to(dev)
+        zs, ys = flat[pick_d].float().cpu(), flat_labels[pick_d].cpu()
+        z1 = logits.detach().requires_grad_()
+        dyn = dict(use_dynamic_bsz=True, actual_micro_batch_size=n_seq / n_micro, index=None)
+        loss_f, stats_f = f.compute_loss(z1, mb, fused=True, **dyn, **kw)
+        (loss_f / n_micro).backward()
+        dz_f = z1.grad.view(-1, vocab)
+        total_loss += loss_f.item() / n_micro
+        got = dz_f[pick_d].float().cpu() * n_micro
+        # the split kernels on the same micro-batch, gradient written over the logits
+        z2 = logits.detach().requires_grad_()
+        loss_s, stats_s = f.compute_loss(z2, mb, fused=False, grad_inplace=True, **dyn, **kw)
+        (dz_s,) = torch.autograd.grad(loss_s / n_micro, z2)
+        dz_s = dz_s.view(-1, vocab)
+        assert loss_s.item() == pytest.approx(loss_f.item(), rel=TOL_LOSS_REL), k
+        for name in stats_f:
+            assert stats_s[name] == pytest.approx(stats_f[name], rel=TOL_LOSS_REL, abs=2e-6), (k, name)
+        scale, worst_sum, worst_diff = 0.0, 0.0, 0.0
+        for lo in range(0, total, 8192):
+            a, c = dz_f[lo:lo + 8192].float(), dz_s[lo:lo + 8192].float()
+            scale = max(scale, a.abs().max().item())
+            worst_diff = max(worst_diff, (a - c).abs().max().item())
+            worst_sum = max(worst_sum, a.sum(-1).abs().max().item())
+            dead = ~live_d[lo:lo + 8192]
+            if dead.any().item():
+                assert a.abs().amax(-1)[dead].max().item() == 0 and c.abs().amax(-1)[dead].max().item() == 0, k
+            del a, c
+        assert scale > 0 and worst_diff <= 2 ** -7 * scale and worst_sum <= 0.02 * scale, k
+        # sampled rows: the gradient is c0 (onehot - p) - c1 p (z - E z) for some c0, c1
+        p = torch.softmax(zs, -1)
+        onehot = torch.zeros_like(p)
+        onehot[torch.arange(len(ys)), ys] = 1.0
+        basis0, basis1 = onehot - p, -(p * (zs - (p * zs).sum(-1, keepdim=True)))
+        for i in range(len(pick)):
+            if not live[pick[i]]:
+                assert not got[i].any().item()
+                continue
+            a = torch.stack([basis0[i], basis1[i]], 1).double()
+            coef = torch.linalg.lstsq(a, got[i].double().unsqueeze(1)).solution
+            resid = (a @ coef).squeeze(1) - got[i].double()
+            assert resid.abs().max().item() <= 2 ** -8 * got[i].abs().max().item() + 1e-12, (k, i)
+            checked += 1
+        del z1, z2, dz_f, dz_s, logits, flat
+    assert rows_seen == sum(lengths) and checked >= 5 * n_micro
+    assert total_loss == total_loss and abs(total_loss) < 10           # finite
+    assert f.grad_scale_state(dev).rescales.item() == 1
 
 
 def _small_padded_micro_batch(seed, n_seq, seq_len, vocab):
