@@ -167,18 +167,24 @@ __device__ __forceinline__ void zero_part(const RowRef& dst) {
     }
 }
 
-// Online-softmax statistics of the vectors one thread holds.  A vector past the end of the row
-// (zeros from the range-checked load) is processed like any other and its result discarded, which
-// costs three selects on the few vectors that can be affected and keeps the pass free of branches.
+// Online-softmax statistics of the vectors one thread holds, the careful way: the running maximum is
+// brought up to date before every vector, so the exponentials never exceed 1 whatever the logits are
+// (infinities and NaN included).  A vector past the end of the row (zeros from the range-checked load)
+// is processed like any other and its result discarded, which costs three selects on the few vectors
+// that can be affected and keeps the pass free of branches.
 template <int DT, int NV, bool kEntropy>
-__device__ __forceinline__ Stats thread_stats(const u32x4 (&v)[NV], int n_vec, float k) {
+__device__ __forceinline__ Stats thread_stats_careful(const u32x4 (&v)[NV], int n_vec, float k) {
     using E = Elem<DT>;
     constexpr int kVec = E::kVec;
     Stats st = {kMaxInit, 0.f, 0.f};
 #pragma unroll
     for (int q = 0; q < NV; ++q) {
+        // through an empty asm statement, as in grad_vec: entries that another pass has unpacked
+        // must not be kept for this one
+        u32x4 x = v[q];
+        asm volatile("" : "+v"(x));
         float z[kVec];
-        E::unpack(v[q], z);
+        E::unpack(x, z);
         Stats nx = st;
         float vmax = nx.m;
 #pragma unroll
@@ -199,6 +205,76 @@ __device__ __forceinline__ Stats thread_stats(const u32x4 (&v)[NV], int n_vec, f
         // into one chain per statistic and parks every exponential in scratch memory in between
         asm volatile("" : "+v"(st.m), "+v"(st.s), "+v"(st.u));
     }
+    return st;
+}
+
+// A thread's sums may be taken against any reference value in place of the running maximum, as long
+// as no exponential overflows: the result (m, s, u) then simply carries that reference as its m, and
+// every later merge treats it like a maximum.  An entry of the row is a safe reference from below
+// (the largest entry then contributes at least 1), and for ordinary logits it is within a few units
+// of the maximum, so nothing comes near the 2^127 an fp32 holds.  Taking the largest entry of the
+// thread's first vector saves the maximum over every vector and the rescale that follows it - a
+// quarter of the arithmetic of the pass.  If a sum does end up beyond 2^120, infinite or NaN (logits
+// that climb by more than 80 above that entry, infinities, NaN), the thread takes its statistics
+// once more, carefully.  Which way a thread went depends only on its own entries.
+constexpr float kSumLimit = 1.329228e36f;      // 2^120
+
+template <int DT, bool kEntropy>
+__device__ __forceinline__ void add_vector(const u32x4& vec, float k, float rk, float& s, float& u) {
+    using E = Elem<DT>;
+    constexpr int kVec = E::kVec;
+    float z[kVec];
+    E::unpack(vec, z);
+#pragma unroll
+    for (int i = 0; i < kVec; ++i) {
+        const float e = fast_exp2(__builtin_fmaf(z[i], k, -rk));
+        s += e;
+        if (kEntropy) u = __builtin_fmaf(e, z[i], u);
+    }
+}
+
+template <int DT>
+__device__ __forceinline__ float vector_max(const u32x4& vec) {
+    using E = Elem<DT>;
+    constexpr int kVec = E::kVec;
+    float z[kVec];
+    E::unpack(vec, z);
+    float r = z[0];
+#pragma unroll
+    for (int i = 1; i < kVec; ++i) r = fmaxf(r, z[i]);
+    return r;
+}
+
+// want_max (uniform over the workgroup): the caller needs the true maximum of the row in m (a label
+// outside the vocabulary scores the row maximum), which only the careful pass delivers.
+template <int DT, int NV, bool kEntropy>
+__device__ __forceinline__ Stats thread_stats(const u32x4 (&v)[NV], int n_vec, float k, bool want_max) {
+    Stats st = {kMaxInit, 0.f, 0.f};
+    // rows so short that a thread may hold no complete vector at all have nothing to gain
+    bool careful = Tail<NV>::kFull == 0 || want_max;
+    if (!careful) {
+        st.m = vector_max<DT>(v[0]);
+        const float rk = st.m * k;
+#pragma unroll
+        for (int q = 0; q < NV; ++q) {
+            float s = st.s, u = st.u;
+            add_vector<DT, kEntropy>(v[q], k, rk, s, u);
+            if (q >= Tail<NV>::kFull) {
+                const bool valid = q * kBlock + (int)threadIdx.x < n_vec;
+                st.s = valid ? s : st.s;
+                st.u = valid ? u : st.u;
+            } else {
+                st.s = s;
+                st.u = u;
+            }
+            asm volatile("" : "+v"(st.s), "+v"(st.u));       // as in the careful pass
+            // nothing but the two sums links one vector to the next here, so the scheduler would
+            // unpack many vectors ahead of their use; keep each vector's work together
+            vector_fence();
+        }
+        careful = !(st.s < kSumLimit);
+    }
+    if (careful) st = thread_stats_careful<DT, NV, kEntropy>(v, n_vec, k);
     return st;
 }
 
@@ -331,7 +407,7 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_kernel(
     const float z_y = E::load(row + (y_ok ? y : 0));
 
     const float k = inv_t * kLog2e;
-    const Stats st = thread_stats<DT, NV, kEntropy>(v, n_vec, k);
+    const Stats st = thread_stats<DT, NV, kEntropy>(v, n_vec, k, !y_ok);
     const Stats tot = block_reduce_1024<kEntropy>(st, k, lds);
 
     // row scalars, computed redundantly by every thread (uniform values)
@@ -408,23 +484,37 @@ __device__ __forceinline__ unsigned long long pack2f(float lo, float hi) {
 
 // Statistics of a stretch of a row streamed from memory by the whole workgroup (the fallback above):
 // thread t takes vectors t, t + 1024, ... in this order, as thread_stats does with the vectors a
-// thread holds, and the reduction is the same.
+// thread holds - the same reference, the same sums, the same second attempt - and the reduction is
+// the same.  `whole`: every thread has at least one vector and the row maximum is not asked for (what
+// makes thread_stats take the short way).
 template <int DT, bool kEntropy>
-__device__ __forceinline__ Stats stream_stats(const typename Elem<DT>::T* base, int n_vec, float k, Stats* lds) {
+__device__ __forceinline__ Stats stream_stats(const typename Elem<DT>::T* base, int n_vec, float k, bool whole,
+                                              Stats* lds) {
     using E = Elem<DT>;
     constexpr int kVec = E::kVec;
     const u32x4* vec = reinterpret_cast<const u32x4*>(base);
     Stats st = {kMaxInit, 0.f, 0.f};
-    for (int idx = threadIdx.x; idx < n_vec; idx += kBlock) {
-        float z[kVec];
-        E::unpack(__builtin_nontemporal_load(vec + idx), z);
-        float vmax = st.m;
+    bool careful = !whole;
+    if (whole) {
+        st.m = vector_max<DT>(__builtin_nontemporal_load(vec + threadIdx.x));
+        const float rk = st.m * k;
+        for (int idx = threadIdx.x; idx < n_vec; idx += kBlock)
+            add_vector<DT, kEntropy>(__builtin_nontemporal_load(vec + idx), k, rk, st.s, st.u);
+        careful = !(st.s < kSumLimit);
+    }
+    if (careful) {
+        st = {kMaxInit, 0.f, 0.f};
+        for (int idx = threadIdx.x; idx < n_vec; idx += kBlock) {
+            float z[kVec];
+            E::unpack(__builtin_nontemporal_load(vec + idx), z);
+            float vmax = st.m;
 #pragma unroll
-        for (int i = 0; i < kVec; ++i) vmax = fmaxf(vmax, z[i]);
-        grow_max<kEntropy>(st, vmax, k);
-        const float mk = st.m * k;
+            for (int i = 0; i < kVec; ++i) vmax = fmaxf(vmax, z[i]);
+            grow_max<kEntropy>(st, vmax, k);
+            const float mk = st.m * k;
 #pragma unroll
-        for (int i = 0; i < kVec; ++i) add_one<kEntropy>(st, z[i], k, mk);
+            for (int i = 0; i < kVec; ++i) add_one<kEntropy>(st, z[i], k, mk);
+        }
     }
     __syncthreads();            // lds may still be read by a slow wavefront of the previous reduction
     return block_reduce_1024<kEntropy>(st, k, lds);
@@ -459,7 +549,7 @@ __device__ __forceinline__ void fill_inbox(Inbox* in, unsigned long long a, unsi
 template <int DT, bool kEntropy>
 __device__ __forceinline__ Stats exchange_halves(const Stats& mine, int half, HalfRecord* rec, uint32_t spin_limit,
                                                  const typename Elem<DT>::T* other_base, int other_vec, float k,
-                                                 Stats* lds, Inbox* inbox, bool zy_here, bool zy_there,
+                                                 bool other_whole, Stats* lds, Inbox* inbox, bool zy_here, bool zy_there,
                                                  const typename Elem<DT>::T* zy_ptr, float& z_y) {
     using E = Elem<DT>;
     if (threadIdx.x == 0) {
@@ -483,7 +573,7 @@ __device__ __forceinline__ Stats exchange_halves(const Stats& mine, int half, Ha
     __syncthreads();
     Stats other = inbox->st;
     if (inbox->arrived == 0u) {                                  // uniform branch
-        other = stream_stats<DT, kEntropy>(other_base, other_vec, k, lds);
+        other = stream_stats<DT, kEntropy>(other_base, other_vec, k, other_whole, lds);
         if (threadIdx.x == 0) {
             // the logit at the label from the other half, then - once it has arrived - the record again
             uint32_t zy_mem = zy_there ? __float_as_uint(E::load(zy_ptr)) : 0u;
@@ -602,7 +692,7 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
         bool wrote = false;                 // dlogits of row r written and the next row requested
         if (m != 0.f) {
             float z_y = E::from_bits(zy_bits);
-            const Stats st = thread_stats<DT, NV, kEntropy>(v, n_vec, k);
+            const Stats st = thread_stats<DT, NV, kEntropy>(v, n_vec, k, !y_ok);
             Stats tot = block_reduce_1024<kEntropy>(st, k, lds);
             if (kWide) {
                 // the logit at the label as this unit loaded it counts only if the label lies in this
@@ -610,7 +700,7 @@ __global__ __launch_bounds__(kBlock) void fused_sweep_persistent_kernel(
                 const int other_first = half ? 0 : half_elems;
                 const T* whole = logits + row * row_stride;
                 tot = exchange_halves<DT, kEntropy>(tot, half, half_records + row * 2, spin_limit, whole + other_first,
-                                                    (int)(unit_bytes[half ^ 1] / 16u), k, lds, &inbox, y_mine,
+                                                    (int)(unit_bytes[half ^ 1] / 16u), k, Tail<NV>::kFull != 0 && y_ok, lds, &inbox, y_mine,
                                                     y_ok && !y_mine, whole + (y_ok ? y : 0), z_y);
             }
             float lse;
@@ -744,15 +834,29 @@ __global__ __launch_bounds__(256) void scale_rows_note_kernel(typename Elem<DT>:
     const float was = applied[0];
     const float ratio = u / was;
     if (ratio != 1.f) {
+        // few workgroups (each counts itself with one atomic below, also when nothing is to be moved):
+        // four vectors per thread in flight make up for them
         const int n_vec = vocab / kVec;
         for (int64_t r = blockIdx.x; r < n_rows; r += gridDim.x) {
             u32x4* vec = reinterpret_cast<u32x4*>(x + r * row_stride);
-            for (int idx = threadIdx.x; idx < n_vec; idx += 256) {
-                float z[kVec];
-                E::unpack(vec[idx], z);
+            for (int base = 0; base < n_vec; base += 4 * 256) {
+                u32x4 v[4];
 #pragma unroll
-                for (int i = 0; i < kVec; ++i) z[i] *= ratio;
-                vec[idx] = E::pack(z);
+                for (int j = 0; j < 4; ++j) {
+                    const int idx = base + j * 256 + (int)threadIdx.x;
+                    if (idx < n_vec) v[j] = vec[idx];
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int idx = base + j * 256 + (int)threadIdx.x;
+                    if (idx < n_vec) {
+                        float z[kVec];
+                        E::unpack(v[j], z);
+#pragma unroll
+                        for (int i = 0; i < kVec; ++i) z[i] *= ratio;
+                        vec[idx] = E::pack(z);
+                    }
+                }
             }
         }
     }
@@ -1084,7 +1188,7 @@ extern "C" int mrl_scale_rows_note(void* x, int dtype, int64_t n_rows, int64_t v
     MRL_REQUIRE(vocab % (16 / eb) == 0 && mrl::aligned(x, 16) && (n_rows == 1 || (row_stride * eb) % 16 == 0),
                 MRL_ERR_UNSUPPORTED, "%s: needs 16-byte aligned rows", fn);
     hipStream_t s = mrl::as_stream(stream);
-    const dim3 grid((unsigned)(n_rows < 1024 ? n_rows : 1024)), block(256);
+    const dim3 grid((unsigned)(n_rows < 512 ? n_rows : 512)), block(256);
     switch (dtype) {
         case MRL_F32:
             hipLaunchKernelGGL(scale_rows_note_kernel<MRL_F32>, grid, block, 0, s, (float*)x, row_stride, (int)vocab,

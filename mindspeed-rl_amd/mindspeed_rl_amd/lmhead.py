@@ -178,11 +178,14 @@ class _FusedLmHeadLoss(torch.autograd.Function):
         ctx.meta = (tuple(hidden.shape), cfg.get("scale_state"))
         ctx.handed_out = False
         ctx.mark_non_differentiable(ops.out)
+        ctx.set_materialize_grads(False)
         return ops.loss, ops.out
 
     @staticmethod
     def backward(ctx, g_loss, _g_out):
         from .loss import _deliver_eager_grads
+        if g_loss is None:
+            return None, None, None, None, None
         d_hidden, d_weight, applied = ctx.saved_tensors
         shape, state = ctx.meta
         d_hidden, d_weight = _deliver_eager_grads(ctx, (d_hidden, d_weight), applied, state, g_loss)

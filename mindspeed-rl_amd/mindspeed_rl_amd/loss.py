@@ -96,10 +96,13 @@ class _PolicyLoss(torch.autograd.Function):
         ctx.scalars = scalars
         ctx.want_entropy_grad = entropy is not None and entropy.requires_grad
         ctx.mark_non_differentiable(out)
+        ctx.set_materialize_grads(False)
         return out[0].clone(), out      # the loss gets its own storage: autograd outputs must not alias
 
     @staticmethod
     def backward(ctx, g_loss, _g_out):
+        if g_loss is None:
+            return (None,) * 8
         lp, old, ref, adv, mask, lens, row_sums, out = ctx.saved_tensors
         dev = lp.device
         batch, width = lp.shape
@@ -328,10 +331,13 @@ class _FusedLogprobLoss(torch.autograd.Function):
         ctx.meta = (tuple(output.shape), cfg.get("scale_state"))
         ctx.handed_out = False
         ctx.mark_non_differentiable(ops.out)
+        ctx.set_materialize_grads(False)        # no zero tensor for the statistics output in every backward
         return ops.loss, ops.out
 
     @staticmethod
     def backward(ctx, g_loss, _g_out):
+        if g_loss is None:
+            return None, None, None, None
         dlogits, applied = ctx.saved_tensors
         shape, state = ctx.meta
         (grad,) = _deliver_eager_grads(ctx, (dlogits,), applied, state, g_loss)

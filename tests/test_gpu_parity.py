@@ -3078,6 +3078,40 @@ def test_two_backwards_over_one_retained_graph(dev, kind):
         assert a.data_ptr() != c.data_ptr() and torch.equal(a, c)
 
 
+@pytest.mark.parametrize("upstream", [0.0, float("inf")])
+def test_backward_with_a_zero_or_infinite_upstream_gradient(dev, upstream):
+    """A skipped or overflowed loss-scale step reaches the loss as an upstream gradient of 0 or Inf.  It
+    is applied like any other value (zeros, or infinities and NaN, come out - autograd's own product),
+    it is NOT taken as the scale of the next sweep, and the next step is exact again.  What cannot be
+    had afterwards is a second backward over the SAME retained graph: the stored gradients have been
+    multiplied by 0 or Inf, so it yields NaN - a value that cannot pass for a gradient - rather than a
+    wrong finite one."""
+    meta = dict(clip_ratio=0.2, kl_coef=0.01, kl_penalty="low_var_kl", entropy_coeff=0.001)
+    z, b = _small_padded_micro_batch(13, 4, 24, 520)
+    bd = _to_dev(b, dev)
+    zo = z.clone().requires_grad_()
+    (want,) = torch.autograd.grad(o_loss.grpo_compute_loss(zo, b, meta)[0] * 0.5, zo)
+    f = mrl.GRPOActorLossFunc()
+    f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.01), "kl_penalty": "low_var_kl",
+                          "entropy_coeff": 0.001})
+    state = f.grad_scale_state(dev)
+    zd = z.to(dev).requires_grad_()
+    (g0,) = torch.autograd.grad(f.compute_loss(zd, bd, fused=True)[0] * 0.5, zd)          # learns 0.5
+    assert state.learned.item() == 0.5
+    loss, _ = f.compute_loss(zd, bd, fused=True)
+    (g1,) = torch.autograd.grad(loss * upstream, zd, retain_graph=True)
+    live = want != 0
+    if upstream == 0.0:
+        assert not g1.any().item()
+    else:
+        assert not torch.isfinite(g1.cpu()[live]).any().item()
+    assert state.learned.item() == 0.5                               # not learned
+    (g2,) = torch.autograd.grad(loss * 0.5, zd)                      # same graph again: cannot be recovered
+    assert torch.isnan(g2.cpu()[live]).all().item()
+    (g3,) = torch.autograd.grad(f.compute_loss(zd, bd, fused=True)[0] * 0.5, zd)          # the next step
+    assert (g3.cpu() - want).abs().max().item() <= 1e-6 and torch.equal(g3, g0)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("bounds", [(0, 2048, 4096), (0, 1024, 2048, 3072, 4096), (0, 520, 528, 3000, 4096)])
 def test_vocabulary_shards_merge_to_the_full_sweep(dev, dtype, bounds):
