@@ -412,7 +412,7 @@ PROFILED_TRAFFIC = {
     ("c1", "bf16", "split", "mrl_vocab_logprob_bwd"):
         (104.06e9, "profiles/vocab_fwd_kernel_and_bwd_chunk_kernel__c1_split_path.md"),
     ("c1", "f32", "fused", "mrl_fused_logprob_loss"):
-        (208.18e9, "profiles/fused_sweep_persistent_kernel_half_rows__c1_fp32_logits.md"),
+        (208.20e9, "profiles/fused_sweep_persistent_kernel_half_rows__c1_fp32_logits.md"),
 }
 
 

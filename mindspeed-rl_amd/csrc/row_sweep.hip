@@ -822,8 +822,11 @@ __global__ __launch_bounds__(256) void scale_rows_kernel(typename Elem<DT>::T* x
 }
 
 // One backward of one buffer in a single launch: the conditional rescale above, then the book-keeping
-// of grad_scale_note_kernel by whichever workgroup finishes last (a counter next to the scale tells;
-// every workgroup has read the scale before it counts itself, so the last one may overwrite it).
+// of grad_scale_note_kernel.  When nothing is to be moved (the ratio is 1, i.e. the new scale equals
+// the old one) workgroup 0 does the book-keeping at once - what it stores over the scale is the value
+// every other workgroup reads there anyway - and the others leave.  Otherwise the workgroup that
+// finishes last does it (a counter next to the scale tells; every workgroup has read the scale before
+// it counts itself, so the last one may overwrite it).
 template <int DT>
 __global__ __launch_bounds__(256) void scale_rows_note_kernel(typename Elem<DT>::T* x, int64_t row_stride, int vocab,
                                                               int64_t n_rows, const float* __restrict__ upstream,
@@ -833,31 +836,22 @@ __global__ __launch_bounds__(256) void scale_rows_note_kernel(typename Elem<DT>:
     const float u = *upstream;
     const float was = applied[0];
     const float ratio = u / was;
-    if (ratio != 1.f) {
-        // few workgroups (each counts itself with one atomic below, also when nothing is to be moved):
-        // four vectors per thread in flight make up for them
-        const int n_vec = vocab / kVec;
-        for (int64_t r = blockIdx.x; r < n_rows; r += gridDim.x) {
-            u32x4* vec = reinterpret_cast<u32x4*>(x + r * row_stride);
-            for (int base = 0; base < n_vec; base += 4 * 256) {
-                u32x4 v[4];
+    if (ratio == 1.f) {
+        if (blockIdx.x == 0 && threadIdx.x == 0) {
+            applied[0] = u;
+            if (learned && u != 0.f && __builtin_isfinite(u)) *learned = u;
+        }
+        return;
+    }
+    const int n_vec = vocab / kVec;
+    for (int64_t r = blockIdx.x; r < n_rows; r += gridDim.x) {
+        u32x4* vec = reinterpret_cast<u32x4*>(x + r * row_stride);
+        for (int idx = threadIdx.x; idx < n_vec; idx += 256) {
+            float z[kVec];
+            E::unpack(vec[idx], z);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int idx = base + j * 256 + (int)threadIdx.x;
-                    if (idx < n_vec) v[j] = vec[idx];
-                }
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int idx = base + j * 256 + (int)threadIdx.x;
-                    if (idx < n_vec) {
-                        float z[kVec];
-                        E::unpack(v[j], z);
-#pragma unroll
-                        for (int i = 0; i < kVec; ++i) z[i] *= ratio;
-                        vec[idx] = E::pack(z);
-                    }
-                }
-            }
+            for (int i = 0; i < kVec; ++i) z[i] *= ratio;
+            vec[idx] = E::pack(z);
         }
     }
     __syncthreads();
@@ -865,9 +859,9 @@ __global__ __launch_bounds__(256) void scale_rows_note_kernel(typename Elem<DT>:
         uint32_t* done = reinterpret_cast<uint32_t*>(applied) + 1;
         const uint32_t before = __hip_atomic_fetch_add(done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (before == gridDim.x - 1) {
-            if (rescales && ratio != 1.f) *rescales += 1u;
+            if (rescales) *rescales += 1u;
             applied[0] = u;
-            *done = 0u;
+            __hip_atomic_store(done, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (learned && u != 0.f && __builtin_isfinite(u)) *learned = u;
         }
     }
@@ -1188,7 +1182,7 @@ extern "C" int mrl_scale_rows_note(void* x, int dtype, int64_t n_rows, int64_t v
     MRL_REQUIRE(vocab % (16 / eb) == 0 && mrl::aligned(x, 16) && (n_rows == 1 || (row_stride * eb) % 16 == 0),
                 MRL_ERR_UNSUPPORTED, "%s: needs 16-byte aligned rows", fn);
     hipStream_t s = mrl::as_stream(stream);
-    const dim3 grid((unsigned)(n_rows < 512 ? n_rows : 512)), block(256);
+    const dim3 grid((unsigned)(n_rows < 2048 ? n_rows : 2048)), block(256);
     switch (dtype) {
         case MRL_F32:
             hipLaunchKernelGGL(scale_rows_note_kernel<MRL_F32>, grid, block, 0, s, (float*)x, row_stride, (int)vocab,
