@@ -18,7 +18,8 @@ same line carries, under "other_workloads", a few steps of every other configura
 CPU-sized batch (c0), the padded layout (c2), the whole long-response DAPO batch in token-budget
 micro-batches (c4), fp32 logits, an upstream gradient the loss object is not told (upstream0.25)
 and the lm_head forward and training step (c3fwd, c3); the headline keys stay those of the
-headline workload.
+headline workload.  That run also measures roofline.traffic itself: two short child runs of this
+script under rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), scaled by the copy probe of the same run.
 """
 import argparse
 import json
@@ -78,6 +79,9 @@ def parse_args():
                     help="scalar the step multiplies the loss by before backward(), as Megatron's schedule does with "
                          "1/num_microbatches; the loss object is not told and learns it from the first backward")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-traffic", action="store_true",
+                    help="do not measure the sweep's HBM traffic (two short child runs of this script under "
+                         "rocprofv3 --pmc); roofline.traffic then comes from the committed profile")
     ap.add_argument("--cpu-rows", type=int, default=2048, help="rows of the CPU baseline sample")
     ap.add_argument("--seed", type=int, default=0)
     return ap.parse_args()
@@ -421,6 +425,58 @@ def _profiled_traffic(args, workload, w, path, dominant):
     if args.entropy_coeff != 0.001 or any(k.startswith("MRL_") for k in os.environ):
         return None, None
     return PROFILED_TRAFFIC.get((workload, w["dtype"], path, dominant), (None, None))
+
+
+def measure_traffic(args):
+    """HBM bytes per launch of the headline workload's sweep, measured now: this script is run twice more
+    as a child process under `rocprofv3 --pmc` (FETCH_SIZE, then WRITE_SIZE - one counter per run), and
+    each reading of the sweep is scaled by what the same counter reads for the copy probe of known size
+    in that same run.  Returns a dict, or None when rocprofv3 is missing, times out or yields nothing."""
+    import csv
+    import glob
+    import shutil
+    import signal
+    import subprocess
+    import tempfile
+    rocprof = shutil.which("rocprofv3") or "/opt/rocm/bin/rocprofv3"
+    if not os.path.exists(rocprof) or any(k.startswith(("ROCP_", "ROCPROF")) for k in os.environ):
+        return None                                        # absent, or this process is itself being profiled
+    probe_bytes = 32768 * 304128                           # what probe_copy_kernel reads, and writes
+    out = {}
+    work = tempfile.mkdtemp(prefix="mrl_traffic_", dir="/tmp")
+    try:
+        for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+            d = os.path.join(work, counter)
+            cmd = [rocprof, "--pmc", counter, "--output-format", "csv", "-d", d, "-o", "t", "--", sys.executable,
+                   os.path.abspath(__file__), "--workload", "c1", "--steps", "1", "--warmup", "1", "--no-cpu-baseline",
+                   "--no-traffic", "--seed", str(args.seed), "--entropy-coeff", str(args.entropy_coeff)]
+            proc = subprocess.Popen(cmd, cwd="/tmp", env=dict(os.environ, TMPDIR="/tmp"), stdout=subprocess.DEVNULL,
+                                    stderr=subprocess.DEVNULL, start_new_session=True)
+            try:
+                proc.wait(timeout=150)
+            except subprocess.TimeoutExpired:
+                os.killpg(proc.pid, signal.SIGKILL)
+                proc.wait()
+                return None
+            sweep, probe = [], []
+            for f in glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True):
+                for row in csv.DictReader(open(f)):
+                    if row.get("Counter_Name") != counter:
+                        continue
+                    if "fused_sweep_persistent_kernel" in row["Kernel_Name"]:
+                        sweep.append(float(row["Counter_Value"]))
+                    elif "probe_copy_kernel" in row["Kernel_Name"]:
+                        probe.append(float(row["Counter_Value"]))
+            if not sweep or not probe:
+                return None
+            factor = probe_bytes / (sum(probe) / len(probe) * 1024.0)        # bytes per counted byte
+            out[counter] = {"raw_KiB_per_launch": sum(sweep) / len(sweep), "copy_probe_raw_KiB": sum(probe) / len(probe),
+                            "scale_factor": factor, "bytes_per_launch": sum(sweep) / len(sweep) * 1024.0 * factor,
+                            "launches": len(sweep)}
+    finally:
+        shutil.rmtree(work, ignore_errors=True)
+    return {"bytes": out["FETCH_SIZE"]["bytes_per_launch"] + out["WRITE_SIZE"]["bytes_per_launch"],
+            "fetch": out["FETCH_SIZE"], "write": out["WRITE_SIZE"]}
 
 
 def _median(xs):
@@ -847,6 +903,16 @@ def main():
         others["c3fwd"] = _compact(run_lmhead(args, steps=k, warmup=1))
         others["c3"] = _compact(run_lmhead_train(args, steps=max(1, k - 1), warmup=1))
         result["other_workloads"] = others
+        # the sweep's HBM traffic, measured now (the card is free again: children of this process run it)
+        if not args.no_traffic and args.dtype in (None, "bf16") and args.path == "fused":
+            measured = measure_traffic(args)
+            if measured is not None:
+                result["roofline"]["traffic"] = measured["bytes"]
+                result["roofline"]["traffic_source"] = {
+                    "measured_this_run": True,
+                    "method": "two child runs of `bench.py --workload c1 --steps 1 --warmup 1` under rocprofv3 --pmc "
+                              "(FETCH_SIZE, then WRITE_SIZE), each scaled by the copy probe of the same run",
+                    "fetch": measured["fetch"], "write": measured["write"]}
     print(json.dumps(result), flush=True)
 
 
