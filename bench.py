@@ -79,6 +79,9 @@ def parse_args():
                     help="scalar the step multiplies the loss by before backward(), as Megatron's schedule does with "
                          "1/num_microbatches; the loss object is not told and learns it from the first backward")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--deferred-stats", action="store_true",
+                    help="compute_loss(..., deferred_stats=True): the statistics are copied to the host asynchronously and "
+                         "become python floats when first looked at (after the timed loop here)")
     ap.add_argument("--no-traffic", action="store_true",
                     help="do not measure the sweep's HBM traffic (two short child runs of this script under "
                          "rocprofv3 --pmc); roofline.traffic then comes from the committed profile")
@@ -491,7 +494,7 @@ def _release(torch):
 
 
 def run_sweep(args, workload, dtype=None, upstream=1.0, path=None, steps=None, warmup=None, probes=True, cpu=True,
-              flush=False):
+              flush=False, deferred=None):
     """One of the logits workloads (c1, c2, c0, c4chunk) through a loss object: K timed steps bracketed by
     synchronisations, HIP events around every step (median) and around every vocabulary sweep.
     flush: a 1 GiB buffer is rewritten between the steps, outside the per-step events, so that a working
@@ -505,6 +508,7 @@ def run_sweep(args, workload, dtype=None, upstream=1.0, path=None, steps=None, w
     steps = args.steps if steps is None else steps
     warmup = args.warmup if warmup is None else warmup
     path = args.path if path is None else path
+    deferred = args.deferred_stats if deferred is None else deferred
     w = dict(WORKLOADS[workload])
     if dtype is not None and dtype != w["dtype"]:
         w["dtype"] = dtype
@@ -529,7 +533,7 @@ def run_sweep(args, workload, dtype=None, upstream=1.0, path=None, steps=None, w
 
     def step():
         z = logits.detach().requires_grad_()
-        loss, stats = f.compute_loss(z, b, fused=(path == "fused"), **kw)
+        loss, stats = f.compute_loss(z, b, fused=(path == "fused"), deferred_stats=deferred, **kw)
         (dz,) = torch.autograd.grad(loss, z, grad_outputs=root)
         return loss, stats, dz
 
@@ -560,6 +564,15 @@ def run_sweep(args, workload, dtype=None, upstream=1.0, path=None, steps=None, w
     vocab_ops.kernel_events = None
     step_ms = [s_ev.elapsed_time(e_ev) for s_ev, e_ev in step_events]
     ms_per_step = _median(step_ms) if flush else elapsed * 1e3 / steps
+    hot_ms = None
+    if flush:
+        # the same steps back to back, caches warm, no events: what a loop over micro-batches of this size sees
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            del dz
+            loss, stats, dz = step()
+        torch.cuda.synchronize()
+        hot_ms = (time.perf_counter() - t0) * 1e3 / steps
 
     def avg_ms(name):
         ts = [s.elapsed_time(e) for (n, s, e, _) in events if n == name]
@@ -621,6 +634,7 @@ def run_sweep(args, workload, dtype=None, upstream=1.0, path=None, steps=None, w
             # the scalar autograd starts the backward from; the loss object is not told
             "upstream": upstream,
             "caches_flushed_between_steps": bool(flush),
+            "deferred_stats": bool(deferred),
         },
         "roofline": {
             "kernel": "%s (%s)" % (kernels[dominant]["symbol"], dominant), "bound": "hbm",
@@ -631,6 +645,7 @@ def run_sweep(args, workload, dtype=None, upstream=1.0, path=None, steps=None, w
         },
         "ms_per_step_median": _median(step_ms),
         "ms_per_step_mean_wall": elapsed * 1e3 / steps,
+        "ms_per_step_hot": hot_ms,
         "kernels": kernels,
         "step_hbm": {"GBps": step_gbps, "frac": step_gbps / HBM_PEAK_GBPS, "algorithmic_bytes_per_step": step_bytes},
         # NOT a roofline fraction: the step's time applied to the bytes a 3-pass (read, read, write)
@@ -853,8 +868,8 @@ def _compact(r):
            "workload": r["config"]["workload"],
            "roofline": {"kernel": roof["kernel"], "bound": roof["bound"], "achieved": roof["achieved"],
                         "unit": roof["unit"], "frac": roof["frac"], "avg_ms": roof.get("avg_ms")}}
-    for key in ("ms_per_step_median", "rescale_passes_in_timed_steps", "library_products_comparison", "micro_batch_rows",
-                "micro_batch_step_ms"):
+    for key in ("ms_per_step_median", "ms_per_step_hot", "rescale_passes_in_timed_steps", "library_products_comparison",
+                "micro_batch_rows", "micro_batch_step_ms"):
         if key in r:
             out[key] = r[key]
     for key in ("per_micro_batch_GBps", "fused_sweeps_ms_per_step", "logits_products_ms_per_step",
@@ -895,7 +910,12 @@ def main():
         # the headline first and alone on the card, then a few steps of everything else
         result = run_sweep(args, "c1", dtype=args.dtype, upstream=args.upstream, cpu=cpu)
         k, others = args.other_steps, {}
-        others["c0"] = _compact(run_sweep(args, "c0", steps=max(k, 20), warmup=3, probes=False, cpu=False, flush=True))
+        others["c0"] = _compact(run_sweep(args, "c0", steps=max(k, 20), warmup=3, probes=False, cpu=False, flush=True,
+                                          deferred=False))
+        # the same with the statistics fetched lazily (no synchronisation between forward and backward)
+        lazy = run_sweep(args, "c0", steps=max(k, 20), warmup=3, probes=False, cpu=False, flush=True, deferred=True)
+        others["c0"]["ms_per_step_deferred_stats"] = lazy["ms_per_step"]
+        others["c0"]["ms_per_step_hot_deferred_stats"] = lazy["ms_per_step_hot"]
         others["c2"] = _compact(run_sweep(args, "c2", steps=k, warmup=1, probes=False, cpu=False))
         others["c4"] = _compact(run_c4(args, steps=1, warmup=1))
         others["f32"] = _compact(run_sweep(args, "c1", dtype="f32", steps=k, warmup=1, probes=False, cpu=False))

@@ -9,7 +9,7 @@ from .advantage import (FixedKLController, compute_group_norm_advantage_return, 
                         dynamic_sampling_keep_mask)
 from .functional import clip_by_value, is_multimodal, masked_mean, masked_sum
 from .lmhead import fused_lmhead_policy_loss, lmhead_logprob
-from .loss import (BaseLossFunc, DAPOActorLossFunc, GradScaleState, GRPOActorLossFunc, LossFuncFactory, LossRegister,
+from .loss import (BaseLossFunc, DAPOActorLossFunc, DeferredStats, GradScaleState, GRPOActorLossFunc, LossFuncFactory, LossRegister,
                    MultimodalLogProbComputer, PPOActorLossFunc, ReferenceLossFunc, RewardLossFunc,
                    StandardLogProbComputer, fused_logprob_policy_loss, fused_supported, policy_loss)
 from .packing import (generate_mask, pack_index, postprocess_packed_seqs, preprocess_packed_seqs, response_window,

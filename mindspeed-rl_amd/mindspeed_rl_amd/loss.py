@@ -579,18 +579,125 @@ class BaseLossFunc(ABC):
         return self.logprob_computer.compute(output, batch, skip_entropy, **kwargs)
 
 
-def _finish(loss, out):
+class DeferredStats(dict):
+    """The statistics dict of ``compute_loss`` with the device-to-host copy taken off the critical path:
+    the eight output scalars are copied into pinned host memory asynchronously, and the python floats
+    are made when a value is first looked at (``stats[key]``, ``items()``, ``values()``, ``get``,
+    printing, copying, pickling) - typically after the backward, when the reference's engine gathers
+    the metrics of all micro-batches.  Keys, ``len`` and ``in`` need no synchronisation.  Selected with
+    ``deferred_stats=True`` (keyword of ``compute_loss``) or the environment variable
+    MRL_DEFERRED_STATS=1; the default returns plain floats at once, like the reference."""
+
+    __slots__ = ("_pending", "__weakref__")
+
+    def __init__(self, spec, host, event):
+        super().__init__((key, None) for key, _, _ in spec)
+        self._pending = (spec, host, event)
+
+    def _fetch(self):
+        if self._pending is not None:
+            spec, host, event = self._pending
+            self._pending = None
+            event.synchronize()
+            values = host.tolist()
+            for key, index, use_abs in spec:
+                dict.__setitem__(self, key, abs(values[index]) if use_abs else values[index])
+        return self
+
+    # every way to a value goes through _fetch(); __iter__ / keys are overridden so that dict(), {**x} and
+    # update() cannot take the interpreter's short cut past these methods
+    def __getitem__(self, key):
+        return dict.__getitem__(self._fetch(), key)
+
+    def get(self, key, default=None):
+        return dict.get(self._fetch(), key, default)
+
+    def items(self):
+        return dict.items(self._fetch())
+
+    def values(self):
+        return dict.values(self._fetch())
+
+    def keys(self):
+        return dict.keys(self)
+
+    def __iter__(self):
+        return dict.__iter__(self)
+
+    def pop(self, key, *default):
+        return dict.pop(self._fetch(), key, *default)
+
+    def popitem(self):
+        return dict.popitem(self._fetch())
+
+    def setdefault(self, key, default=None):
+        return dict.setdefault(self._fetch(), key, default)
+
+    def copy(self):
+        return dict(dict.items(self._fetch()))
+
+    def __eq__(self, other):
+        return dict.__eq__(self._fetch(), other)
+
+    def __ne__(self, other):
+        return not self.__eq__(other)
+
+    __hash__ = None
+
+    def __repr__(self):
+        return dict.__repr__(self._fetch())
+
+    def __reduce__(self):
+        return (dict, (self.copy(),))
+
+
+class _PinnedRing:
+    """Pinned host slots for the deferred statistics of one device: allocated once, used in turn.  A
+    slot is handed out again only after 256 later calls; whoever still holds it then is fetched first."""
+
+    def __init__(self, slots=256):
+        import weakref
+        self._weakref = weakref
+        self.buffer = torch.empty((slots, 8), dtype=torch.float32, pin_memory=True)
+        self.holders = [None] * slots
+        self.next = 0
+
+    def take(self, make):
+        slot = self.next
+        self.next = (slot + 1) % len(self.holders)
+        old = self.holders[slot]
+        old = old() if old is not None else None
+        if old is not None:
+            old._fetch()
+        holder = make(self.buffer[slot])
+        self.holders[slot] = self._weakref.ref(holder)
+        return holder
+
+
+_pinned_rings = {}
+
+
+def _finish(loss, out, kwargs=None, skip=()):
     """The five statistics as python floats from ONE device-to-host copy (the reference issues five
-    ``.item()`` calls); ``abs`` on the policy loss as in ``grpo_actor_loss_func.py:91-97``."""
-    host = out.detach().cpu().tolist()
-    stats = {
-        STAT_KEYS[0]: abs(host[1]),
-        STAT_KEYS[1]: host[2],
-        STAT_KEYS[2]: host[3],
-        STAT_KEYS[3]: host[4],
-        STAT_KEYS[4]: host[5],
-    }
-    return loss, stats
+    ``.item()`` calls); ``abs`` on the policy loss as in ``grpo_actor_loss_func.py:91-97``.  With
+    deferred statistics the copy is asynchronous and the floats are made on first access."""
+    spec = [(STAT_KEYS[i], i + 1, i == 0) for i in range(5) if STAT_KEYS[i] not in skip]
+    deferred = (kwargs or {}).get("deferred_stats", os.environ.get("MRL_DEFERRED_STATS", "0") == "1")
+    if not deferred:
+        host = out.detach().cpu().tolist()
+        return loss, {key: (abs(host[index]) if use_abs else host[index]) for key, index, use_abs in spec}
+    dev = out.device
+    ring = _pinned_rings.get(dev)
+    if ring is None:
+        ring = _pinned_rings[dev] = _PinnedRing()
+
+    def make(host):
+        host.copy_(out.detach(), non_blocking=True)
+        event = torch.cuda.Event()
+        event.record(torch.cuda.current_stream(dev))
+        return DeferredStats(spec, host, event)
+
+    return loss, ring.take(make)
 
 
 def _dynamic_scale(batch, forward_only, kwargs):
@@ -638,7 +745,7 @@ class GRPOActorLossFunc(BaseLossFunc):
                 clip_high=self.clip_ratio, kl_penalty=self.kl_penalty, kl_coef=self.kl_ctrl.value,
                 entropy_coeff=self.entropy_coeff, token_level_loss=True,
                 loss_scale=_dynamic_scale(batch, forward_only, kwargs))
-            return _finish(loss, out)
+            return _finish(loss, out, kwargs)
         if self._fused(output, kwargs):
             loss, out = fused_logprob_policy_loss(
                 output, batch, ref_log_prob=batch.get("ref_log_prob"), clip_low=self.clip_ratio,
@@ -646,7 +753,7 @@ class GRPOActorLossFunc(BaseLossFunc):
                 entropy_coeff=self.entropy_coeff, token_level_loss=True,
                 loss_scale=_dynamic_scale(batch, forward_only, kwargs),
                 **_fused_kwargs(kwargs, self.grad_scale_state(output.device)))
-            return _finish(loss, out)
+            return _finish(loss, out, kwargs)
         log_probs, entropy = super().compute_log_probs(output=output, batch=batch,
                                                        skip_entropy=(self.entropy_coeff == 0), **kwargs)
         # batch['response_mask'] is ignored here, as in the reference: the mask is j < response_length
@@ -656,7 +763,7 @@ class GRPOActorLossFunc(BaseLossFunc):
                                 clip_high=self.clip_ratio, kl_penalty=self.kl_penalty, kl_coef=self.kl_ctrl.value,
                                 entropy_coeff=self.entropy_coeff, token_level_loss=True,
                                 loss_scale=_dynamic_scale(batch, forward_only, kwargs))
-        return _finish(loss, out)
+        return _finish(loss, out, kwargs)
 
     @staticmethod
     def _compute_grpo_policy_loss(old_log_prob, log_prob, ref_log_prob, advantages, entropy, eos_mask, cliprange,
@@ -711,14 +818,14 @@ class DAPOActorLossFunc(BaseLossFunc):
                 output, batch, kwargs, mask=mask, clip_low=self.clip_ratio_low, clip_high=self.clip_ratio_high,
                 kl_penalty=None, entropy_coeff=self.entropy_coeff, token_level_loss=self.token_level_loss,
                 loss_scale=_dynamic_scale(batch, forward_only, kwargs))
-            return _finish(loss, out)
+            return _finish(loss, out, kwargs)
         if self._fused(output, kwargs):
             loss, out = fused_logprob_policy_loss(
                 output, batch, mask=mask, clip_low=self.clip_ratio_low, clip_high=self.clip_ratio_high,
                 kl_penalty=None, entropy_coeff=self.entropy_coeff, token_level_loss=self.token_level_loss,
                 loss_scale=_dynamic_scale(batch, forward_only, kwargs),
                 **_fused_kwargs(kwargs, self.grad_scale_state(output.device)))
-            return _finish(loss, out)
+            return _finish(loss, out, kwargs)
         log_probs, entropy = super().compute_log_probs(output=output, batch=batch,
                                                        skip_entropy=(self.entropy_coeff == 0), **kwargs)
         loss, out = policy_loss(log_probs, entropy if self.entropy_coeff != 0 else None, batch.get("old_log_prob"),
@@ -727,7 +834,7 @@ class DAPOActorLossFunc(BaseLossFunc):
                                 clip_low=self.clip_ratio_low, clip_high=self.clip_ratio_high, kl_penalty=None,
                                 entropy_coeff=self.entropy_coeff, token_level_loss=self.token_level_loss,
                                 loss_scale=_dynamic_scale(batch, forward_only, kwargs))
-        return _finish(loss, out)
+        return _finish(loss, out, kwargs)
 
     @staticmethod
     def _compute_dapo_policy_loss(old_log_prob, log_prob, entropy, entropy_coeff, advantages, eos_mask,
@@ -787,9 +894,7 @@ class PPOActorLossFunc(BaseLossFunc):
             loss, out = policy_loss(log_probs, entropy if self.entropy_coeff != 0 else None,
                                     batch.get("old_log_prob"), None, batch.get("advantages"),
                                     response_length=batch["response_length"], **common)
-        loss, stats = _finish(loss, out)
-        del stats[STAT_KEYS[3]]                  # PPO reports no actor/kl_loss
-        return loss, stats
+        return _finish(loss, out, kwargs, skip=(STAT_KEYS[3],))          # PPO reports no actor/kl_loss
 
     @staticmethod
     def _compute_ppo_policy_loss(old_log_prob, log_prob, advantages, eos_mask, cliprange, entropy, entropy_coeff):

@@ -3078,6 +3078,40 @@ def test_two_backwards_over_one_retained_graph(dev, kind):
         assert a.data_ptr() != c.data_ptr() and torch.equal(a, c)
 
 
+def test_deferred_statistics_equal_the_eager_ones(dev):
+    """deferred_stats=True takes the device-to-host copy of the statistics off the path between forward
+    and backward: the floats that come out when the dict is finally read are those of the eager call,
+    for every loss object, fused and split, and many deferred dicts may be outstanding at once."""
+    gen = torch.Generator().manual_seed(3)
+    logits, b, kw, _, _ = _make_batch(gen, 2, 4, 5, 30, 2048, torch.bfloat16, 2.0, 1)
+    bd, kwd = _to_dev(b, dev), _to_dev(kw, dev)
+    metas = {("ray_grpo", "actor"): {"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.01), "kl_penalty": "low_var_kl",
+                                     "entropy_coeff": 0.001},
+             ("ray_dapo", "actor"): {"clip_ratio": 0.2, "clip_higher_enable": True, "clip_ratio_low": 0.2,
+                                     "clip_ratio_high": 0.28, "token_level_loss": True, "entropy_coeff": 0.001},
+             ("ray_ppo", "actor"): {"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.0), "entropy_coeff": 0.001}}
+    held = []
+    for key, meta in metas.items():
+        for fused in (True, False):
+            f = mrl.LossFuncFactory.get_instance(*key)
+            f.add_loss_meta_info(meta)
+            z = logits.to(dev).requires_grad_()
+            loss_e, eager = f.compute_loss(z, bd, fused=fused, **kwd)
+            loss_d, lazy = f.compute_loss(z, bd, fused=fused, deferred_stats=True, **kwd)
+            (g,) = torch.autograd.grad(loss_d, z)                       # the backward runs before anyone looks
+            assert type(eager) is dict and isinstance(lazy, mrl.DeferredStats) and set(lazy) == set(eager)
+            held.append((eager, lazy, loss_e.item(), loss_d.item()))
+    for eager, lazy, le, ld in held:
+        assert le == ld and dict(lazy) == eager and all(isinstance(v, float) for v in lazy.values())
+    # more outstanding dicts than pinned slots: the oldest are fetched when their slot comes round again
+    f = mrl.GRPOActorLossFunc()
+    f.add_loss_meta_info(metas[("ray_grpo", "actor")])
+    z = logits.to(dev).requires_grad_()
+    _, want = f.compute_loss(z, bd, fused=True, **kwd)
+    many = [f.compute_loss(z, bd, fused=True, deferred_stats=True, **kwd)[1] for _ in range(300)]
+    assert all(dict(m) == want for m in many)
+
+
 @pytest.mark.parametrize("upstream", [0.0, float("inf")])
 def test_backward_with_a_zero_or_infinite_upstream_gradient(dev, upstream):
     """A skipped or overflowed loss-scale step reaches the loss as an upstream gradient of 0 or Inf.  It

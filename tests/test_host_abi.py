@@ -277,3 +277,39 @@ def test_multimodal_switch_selects_strategy_and_partitioner(monkeypatch):
     assert sb.rearrange_micro_batches(lengths, 100, multimodal=False) == plain
     monkeypatch.setenv("IS_MULTIMODAL", "False")
     assert type(mrl.GRPOActorLossFunc().logprob_computer) is mrl.StandardLogProbComputer
+
+
+def test_deferred_stats_behaves_like_the_dict_of_floats_it_stands_for():
+    """compute_loss(..., deferred_stats=True) returns a dict whose values are fetched from the device on
+    first access: keys, len and `in` are known at once; every way to a value (indexing, items, values,
+    get, dict(), {**x}, update, json, pickle, ==) synchronises once and then yields plain floats."""
+    import json
+    import pickle
+    from mindspeed_rl_amd.loss import STAT_KEYS, DeferredStats
+
+    class Event:
+        waits = 0
+
+        def synchronize(self):
+            Event.waits += 1
+
+    spec = [(STAT_KEYS[i], i + 1, i == 0) for i in range(5)]
+    host = torch.tensor([9.0, -1.0, 2.0, 3.0, 4.0, 5.0, 6.0, 7.0])
+    want = dict(zip(STAT_KEYS, [1.0, 2.0, 3.0, 4.0, 5.0]))           # abs() on the policy loss
+
+    def fresh():
+        return DeferredStats(spec, host, Event())
+
+    d = fresh()
+    assert isinstance(d, dict) and len(d) == 5 and STAT_KEYS[2] in d and list(d) == list(STAT_KEYS) and Event.waits == 0
+    assert d[STAT_KEYS[0]] == 1.0 and Event.waits == 1 and d[STAT_KEYS[4]] == 5.0 and Event.waits == 1
+    assert dict(fresh()) == want and {**fresh()} == want and fresh() == want and fresh().copy() == want
+    assert json.loads(json.dumps(fresh())) == want
+    restored = pickle.loads(pickle.dumps(fresh()))
+    assert type(restored) is dict and restored == want
+    merged = {}
+    merged.update(fresh())
+    assert merged == want and sorted(fresh().values()) == [1.0, 2.0, 3.0, 4.0, 5.0]
+    assert fresh().get("absent", 7) == 7 and fresh().get(STAT_KEYS[1]) == 2.0
+    assert all(isinstance(v, float) for _, v in fresh().items())
+    assert "actor/pg_loss" in repr(fresh())
