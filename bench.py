@@ -248,6 +248,65 @@ def cpu_baseline(torch, w, rows_target, entropy_coeff, seed, mrl=None, dev=None,
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 
+class BoardSampler:
+    """Samples the shader clock and the board power from sysfs while a timed region runs (a thread that reads two
+    small files every 20 ms; no GPU call).  The bf16 products run against the board's power cap, where the clock
+    falls below its 2400 MHz peak: `peak_at_sclk` is the MFMA peak scaled to the clock that was actually held."""
+
+    PEAK_SCLK_MHZ = 2400.0
+
+    def __init__(self):
+        import glob
+        self.clock_files = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))[:1]
+        self.power_files = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input"))[:1]
+        self.cap_files = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap"))[:1]
+        self.sclk, self.power, self._stop, self._thread = [], [], False, None
+
+    def _read_once(self):
+        try:
+            for f in self.clock_files:
+                for line in open(f).read().splitlines():
+                    if line.rstrip().endswith("*"):
+                        self.sclk.append(float(line.split(":")[1].lower().replace("mhz", "").replace("*", "").strip()))
+            for f in self.power_files:
+                self.power.append(float(open(f).read().strip()) / 1e6)
+        except (OSError, ValueError, IndexError):
+            pass
+
+    def _loop(self):
+        while not self._stop:
+            self._read_once()
+            time.sleep(0.02)
+
+    def __enter__(self):
+        import threading
+        self._thread = threading.Thread(target=self._loop, daemon=True)
+        self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop = True
+        self._thread.join()
+        return False
+
+    def summary(self, tflops=None):
+        if not self.sclk:
+            return None
+        # the first samples still see the idle clock: the median of the second half is the load's
+        sclk = _median(self.sclk[len(self.sclk) // 2:])
+        out = {"sclk_mhz": sclk, "samples": len(self.sclk), "sclk_peak_mhz": self.PEAK_SCLK_MHZ}
+        if self.power:
+            out["power_w"] = _median(self.power[len(self.power) // 2:])
+        try:
+            out["power_cap_w"] = float(open(self.cap_files[0]).read().strip()) / 1e6
+        except (OSError, ValueError, IndexError):
+            pass
+        if tflops is not None:
+            out["peak_at_sclk"] = MFMA_BF16_PEAK_TFLOPS * sclk / self.PEAK_SCLK_MHZ
+            out["frac_of_peak_at_sclk"] = tflops / out["peak_at_sclk"]
+        return out
+
+
 def run_lmhead(args, steps=None, warmup=None):
     """configs[3], forward part: hidden [T, 3584] ~N(0,1), W [152064, 3584] ~N(0,0.02), bf16; one step =
     log-prob + entropy + logsumexp of every token without materialising the logits."""
@@ -267,11 +326,12 @@ def run_lmhead(args, steps=None, warmup=None):
         mrl.lmhead_logprob(hidden, weight, labels)
     torch.cuda.synchronize()
     lmhead.kernel_events = []
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        lp, ent, lse = mrl.lmhead_logprob(hidden, weight, labels)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    with BoardSampler() as board:
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            lp, ent, lse = mrl.lmhead_logprob(hidden, weight, labels)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
     events, lmhead.kernel_events = lmhead.kernel_events, None
     ms = sum(s.elapsed_time(e) for (_, s, e, _) in events) / len(events)
     flops = 2.0 * tokens * vocab * hdim
@@ -291,6 +351,7 @@ def run_lmhead(args, steps=None, warmup=None):
                      "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "flops_per_launch": flops, "avg_ms": ms},
         "max_abs_err_vs_fp32_gemm_256_rows": err,
     }
+    result["roofline"]["board"] = board.summary(tflops)
     return result
 
 
@@ -345,11 +406,12 @@ def run_lmhead_train(args, steps=None, warmup=None):
     torch.cuda.synchronize()
     vocab_ops.kernel_events = []
     lmhead.kernel_events = []
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        loss, stats, dh, dw = step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    with BoardSampler() as board:
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            loss, stats, dh, dw = step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
     events, vocab_ops.kernel_events = vocab_ops.kernel_events, None
     gemm_events, lmhead.kernel_events = lmhead.kernel_events, None
     sweep_ms = sum(s.elapsed_time(e) for (_, s, e, _) in events) / steps
@@ -379,11 +441,12 @@ def run_lmhead_train(args, steps=None, warmup=None):
 
     library_products()
     s_ev, e_ev = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    s_ev.record()
-    for _ in range(3):
-        library_products()
-    e_ev.record()
-    torch.cuda.synchronize()
+    with BoardSampler() as lib_board:
+        s_ev.record()
+        for _ in range(3):
+            library_products()
+        e_ev.record()
+        torch.cuda.synchronize()
     lib_chunk_ms = s_ev.elapsed_time(e_ev) / 3
     del z, w_hv, dh_c, dw32, h_t
     result = {
@@ -403,9 +466,11 @@ def run_lmhead_train(args, steps=None, warmup=None):
         "library_products_comparison": {
             "what": "torch.mm / addmm (hipBLASLt) for the same three products of one %d-row chunk, timed alone" % rows,
             "ms_per_chunk": lib_chunk_ms, "scaled_to_step_ms": lib_chunk_ms * total / rows,
-            "hand_written_products_ms_per_step": logits_ms + bwd_ms},
+            "hand_written_products_ms_per_step": logits_ms + bwd_ms,
+            "board": lib_board.summary(6.0 * rows * vocab * hdim / (lib_chunk_ms * 1e-3) / 1e12)},
         "loss": float(loss.detach()), "stats": stats[1:6],
     }
+    result["roofline"]["board"] = board.summary(tflops)
     return result
 
 
@@ -547,19 +612,20 @@ def run_sweep(args, workload, dtype=None, upstream=1.0, path=None, steps=None, w
     dz = None
     step_events = []
     stream = torch.cuda.current_stream(dev)
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        del dz                      # the previous gradient is released before the next one is allocated
-        if flush:
-            scrub.fill_(1)
-            torch.cuda.synchronize()
-        s_ev, e_ev = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        s_ev.record(stream)
-        loss, stats, dz = step()
-        e_ev.record(stream)
-        step_events.append((s_ev, e_ev))
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    with BoardSampler() as board:
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            del dz                      # the previous gradient is released before the next one is allocated
+            if flush:
+                scrub.fill_(1)
+                torch.cuda.synchronize()
+            s_ev, e_ev = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s_ev.record(stream)
+            loss, stats, dz = step()
+            e_ev.record(stream)
+            step_events.append((s_ev, e_ev))
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
     events = vocab_ops.kernel_events
     vocab_ops.kernel_events = None
     step_ms = [s_ev.elapsed_time(e_ev) for s_ev, e_ev in step_events]
@@ -654,6 +720,7 @@ def run_sweep(args, workload, dtype=None, upstream=1.0, path=None, steps=None, w
         "rescale_passes_in_timed_steps": int(rescales.item()) - rescales_before if path == "fused" else None,
         "stats": {k: float(v) for k, v in stats.items()},
         "loss": float(loss.detach()),
+        "board": board.summary(),
     }
     del dz, scrub, logits, b
     _release(torch)
@@ -873,7 +940,7 @@ def _compact(r):
         if key in r:
             out[key] = r[key]
     for key in ("per_micro_batch_GBps", "fused_sweeps_ms_per_step", "logits_products_ms_per_step",
-                "backward_products_ms_per_step"):
+                "backward_products_ms_per_step", "board"):
         if key in roof:
             out["roofline"][key] = roof[key]
     for key in ("micro_batches", "responses_kept", "groups_dropped", "caches_flushed_between_steps"):
