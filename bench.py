@@ -639,6 +639,46 @@ def run_sweep(args, workload, dtype=None, upstream=1.0, path=None, steps=None, w
             loss, stats, dz = step()
         torch.cuda.synchronize()
         hot_ms = (time.perf_counter() - t0) * 1e3 / steps
+    graph_ms = graph_hot_ms = None
+    if flush and path == "fused":
+        # The same step (forward, statistics left on the device, backward) captured once into a graph and
+        # replayed: one launch from the host per step instead of four plus the interpreter between them.
+        # Timed like the eager steps: flushed with per-replay events (median), then back to back.
+        z_static = logits.detach().requires_grad_()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                w_loss, _w_stats = f.compute_loss(z_static, b, fused=True, deferred_stats=True, **kw)
+                torch.autograd.grad(w_loss, z_static, grad_outputs=root)
+        torch.cuda.current_stream(dev).wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            g_loss, g_stats = f.compute_loss(z_static, b, fused=True, **kw)
+            (g_dz,) = torch.autograd.grad(g_loss, z_static, grad_outputs=root)
+        torch.cuda.synchronize()
+        replay_events = []
+        for _ in range(steps):
+            scrub.fill_(1)
+            torch.cuda.synchronize()
+            s_ev, e_ev = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s_ev.record(stream)
+            graph.replay()
+            e_ev.record(stream)
+            replay_events.append((s_ev, e_ev))
+        torch.cuda.synchronize()
+        graph_ms = _median([a.elapsed_time(c) for a, c in replay_events])
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_hot_ms = (time.perf_counter() - t0) * 1e3 / steps
+        # the replayed step is the eager step: same loss, same gradient, same statistics
+        if not (float(g_loss.detach()) == float(loss.detach()) and torch.equal(g_dz, dz)
+                and all(g_stats[k] == float(v) for k, v in stats.items())):
+            raise RuntimeError("graph replay differs from the eager step")
+        del graph, g_dz
 
     def avg_ms(name):
         ts = [s.elapsed_time(e) for (n, s, e, _) in events if n == name]
@@ -712,6 +752,8 @@ def run_sweep(args, workload, dtype=None, upstream=1.0, path=None, steps=None, w
         "ms_per_step_median": _median(step_ms),
         "ms_per_step_mean_wall": elapsed * 1e3 / steps,
         "ms_per_step_hot": hot_ms,
+        "ms_per_step_graph_replay": graph_ms,
+        "ms_per_step_hot_graph_replay": graph_hot_ms,
         "kernels": kernels,
         "step_hbm": {"GBps": step_gbps, "frac": step_gbps / HBM_PEAK_GBPS, "algorithmic_bytes_per_step": step_bytes},
         # NOT a roofline fraction: the step's time applied to the bytes a 3-pass (read, read, write)
@@ -935,7 +977,8 @@ def _compact(r):
            "workload": r["config"]["workload"],
            "roofline": {"kernel": roof["kernel"], "bound": roof["bound"], "achieved": roof["achieved"],
                         "unit": roof["unit"], "frac": roof["frac"], "avg_ms": roof.get("avg_ms")}}
-    for key in ("ms_per_step_median", "ms_per_step_hot", "rescale_passes_in_timed_steps", "library_products_comparison",
+    for key in ("ms_per_step_median", "ms_per_step_hot", "ms_per_step_graph_replay", "ms_per_step_hot_graph_replay",
+                "rescale_passes_in_timed_steps", "library_products_comparison",
                 "micro_batch_rows", "micro_batch_step_ms"):
         if key in r:
             out[key] = r[key]

@@ -586,7 +586,12 @@ class DeferredStats(dict):
     printing, copying, pickling) - typically after the backward, when the reference's engine gathers
     the metrics of all micro-batches.  Keys, ``len`` and ``in`` need no synchronisation.  Selected with
     ``deferred_stats=True`` (keyword of ``compute_loss``) or the environment variable
-    MRL_DEFERRED_STATS=1; the default returns plain floats at once, like the reference."""
+    MRL_DEFERRED_STATS=1; the default returns plain floats at once, like the reference.
+
+    A ``compute_loss`` that runs while its stream is being captured into a graph (``torch.cuda.graph``)
+    always returns this type, bound to the device scalars instead of a host copy: it must not be read
+    during the capture, and after every replay it yields that replay's values (one synchronous
+    32-byte copy per access)."""
 
     __slots__ = ("_pending", "__weakref__")
 
@@ -596,10 +601,15 @@ class DeferredStats(dict):
 
     def _fetch(self):
         if self._pending is not None:
-            spec, host, event = self._pending
-            self._pending = None
-            event.synchronize()
-            values = host.tolist()
+            spec, source, event = self._pending
+            if event is None:
+                # made while a graph was being captured: `source` is the device tensor, which every
+                # replay rewrites, so it is read afresh on every access and nothing is cached
+                values = source.detach().cpu().tolist()
+            else:
+                self._pending = None
+                event.synchronize()
+                values = source.tolist()
             for key, index, use_abs in spec:
                 dict.__setitem__(self, key, abs(values[index]) if use_abs else values[index])
         return self
@@ -683,6 +693,10 @@ def _finish(loss, out, kwargs=None, skip=()):
     deferred statistics the copy is asynchronous and the floats are made on first access."""
     spec = [(STAT_KEYS[i], i + 1, i == 0) for i in range(5) if STAT_KEYS[i] not in skip]
     deferred = (kwargs or {}).get("deferred_stats", os.environ.get("MRL_DEFERRED_STATS", "0") == "1")
+    if out.is_cuda and torch.cuda.is_current_stream_capturing():
+        # under graph capture nothing may wait for the device: the dict reads the device scalars when it
+        # is looked at (after a replay), whatever was asked for
+        return loss, DeferredStats(spec, out, None)
     if not deferred:
         host = out.detach().cpu().tolist()
         return loss, {key: (abs(host[index]) if use_abs else host[index]) for key, index, use_abs in spec}

@@ -3112,6 +3112,68 @@ def test_deferred_statistics_equal_the_eager_ones(dev):
     assert all(dict(m) == want for m in many)
 
 
+@pytest.mark.parametrize("source", ["logits", "hidden_states"])
+def test_whole_step_captured_in_a_graph_and_replayed(dev, source):
+    """compute_loss + backward captured once (torch.cuda.graph) and replayed on new inputs written into the
+    same buffers: nothing on the path waits for the device or allocates outside torch's pool, the cleared
+    words are cleared by a kernel, and the statistics stay on the device until they are read.  Every replay
+    is checked against an eager step on the same inputs (bit-identical: the same kernels on the same data),
+    with that eager work and synchronisations between the replays.  From the hidden states the live rows are
+    not gathered (lm_head_compact_rows=False): their number would have to be read back."""
+    gen = torch.Generator().manual_seed(77)
+    f = mrl.GRPOActorLossFunc()
+    f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.01), "kl_penalty": "low_var_kl",
+                          "entropy_coeff": 0.001})
+    if source == "logits":
+        logits, b, kw, _, _ = _make_batch(gen, 2, 4, 5, 30, 2048, torch.bfloat16, 2.0, 1)
+        shapes, extra = [tuple(logits.shape)], {"fused": True}
+        fresh = lambda: [(torch.randn(shapes[0], generator=gen) * 2).to(torch.bfloat16).to(dev)]
+    else:
+        vocab, hdim = 2048, 128
+        _, b, kw, _, _ = _make_batch(gen, 2, 4, 5, 24, vocab, torch.bfloat16, 1.0, 2, prompt_hi=6)
+        total = b["labels"].shape[1]
+        extra = {"lm_head_compact_rows": False}
+        fresh = lambda: [torch.randn(1, total, hdim, generator=gen).to(torch.bfloat16).to(dev),
+                         (torch.randn(vocab, hdim, generator=gen) * (3.0 / hdim ** 0.5)).to(torch.bfloat16).to(dev)]
+    bd, kwd = _to_dev(b, dev), _to_dev(kw, dev)
+
+    def step(inputs):
+        if source == "logits":
+            loss, stats = f.compute_loss(inputs[0], bd, **extra, **kwd)
+        else:
+            loss, stats = f.compute_loss(inputs[0], bd, lm_head_weight=inputs[1], **extra, **kwd)
+        return loss, stats, torch.autograd.grad(loss, inputs)
+
+    static = [t.requires_grad_() for t in fresh()]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):                       # warm-up off the default stream, as capture asks for
+        for _ in range(2):
+            step(static)
+    torch.cuda.current_stream(dev).wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        loss_g, stats_g, grads_g = step(static)
+    torch.cuda.synchronize()
+    assert isinstance(stats_g, mrl.DeferredStats)
+    seen = set()
+    for _ in range(4):
+        new = fresh()
+        with torch.no_grad():
+            for dst, src in zip(static, new):
+                dst.copy_(src)
+        loss_e, stats_e, grads_e = step([t.clone().requires_grad_() for t in new])      # eager, between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert loss_g.item() == loss_e.item() and dict(stats_g) == stats_e
+        for got, want in zip(grads_g, grads_e):
+            assert torch.equal(got, want)
+        seen.add(loss_e.item())
+    assert len(seen) == 4                               # the replays did see different inputs
+
+
 @pytest.mark.parametrize("upstream", [0.0, float("inf")])
 def test_backward_with_a_zero_or_infinite_upstream_gradient(dev, upstream):
     """A skipped or overflowed loss-scale step reaches the loss as an upstream gradient of 0 or Inf.  It

@@ -313,3 +313,9 @@ def test_deferred_stats_behaves_like_the_dict_of_floats_it_stands_for():
     assert fresh().get("absent", 7) == 7 and fresh().get(STAT_KEYS[1]) == 2.0
     assert all(isinstance(v, float) for _, v in fresh().items())
     assert "actor/pg_loss" in repr(fresh())
+    # the form handed out under graph capture (no event): bound to the scalars themselves, read afresh on
+    # every access, so that it shows what the latest replay left there
+    live = DeferredStats(spec, host.clone(), None)
+    assert dict(live) == want
+    live._pending[1].mul_(2.0)
+    assert live[STAT_KEYS[1]] == 4.0 and dict(live) == {k: 2.0 * v for k, v in want.items()}
