@@ -14,9 +14,13 @@ Restates ``mindspeed_rl/utils/seqlen_balancing.py`` of the reference:
   count is not on this path)
 * ``:383-388``  ``get_reverse_idx``
 
-PARITY UNPINNED against reference-held vectors: the reference has no test or fixture for this
-module.  Pinned by textbook results of the differencing method, by brute force over all
-assignments on small inputs, and by the invariants every partitioner must keep.
+Pinned by outputs of the reference's own module: it holds no test or fixture for these functions
+and their tie-breaking follows from no closed form, so the module was executed in the build
+container on seeded inputs (``tests/golden/make_reference_partition_vectors.py`` loads that one
+file by path; the vectors are ``tests/golden/reference_partition_vectors.json``) and every function
+here must return the same partitions index for index.  Also held to textbook results of the
+differencing method, brute force over all assignments on small inputs, and the invariants every
+partitioner must keep.
 """
 import copy
 import heapq

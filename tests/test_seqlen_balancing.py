@@ -1,7 +1,11 @@
 """Token-budget micro-batching (host logic, no GPU): the oracle's restatement of the reference against
-textbook results of the largest differencing method, brute force and invariants (the reference holds no
-vectors for this module), and the package's implementation against the oracle, partition for partition."""
+outputs of the reference's own module (tests/golden/reference_partition_vectors.json: the reference
+holds no vectors for it, so its functions were run on seeded inputs, ties included), textbook results of
+the largest differencing method, brute force and invariants; and the package's implementation against
+the same vectors and against the oracle, partition for partition."""
 import itertools
+import json
+import os
 import random
 
 import pytest
@@ -189,3 +193,48 @@ def test_bin_packing_matches_oracle():
         assert sb.balanced_bin_packing(lengths, cap) == ob.balanced_bin_packing(lengths, cap)
     with pytest.raises(ValueError, match="exceeds max_capacity"):
         sb.balanced_bin_packing([3, 11], 10)
+
+
+def _plain(x):
+    return [_plain(v) for v in x] if isinstance(x, (list, tuple)) else int(x)
+
+
+def _call(mod, case, flag_by_env):
+    fn = case["fn"]
+    if fn in ("karmarkar_karp", "heapq_partition", "get_seqlen_balanced_partitions"):
+        return getattr(mod, fn)(list(case["seqlen_list"]), case["k_partitions"], case["equal_size"])
+    if fn == "heapq_partition_with_max":
+        return mod.heapq_partition_with_max(list(case["seqlen_list"]), case["k_partitions"], case["max_token_len"])
+    if fn == "balanced_bin_packing":
+        return mod.balanced_bin_packing(list(case["seqlen_list"]), case["max_capacity"])
+    if fn == "get_reverse_idx":
+        return mod.get_reverse_idx(list(case["idx_map"]))
+    assert fn == "rearrange_micro_batches"
+    if flag_by_env:
+        # the reference's own switch: is_multimodal() reads the process environment
+        os.environ["IS_MULTIMODAL"] = "1" if case["multimodal"] else "0"
+        try:
+            return mod.rearrange_micro_batches(list(case["seqlen_list"]), case["max_token_len"], case["dynamic_max_batch_size"])
+        finally:
+            os.environ.pop("IS_MULTIMODAL", None)
+    return mod.rearrange_micro_batches(list(case["seqlen_list"]), case["max_token_len"], case["dynamic_max_batch_size"],
+                                       multimodal=case["multimodal"])
+
+
+@pytest.mark.parametrize("which", ["oracle", "package"])
+def test_partitioners_equal_the_reference_outputs(which):
+    """Every partitioner, partition for partition and index for index, against what the reference's module
+    returned for the same arguments: lists with few distinct lengths (nearly every comparison a tie), all
+    lengths equal, response-like lengths and multiples of 128; 1 to 64 items, 1 to n groups, equal-size
+    and free, budgets from the longest item to the whole batch, with and without a minimum number of
+    micro-batches, and the capacity-bound packing of the multimodal branch."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_partition_vectors.json")
+    with open(path) as fh:
+        cases = json.load(fh)["cases"]
+    assert len(cases) > 1000 and {c["fn"] for c in cases} == {
+        "karmarkar_karp", "heapq_partition", "get_seqlen_balanced_partitions", "heapq_partition_with_max",
+        "balanced_bin_packing", "rearrange_micro_batches", "get_reverse_idx"}
+    mod, by_env = (ob, False) if which == "oracle" else (sb, True)
+    for case in cases:
+        got = _plain(_call(mod, case, by_env))
+        assert got == case["out"], {k: v for k, v in case.items() if k != "out"}
