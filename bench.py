@@ -644,6 +644,8 @@ def run_sweep(args, workload, dtype=None, upstream=1.0, path=None, steps=None, w
         # The same step (forward, statistics left on the device, backward) captured once into a graph and
         # replayed: one launch from the host per step instead of four plus the interpreter between them.
         # Timed like the eager steps: flushed with per-replay events (median), then back to back.
+        import warnings
+        warnings.filterwarnings("ignore", message=".*AccumulateGrad node's stream does not match.*")
         z_static = logits.detach().requires_grad_()
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream(dev))
@@ -980,7 +982,7 @@ def _compact(r):
     for key in ("ms_per_step_median", "ms_per_step_hot", "ms_per_step_graph_replay", "ms_per_step_hot_graph_replay",
                 "rescale_passes_in_timed_steps", "library_products_comparison",
                 "micro_batch_rows", "micro_batch_step_ms"):
-        if key in r:
+        if r.get(key) is not None:
             out[key] = r[key]
     for key in ("per_micro_batch_GBps", "fused_sweeps_ms_per_step", "logits_products_ms_per_step",
                 "backward_products_ms_per_step", "board"):
