@@ -3112,7 +3112,7 @@ def test_deferred_statistics_equal_the_eager_ones(dev):
     assert all(dict(m) == want for m in many)
 
 
-@pytest.mark.parametrize("source", ["logits", "hidden_states"])
+@pytest.mark.parametrize("source", ["logits", "padded_logits_dapo_quarter", "hidden_states"])
 def test_whole_step_captured_in_a_graph_and_replayed(dev, source):
     """compute_loss + backward captured once (torch.cuda.graph) and replayed on new inputs written into the
     same buffers: nothing on the path waits for the device or allocates outside torch's pool, the cleared
@@ -3124,7 +3124,17 @@ def test_whole_step_captured_in_a_graph_and_replayed(dev, source):
     f = mrl.GRPOActorLossFunc()
     f.add_loss_meta_info({"clip_ratio": 0.2, "kl_ctrl": mrl.FixedKLController(0.01), "kl_penalty": "low_var_kl",
                           "entropy_coeff": 0.001})
-    if source == "logits":
+    divide = 1.0                    # the schedule back-propagates loss / divide (number of micro-batches)
+    if source == "padded_logits_dapo_quarter":
+        # padded [B, S, V] fp32 logits, DAPO with a sequence-mean loss, and loss / 4 back-propagated: the
+        # scale reaches the stored gradients through a device scalar, so it is part of the replay as well
+        f = mrl.DAPOActorLossFunc()
+        f.add_loss_meta_info({"clip_ratio": 0.2, "clip_higher_enable": True, "clip_ratio_low": 0.2,
+                              "clip_ratio_high": 0.28, "token_level_loss": False, "entropy_coeff": 0.001})
+        z0, b = _small_padded_micro_batch(5, 6, 24, 1032)
+        kw, extra, divide = {}, {"fused": True}, 4.0
+        fresh = lambda: [(torch.randn(z0.shape, generator=gen) * 2).to(dev)]
+    elif source == "logits":
         logits, b, kw, _, _ = _make_batch(gen, 2, 4, 5, 30, 2048, torch.bfloat16, 2.0, 1)
         shapes, extra = [tuple(logits.shape)], {"fused": True}
         fresh = lambda: [(torch.randn(shapes[0], generator=gen) * 2).to(torch.bfloat16).to(dev)]
@@ -3138,11 +3148,11 @@ def test_whole_step_captured_in_a_graph_and_replayed(dev, source):
     bd, kwd = _to_dev(b, dev), _to_dev(kw, dev)
 
     def step(inputs):
-        if source == "logits":
-            loss, stats = f.compute_loss(inputs[0], bd, **extra, **kwd)
-        else:
+        if source == "hidden_states":
             loss, stats = f.compute_loss(inputs[0], bd, lm_head_weight=inputs[1], **extra, **kwd)
-        return loss, stats, torch.autograd.grad(loss, inputs)
+        else:
+            loss, stats = f.compute_loss(inputs[0], bd, **extra, **kwd)
+        return loss, stats, torch.autograd.grad(loss / divide, inputs)
 
     static = [t.requires_grad_() for t in fresh()]
     side = torch.cuda.Stream()
