@@ -766,6 +766,10 @@ def run_sweep(args, workload, dtype=None, upstream=1.0, path=None, steps=None, w
         "loss": float(loss.detach()),
         "board": board.summary(),
     }
+    host_copy = None
+    if cpu == "whole":
+        to_host = lambda d: {k: (v.cpu() if isinstance(v, torch.Tensor) else v) for k, v in d.items()}
+        host_copy = (logits.detach().cpu(), to_host(b), to_host(kw), tokens)
     del dz, scrub, logits, b
     _release(torch)
     if probes:
@@ -775,9 +779,39 @@ def run_sweep(args, workload, dtype=None, upstream=1.0, path=None, steps=None, w
         for k in kernels.values():
             k["frac_of_measured_copy"] = k["GBps"] / best_copy
         result["roofline"]["frac_of_measured_copy_ceiling"] = kernels[dominant]["GBps"] / best_copy
-    if cpu:
+    if cpu == "whole":
+        result["cpu_baseline"] = cpu_baseline_whole(torch, w, host_copy, args.entropy_coeff, float(result["loss"]))
+    elif cpu:
         result["cpu_baseline"] = cpu_baseline(torch, w, args.cpu_rows, args.entropy_coeff, args.seed, mrl, dev, path)
     return result
+
+
+def cpu_baseline_whole(torch, w, host_copy, entropy_coeff, gpu_loss):
+    """The oracle on the WHOLE batch of a workload that fits the host (configs[0]): the very logits and
+    batch the GPU steps ran on, forward + backward, median of 5 after 2 warm-ups."""
+    from oracle import loss as o_loss
+    threads = os.cpu_count() or 1
+    threads = min(threads, int(os.environ.get("OMP_NUM_THREADS", threads)))
+    torch.set_num_threads(threads)
+    logits, b, kw, tokens = host_copy
+    meta = dict(clip_ratio=0.2, kl_coef=0.001, kl_penalty="low_var_kl", entropy_coeff=entropy_coeff)
+    z32 = logits.float()
+
+    def one():
+        z = z32.detach().requires_grad_()
+        t0 = time.perf_counter()
+        loss, _ = o_loss.grpo_compute_loss(z, b, meta, **kw)
+        loss.backward()
+        return time.perf_counter() - t0, float(loss.detach())
+
+    for _ in range(2):
+        one()
+    runs = sorted(one() for _ in range(5))
+    med, cpu_loss = runs[len(runs) // 2]
+    return {"value": tokens / med, "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": "the whole batch: %d responses, %d packed rows x V=%d, oracle fwd+bwd, median of 5 after 2 warm-ups, "
+                      "%.3f s per pass" % (b["responses"].shape[0], logits.shape[1], logits.shape[-1], med),
+            "loss_rel_err_gpu_vs_oracle": abs(gpu_loss - cpu_loss) / max(abs(cpu_loss), 1e-30)}
 
 
 def bandwidth_ceilings(torch, _lib, dev):
@@ -980,7 +1014,7 @@ def _compact(r):
            "roofline": {"kernel": roof["kernel"], "bound": roof["bound"], "achieved": roof["achieved"],
                         "unit": roof["unit"], "frac": roof["frac"], "avg_ms": roof.get("avg_ms")}}
     for key in ("ms_per_step_median", "ms_per_step_hot", "ms_per_step_graph_replay", "ms_per_step_hot_graph_replay",
-                "rescale_passes_in_timed_steps", "library_products_comparison",
+                "cpu_baseline", "rescale_passes_in_timed_steps", "library_products_comparison",
                 "micro_batch_rows", "micro_batch_step_ms"):
         if r.get(key) is not None:
             out[key] = r[key]
@@ -1015,15 +1049,15 @@ def main():
     elif args.workload == "c4":
         result = run_c4(args)
     elif args.workload == "c0":
-        result = run_sweep(args, "c0", dtype=args.dtype, upstream=args.upstream, cpu=cpu, flush=True)
+        result = run_sweep(args, "c0", dtype=args.dtype, upstream=args.upstream, cpu="whole" if cpu else False, flush=True)
     elif args.workload != "all":
         result = run_sweep(args, args.workload, dtype=args.dtype, upstream=args.upstream, cpu=cpu)
     else:
         # the headline first and alone on the card, then a few steps of everything else
         result = run_sweep(args, "c1", dtype=args.dtype, upstream=args.upstream, cpu=cpu)
         k, others = args.other_steps, {}
-        others["c0"] = _compact(run_sweep(args, "c0", steps=max(k, 20), warmup=3, probes=False, cpu=False, flush=True,
-                                          deferred=False))
+        others["c0"] = _compact(run_sweep(args, "c0", steps=max(k, 20), warmup=3, probes=False,
+                                          cpu="whole" if cpu else False, flush=True, deferred=False))
         # the same with the statistics fetched lazily (no synchronisation between forward and backward)
         lazy = run_sweep(args, "c0", steps=max(k, 20), warmup=3, probes=False, cpu=False, flush=True, deferred=True)
         others["c0"]["ms_per_step_deferred_stats"] = lazy["ms_per_step"]
