@@ -2052,7 +2052,9 @@ def _random_fused_case(i, rnd):
     scale = g_ref.abs().max().item() + 1e-12
     err = (dz.float() - g_ref).abs().max().item()
     rel = 2 ** -7 if dtype != torch.float32 else 2e-5
-    ok = e_lp < 2e-4 and err <= rel * scale + 1e-9 and not dz[~live].any().item()
+    # fp16 gradients below 6.1e-5 are subnormal: their spacing is 2^-24 whatever their size
+    floor = 2 ** -25 if dtype == torch.float16 else 1e-9
+    ok = e_lp < 2e-4 and err <= rel * scale + floor and not dz[~live].any().item()
     if ent_c != 0 and live.any():
         ok = ok and (ent[live] - h_ref.detach()[live]).abs().max().item() < 2e-4
     return None if ok else (i, dtype, rows, vocab, inv_t, ent_c, e_lp, err, scale)
@@ -2118,7 +2120,8 @@ def _random_split_case(i, rnd):
     scale = g_ref.abs().max().item() + 1e-12
     err = (dz.float() - g_ref).abs().max().item()
     rel = 2 ** -7 if dtype != torch.float32 else 3e-5
-    ok = e_lp < 2e-4 and e_h < 2e-4 and err <= rel * scale + 1e-9 and dz.dtype == dtype and dz.shape == z.shape
+    floor = 2 ** -25 if dtype == torch.float16 else 1e-9     # the spacing of fp16 subnormals is 2^-24
+    ok = e_lp < 2e-4 and e_h < 2e-4 and err <= rel * scale + floor and dz.dtype == dtype and dz.shape == z.shape
     if rows > 2 and mode == "both":
         ok = ok and not dz[2].any().item()
     return None if ok else (i, dtype, rows, vocab, pad, inv_t, mode, e_lp, e_h, err, scale)
@@ -2192,7 +2195,8 @@ def _random_loss_case(i, rnd, dev):
             dz_cmp[0, cu[k]:cu[k] + seqlens[k]] = dzp[k, :seqlens[k]].float().cpu()
             if dzp[k, seqlens[k]:].any().item():
                 return (i, "padding rows not zero")
-    tol_l = 1e-4 * abs(want.item()) + 1e-7
+    # the loss is a mean of terms of size ~1 that may cancel: a few fp32 ulps of 1 remain whatever its size
+    tol_l = 1e-4 * abs(want.item()) + 1e-6
     if not abs(got.item() - want.item()) <= tol_l:
         return (i, kind, fused, layout, "loss", got.item(), want.item())
     for k in want_stats:
@@ -2396,7 +2400,8 @@ def _random_value_side_case(i, rnd, dev):
     penalty = rnd.choice(["kl", "abs", "mse", "low_var_kl"])
     want, want_kl = o_adv.kl_token_level_rewards(old, ref, lens, scores, 0.05, penalty)
     got, got_kl = mrl.kl_token_level_rewards(old.to(dev), ref.to(dev), lens.to(dev), scores.to(dev), 0.05, penalty)
-    if not ((got.cpu() - want).abs().max().item() < 1e-6 and abs(got_kl - want_kl) <= 1e-5 * abs(want_kl) + 1e-8):
+    # exp(c) - c - 1 cancels for small c: the mean KL carries an absolute error of a few fp32 ulps of 1
+    if not ((got.cpu() - want).abs().max().item() < 1e-6 and abs(got_kl - want_kl) <= 1e-5 * abs(want_kl) + 2e-7):
         return (i, "kl_rewards", batch, width, penalty)
     # value loss
     values = torch.randn(batch, width, generator=gen)
