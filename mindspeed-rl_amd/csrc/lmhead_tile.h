@@ -173,8 +173,13 @@ __device__ __forceinline__ void mfma_tile_loop(unsigned char* smem, const uint16
         const int g = lane >> 4, kk = (lane >> 2) & 3;
         tr_off[j] = (8 * g + kk) * 128 + ((j * 32) ^ tr_swizzle(8 * g + kk)) + (lane & 3) * 8;
     }
+    // A k-contiguous operand's fragments are ordinary 16-byte loads (the compiler waits for them); a k-major
+    // operand's arrive as the two 8-byte halves that the asm reads below deliver, and stay two values until
+    // `landed` has passed them through the loop's own wait (members that a product does not use fold away).
+    typedef long long2v __attribute__((ext_vector_type(2)));
     struct Frags {
         bf16x8 a[kBlocks], b[kBlocks];
+        long a_lo[kBlocks], a_hi[kBlocks], b_lo[kBlocks], b_hi[kBlocks];
     };
     // fragment of 16-row block `blk` (0..15 inside the tile) of an operand whose stage starts at `op`
     auto read_kcontig = [&](const unsigned char* op, int blk, int ks) {
@@ -183,28 +188,47 @@ __device__ __forceinline__ void mfma_tile_loop(unsigned char* smem, const uint16
     // The transposing read goes out as inline assembly: through the builtin the compiler cannot tell it
     // from an access to the bytes that the requests in flight are writing and waits for all of them
     // (vmcnt(0)) before every read.  The price: it does not wait for the result either - the loop
-    // below does (lgkmcnt(0) before a sub-step consumes fragments read during the one before).
+    // below does (lgkmcnt(0) before a sub-step consumes fragments read during the one before), and
+    // `landed` makes that wait the point where the halves become usable values: whatever the compiler does
+    // with them (join them in place, or copy them) it can only do behind the wait.
     const unsigned smem_lds = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
-    auto read_kmajor = [&](const unsigned char* op, int blk, int ks) {
-        typedef long long2v __attribute__((ext_vector_type(2)));
+    auto read_kmajor = [&](const unsigned char* op, int blk, int ks, long& lo, long& hi) {
         const unsigned addr = smem_lds + (unsigned)(op - smem) + (blk >> 2) * 8192 + ks * (32 * 128) + tr_off[blk & 3];
-        long2v both;
-        long lo, hi;
         asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo) : "v"(addr) : "memory");
         asm volatile("ds_read_b64_tr_b16 %0, %1 offset:512" : "=v"(hi) : "v"(addr) : "memory");
+    };
+    auto join = [](long lo, long hi) {
+        long2v both;
         both[0] = lo;
         both[1] = hi;
         return __builtin_bit_cast(bf16x8, both);
+    };
+    // placed right behind the wait for a fragment set: every half of the set is an input and an output of an
+    // empty statement there, so no use of it (and no copy of it) can be scheduled ahead of the wait
+    auto landed = [&](Frags& f) {
+        static_assert(kBlocks == 8, "the operand lists below name 8 fragments");
+        if (kATrans)
+            asm volatile("" : "+v"(f.a_lo[0]), "+v"(f.a_hi[0]), "+v"(f.a_lo[1]), "+v"(f.a_hi[1]), "+v"(f.a_lo[2]),
+                              "+v"(f.a_hi[2]), "+v"(f.a_lo[3]), "+v"(f.a_hi[3]), "+v"(f.a_lo[4]), "+v"(f.a_hi[4]),
+                              "+v"(f.a_lo[5]), "+v"(f.a_hi[5]), "+v"(f.a_lo[6]), "+v"(f.a_hi[6]), "+v"(f.a_lo[7]),
+                              "+v"(f.a_hi[7]));
+        if (kBTrans)
+            asm volatile("" : "+v"(f.b_lo[0]), "+v"(f.b_hi[0]), "+v"(f.b_lo[1]), "+v"(f.b_hi[1]), "+v"(f.b_lo[2]),
+                              "+v"(f.b_hi[2]), "+v"(f.b_lo[3]), "+v"(f.b_hi[3]), "+v"(f.b_lo[4]), "+v"(f.b_hi[4]),
+                              "+v"(f.b_lo[5]), "+v"(f.b_hi[5]), "+v"(f.b_lo[6]), "+v"(f.b_hi[6]), "+v"(f.b_lo[7]),
+                              "+v"(f.b_hi[7]));
     };
     // read r (0..15) of a fragment set, in the order the MFMAs need them: a0, all of b, a1..a7
     auto read1 = [&](Frags& f, const unsigned char* stage, int ks, int r) {
         const bool is_a = r == 0 || r > kBlocks;
         const int blk = r == 0 ? 0 : (r <= kBlocks ? r - 1 : r - kBlocks);
-        if (is_a)
-            f.a[blk] = kATrans ? read_kmajor(stage, wv * kBlocks + blk, ks) : read_kcontig(stage, wv * kBlocks + blk, ks);
-        else
-            f.b[blk] = kBTrans ? read_kmajor(stage + kOperandBytes, wt * kBlocks + blk, ks)
-                               : read_kcontig(stage + kOperandBytes, wt * kBlocks + blk, ks);
+        if (is_a) {
+            if (kATrans) read_kmajor(stage, wv * kBlocks + blk, ks, f.a_lo[blk], f.a_hi[blk]);
+            else f.a[blk] = read_kcontig(stage, wv * kBlocks + blk, ks);
+        } else {
+            if (kBTrans) read_kmajor(stage + kOperandBytes, wt * kBlocks + blk, ks, f.b_lo[blk], f.b_hi[blk]);
+            else f.b[blk] = read_kcontig(stage + kOperandBytes, wt * kBlocks + blk, ks);
+        }
     };
     floatx4 acc[kBlocks][kBlocks];
     auto zero_acc = [&]() {
@@ -226,7 +250,9 @@ __device__ __forceinline__ void mfma_tile_loop(unsigned char* smem, const uint16
     };
     auto mfma1 = [&](const Frags& f, int i) {
         const int vb = i / kBlocks, tb = i % kBlocks;
-        acc[vb][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.a[vb], f.b[tb], acc[vb][tb], 0, 0, 0);
+        const bf16x8 a = kATrans ? join(f.a_lo[vb], f.a_hi[vb]) : f.a[vb];
+        const bf16x8 b = kBTrans ? join(f.b_lo[tb], f.b_hi[tb]) : f.b[tb];
+        acc[vb][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[vb][tb], 0, 0, 0);
     };
 
     // One wavefront per SIMD: memory instructions are placed between the MFMAs of the same instruction
@@ -270,6 +296,7 @@ __device__ __forceinline__ void mfma_tile_loop(unsigned char* smem, const uint16
             const unsigned char* other = smem + (buf ^ 1) * kStageBytes;
             MRL_SB;
             if (kATrans || kBTrans) __builtin_amdgcn_s_waitcnt(0xC07F);      // lgkmcnt(0): G0 has arrived
+            landed(G0);
             MRL_SB;
 #pragma unroll
             for (int i = 0; i < kMfmas; ++i) {
@@ -286,6 +313,7 @@ __device__ __forceinline__ void mfma_tile_loop(unsigned char* smem, const uint16
             }
             if (kEarly > 0) stage_issued();
             __builtin_amdgcn_s_waitcnt(0x0070);        // vmcnt(0) lgkmcnt(0)
+            landed(G1);
             asm volatile("s_barrier" ::: "memory");
             MRL_SB;
 #pragma unroll
